@@ -1,0 +1,246 @@
+/*
+ * triebwerk_kv.h -- C ABI of the MI355X (gfx950) KV-cache hot path.
+ *
+ * Part 1 keeps the reference engine's own kernel-launcher boundary: the
+ * `extern "C" void launch_*` functions that engine/engine.cpp declares at
+ * lines 105-171 and engine/kernels.cu defines.  Names, parameter order and
+ * parameter meaning are unchanged; `cudaStream_t` becomes `hipStream_t` and
+ * `half*` is any pointer to IEEE binary16 storage.  A HIP build of the engine
+ * links this library in place of the reference's `kernels` static library for
+ * these entry points.
+ *
+ * Part 2 is what the reference does inline in engine.cpp for the same path
+ * (cache sizing, arena carving, reset, rotation matrix, decode-step graph) plus
+ * the paged-cache and fused-append entry points that have no counterpart there.
+ *
+ * Conventions (same as the reference, engine.cpp:105-171):
+ *   - every pointer is a device pointer unless a comment says "host";
+ *   - launchers are asynchronous on `stream`, allocate nothing, keep no pointer,
+ *     and return void; a failed launch or a rejected argument is recorded and
+ *     can be read with tw_kv_last_error() (the reference checks nothing);
+ *   - activations are row-per-sequence: x[g * dim + i];
+ *   - head_dim must be 128 (the reference kernels hard-size their shared
+ *     arrays to 128, kernels.cu:1504, 1671);
+ *   - attention covers cache positions 0..pos INCLUSIVE (kernels.cu:1688).
+ */
+#ifndef TRIEBWERK_KV_H
+#define TRIEBWERK_KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifndef TW_HALF_T
+#define TW_HALF_T uint16_t /* IEEE binary16 storage; `half` in the reference */
+#endif
+typedef TW_HALF_T tw_half;
+
+#ifndef HIP_INCLUDE_HIP_HIP_RUNTIME_API_H
+typedef struct ihipStream_t* hipStream_t;
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ Part 1
+ * Reference launchers (drop-in).                                            */
+
+/* engine.cpp:128, kernels.cu:1351 -- fp16 append of one K row and one V row
+ * per sequence at cache row (g*msl + pos[g]). */
+void launch_kv_cache_write_batch(tw_half* ck, tw_half* cv, const tw_half* k, const tw_half* v,
+                                 const int* pos, int msl, int G, int kv_dim, hipStream_t s);
+
+/* engine.cpp:136, kernels.cu:1963 -- compressed append of `num_tokens` rows of
+ * sequence 0 at rows positions[tok] (prefill and single-sequence decode). */
+void launch_turbo_kv_quantize(uint8_t* cache_q, tw_half* cache_norms, const tw_half* kv_buf,
+                              const tw_half* rotation, const int* positions, int max_seq_len,
+                              int num_tokens, int num_kv_heads, int head_dim, int kv_dim,
+                              int bits, hipStream_t s);
+
+/* engine.cpp:137, kernels.cu:1975 -- compressed append, one row per sequence at
+ * row (g*max_seq_len + positions[g]).  Called once for K and once for V. */
+void launch_turbo_kv_quantize_batch(uint8_t* cache_q, tw_half* cache_norms, const tw_half* kv_buf,
+                                    const tw_half* rotation, const int* positions, int max_seq_len,
+                                    int G, int num_kv_heads, int head_dim, int kv_dim,
+                                    int bits, hipStream_t s);
+
+/* engine.cpp:164, kernels.cu:737 -- fp16 decode attention, one sequence, `pos`
+ * by value.  attn_scratch: num_heads*max_seq_len floats. */
+void launch_gqa_attention(const tw_half* q, const tw_half* k_cache, const tw_half* v_cache,
+                          tw_half* output, float* attn_scratch, int pos, int max_seq_len,
+                          int num_heads, int num_kv_heads, int head_dim, hipStream_t stream);
+
+/* engine.cpp:129, kernels.cu:1354 -- fp16 decode attention for G sequences,
+ * positions read from device memory (graph-capturable).  q_dim is the row
+ * stride of q and out.  as: G*num_heads*msl floats, used as split-K workspace. */
+void launch_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half* ck,
+                                const tw_half* cv, float* as, const int* pos, int msl, int G,
+                                int num_heads, int num_kv_heads, int head_dim, int q_dim,
+                                int kv_dim, hipStream_t s);
+
+/* engine.cpp:139, kernels.cu:2001 -- compressed decode attention, one sequence. */
+void launch_turbo_gqa_attention(const tw_half* q, const uint8_t* ck_q, const uint8_t* cv_q,
+                                const tw_half* k_norms, const tw_half* v_norms,
+                                const tw_half* rotation, tw_half* output, float* as, int pos,
+                                int msl, int num_heads, int num_kv_heads, int head_dim, int bits,
+                                hipStream_t s);
+
+/* engine.cpp:138, kernels.cu:1986 -- compressed decode attention, G sequences. */
+void launch_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const uint8_t* ck_q,
+                                      const uint8_t* cv_q, const tw_half* k_norms,
+                                      const tw_half* v_norms, const tw_half* rotation, float* as,
+                                      const int* pos, int msl, int G, int num_heads,
+                                      int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                      int bits, hipStream_t s);
+
+/* engine.cpp:130, kernels.cu:1359 -- causal fp16 prefill attention over
+ * sequence 0: query tq attends rows 0..tq.  as: T*num_heads*T floats. */
+void launch_gqa_prefill_attention(tw_half* out, const tw_half* q, const tw_half* ck,
+                                  const tw_half* cv, float* as, int T, int msl, int num_heads,
+                                  int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                  hipStream_t s);
+
+/* engine.cpp:140, kernels.cu:2015 -- causal compressed prefill attention. */
+void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const uint8_t* ck_q,
+                                        const uint8_t* cv_q, const tw_half* k_norms,
+                                        const tw_half* v_norms, const tw_half* rotation, float* as,
+                                        int T, int msl, int num_heads, int num_kv_heads,
+                                        int head_dim, int q_dim, int kv_dim, int bits,
+                                        hipStream_t s);
+
+/* engine.cpp:133, kernels.cu:1376 -- positions[g] += 1 on the device. */
+void launch_increment_positions(int* positions, int G, hipStream_t s);
+
+/* ------------------------------------------------------------------ Part 2
+ * Error state, tuning and the entry points the reference has no twin for.   */
+
+/* 0 = no error since the last call to tw_kv_clear_error().  Thread-local. */
+int tw_kv_last_error(void);
+const char* tw_kv_last_error_string(void);
+void tw_kv_clear_error(void);
+
+/* Library version / build info, for the loader to print. */
+const char* tw_kv_build_info(void);
+
+/* Compressed-attention kernel choice for the launchers above and below.
+ * 0 = automatic, 1 = fp32 vector-ALU kernel, 2 = MFMA kernel (kv_bits 4 and 2).
+ * Process-wide; meant for tests and benchmarks. */
+void tw_kv_set_attention_variant(int variant);
+int tw_kv_get_attention_variant(void);
+
+/* Split count override for decode attention (0 = automatic). */
+void tw_kv_set_num_splits(int nsplit);
+
+/* Floats of workspace the *_ws / paged attention entry points need for a
+ * (G, num_heads, max_context) problem at the automatic split count.  The
+ * reference-signature launchers instead fit their split count to the
+ * G*num_heads*msl floats the engine already provides (engine.cpp:1371). */
+size_t tw_attention_workspace_floats(int G, int num_heads, int max_context);
+
+/* K and V compressed append in one launch: what engine.cpp:1985-1990 does with
+ * two launches.  Same layout and arithmetic as launch_turbo_kv_quantize_batch. */
+void tw_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q, tw_half* v_norms,
+                              const tw_half* k_buf, const tw_half* v_buf, const tw_half* rotation,
+                              const int* positions, int max_seq_len, int G, int num_kv_heads,
+                              int head_dim, int kv_dim, int bits, hipStream_t s);
+
+/* Paged cache.  A page holds TW_PAGE_TOKENS consecutive positions of one
+ * sequence in the same row layout the contiguous cache uses, so
+ *   row(g, p) = block_table[g*bt_stride + p/16]*16 + p%16
+ * replaces the reference's row(g, p) = g*msl + p (kernels.cu:973, 1629, 1690)
+ * and nothing else changes.  block_table is device int32. */
+#define TW_PAGE_TOKENS 16
+
+void tw_paged_kv_cache_write_batch(tw_half* ck, tw_half* cv, const tw_half* k, const tw_half* v,
+                                   const int* positions, const int* block_table, int bt_stride,
+                                   int G, int kv_dim, hipStream_t s);
+
+void tw_paged_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q,
+                                    tw_half* v_norms, const tw_half* k_buf, const tw_half* v_buf,
+                                    const tw_half* rotation, const int* positions,
+                                    const int* block_table, int bt_stride, int G,
+                                    int num_kv_heads, int head_dim, int kv_dim, int bits,
+                                    hipStream_t s);
+
+/* max_context bounds positions[g]+1 and fixes the launch grid (graph-safe).
+ * ws: tw_attention_workspace_floats(G, num_heads, max_context) floats. */
+void tw_paged_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half* ck,
+                                  const tw_half* cv, float* ws, const int* positions,
+                                  const int* block_table, int bt_stride, int max_context, int G,
+                                  int num_heads, int num_kv_heads, int head_dim, int q_dim,
+                                  int kv_dim, hipStream_t s);
+
+void tw_paged_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const uint8_t* ck_q,
+                                        const uint8_t* cv_q, const tw_half* k_norms,
+                                        const tw_half* v_norms, const tw_half* rotation, float* ws,
+                                        const int* positions, const int* block_table,
+                                        int bt_stride, int max_context, int G, int num_heads,
+                                        int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                        int bits, hipStream_t s);
+
+/* Host: the rotation matrix of engine.cpp:366-392 (mt19937(42), N(0,1),
+ * modified Gram-Schmidt over rows, fp16).  out: head_dim*head_dim halves, HOST. */
+void tw_make_rotation_host(tw_half* out_host, int head_dim, unsigned seed);
+
+/* ------------------------------------------------------------------ Engine
+ * Host-side owner of the cache: the KV slice of InferenceEngine
+ * (model.h:373-493).  Opaque; one host thread at a time, like the reference. */
+typedef struct tw_engine tw_engine;
+
+typedef struct tw_model_shape {
+    int num_layers;
+    int num_heads;
+    int num_kv_heads;
+    int head_dim;
+} tw_model_shape;
+
+/* InferenceEngine(max_seq_len, kv_bits), engine.cpp:300-317.  kv_bits outside
+ * {0,2,4} prints the reference's warning and falls back to 0. */
+tw_engine* tw_engine_create(int max_seq_len, int kv_bits);
+void tw_engine_destroy(tw_engine* e);
+int tw_engine_kv_bits(const tw_engine* e);      /* engine_py.cpp:25 */
+int tw_engine_max_seq_len(const tw_engine* e);
+
+/* load_config's share of the work: fix the model shape (engine.cpp:769). */
+int tw_engine_set_shape(tw_engine* e, const tw_model_shape* shape);
+
+/* alloc_batch, engine.cpp:1338-1560: one arena for G sequences of max_seq_len
+ * rows, carved with 256-byte alignment in the reference's order (keys, values,
+ * key norms, value norms per layer).  Returns 0 on success. */
+int tw_engine_alloc_batch(tw_engine* e, int G, int max_seq_len);
+/* set_arena, engine.cpp:1609-1620: carve out of caller-owned device memory. */
+int tw_engine_set_arena(tw_engine* e, void* device_ptr, size_t bytes);
+size_t tw_engine_arena_bytes_needed(const tw_engine* e, int G, int max_seq_len);
+
+/* reset(), engine.cpp:893-916 / 2262-2283: zero every cache, positions to 0. */
+int tw_engine_reset(tw_engine* e);
+
+/* Device pointers into the arena (for tests and for callers that keep using
+ * the launchers directly).  which: 0 keys, 1 values, 2 key norms, 3 value norms. */
+void* tw_engine_cache_ptr(tw_engine* e, int layer, int which);
+int* tw_engine_positions(tw_engine* e);          /* device int32[G] */
+const tw_half* tw_engine_rotation(tw_engine* e); /* device, NULL when kv_bits==0 */
+int tw_engine_set_positions(tw_engine* e, const int* host_positions, int G);
+
+/* One decode step of the path for `layer`: append K,V at positions[g], then
+ * attention over 0..positions[g] (forward_layer_batch steps 4-5,
+ * engine.cpp:1979-2006).  q/out: (G, num_heads*head_dim); k/v: (G, kv_dim). */
+int tw_engine_layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k,
+                         const tw_half* v, tw_half* out, hipStream_t s);
+
+/* All layers, then positions += 1.  q/out: (L, G, q_dim); k/v: (L, G, kv_dim).
+ * With use_graph != 0 the step is captured once into a hipGraph and replayed
+ * (engine.cpp:2369-2412, 2480); the capture is dropped when the arena, G or
+ * the buffers change. */
+int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v,
+                          tw_half* out, int use_graph, hipStream_t s);
+
+/* Prefix sharing, engine.cpp:2173-2214: copy rows [0,T) of sequence `src` to
+ * every sequence in [dst_begin, dst_end). */
+int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end, int T,
+                               hipStream_t s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRIEBWERK_KV_H */

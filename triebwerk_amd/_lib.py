@@ -1,0 +1,103 @@
+"""ctypes binding of ``libtriebwerk_kv.so`` (the C ABI in ``include/triebwerk_kv.h``).
+
+The library is the product; there is no Python or CPU fallback.  If the shared
+object is missing, loading raises with the command that builds it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriebwerk_kv.so"
+
+P = C.c_void_p
+I = C.c_int
+LL = C.c_longlong
+SZ = C.c_size_t
+
+
+class ModelShape(C.Structure):
+    _fields_ = [("num_layers", I), ("num_heads", I), ("num_kv_heads", I), ("head_dim", I)]
+
+
+# name -> (restype, argtypes).  Order and meaning follow include/triebwerk_kv.h.
+SIGNATURES = {
+    # Part 1: the reference engine's launchers (engine.cpp:105-171)
+    "launch_kv_cache_write_batch": (None, [P, P, P, P, P, I, I, I, P]),
+    "launch_turbo_kv_quantize": (None, [P, P, P, P, P, I, I, I, I, I, I, P]),
+    "launch_turbo_kv_quantize_batch": (None, [P, P, P, P, P, I, I, I, I, I, I, P]),
+    "launch_gqa_attention": (None, [P, P, P, P, P, I, I, I, I, I, P]),
+    "launch_gqa_attention_batch": (None, [P, P, P, P, P, P, I, I, I, I, I, I, I, P]),
+    "launch_turbo_gqa_attention": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
+    "launch_turbo_gqa_attention_batch": (None, [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
+    "launch_gqa_prefill_attention": (None, [P, P, P, P, P, I, I, I, I, I, I, I, P]),
+    "launch_turbo_gqa_prefill_attention": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
+    "launch_increment_positions": (None, [P, I, P]),
+    # Part 2
+    "tw_kv_last_error": (I, []),
+    "tw_kv_last_error_string": (C.c_char_p, []),
+    "tw_kv_clear_error": (None, []),
+    "tw_kv_build_info": (C.c_char_p, []),
+    "tw_kv_set_attention_variant": (None, [I]),
+    "tw_kv_get_attention_variant": (I, []),
+    "tw_kv_set_num_splits": (None, [I]),
+    "tw_attention_workspace_floats": (SZ, [I, I, I]),
+    "tw_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
+    "tw_paged_kv_cache_write_batch": (None, [P, P, P, P, P, P, I, I, I, P]),
+    "tw_paged_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
+    "tw_paged_gqa_attention_batch": (None, [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
+    "tw_paged_turbo_gqa_attention_batch": (None, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
+    "tw_make_rotation_host": (None, [P, I, C.c_uint]),
+    # Engine
+    "tw_engine_create": (P, [I, I]),
+    "tw_engine_destroy": (None, [P]),
+    "tw_engine_kv_bits": (I, [P]),
+    "tw_engine_max_seq_len": (I, [P]),
+    "tw_engine_set_shape": (I, [P, C.POINTER(ModelShape)]),
+    "tw_engine_alloc_batch": (I, [P, I, I]),
+    "tw_engine_set_arena": (I, [P, P, SZ]),
+    "tw_engine_arena_bytes_needed": (SZ, [P, I, I]),
+    "tw_engine_reset": (I, [P]),
+    "tw_engine_cache_ptr": (P, [P, I, I]),
+    "tw_engine_positions": (P, [P]),
+    "tw_engine_rotation": (P, [P]),
+    "tw_engine_set_positions": (I, [P, P, I]),
+    "tw_engine_layer_step": (I, [P, I, P, P, P, P, P]),
+    "tw_engine_decode_step": (I, [P, P, P, P, P, I, P]),
+    "tw_engine_broadcast_prefix": (I, [P, I, I, I, I, P]),
+}
+
+_lib = None
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def load() -> C.CDLL:
+    """Load the shared library once and attach the signatures."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise LibraryMissing(
+            f"{LIB_PATH} is not built. Build it with `python -m triebwerk_amd.build` "
+            "(needs hipcc); there is no fallback path."
+        )
+    lib = C.CDLL(str(LIB_PATH))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here = header and library disagree
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(lib: C.CDLL | None = None) -> None:
+    """Raise if a launcher recorded an error since the last clear."""
+    lib = lib or load()
+    code = lib.tw_kv_last_error()
+    if code != 0:
+        msg = lib.tw_kv_last_error_string().decode()
+        lib.tw_kv_clear_error()
+        raise RuntimeError(f"triebwerk_kv error {code}: {msg}")

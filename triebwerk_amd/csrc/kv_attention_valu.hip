@@ -1,0 +1,309 @@
+// kv_attention_valu.hip -- GQA decode attention over the fp16 or the compressed
+// cache, fp32 vector-ALU version, for gfx950.
+//
+// Replaces gqa_attention_{decode,batch}_kernel (kernels.cu:244-345, 981-1066),
+// turbo_gqa_attention{,_batch}_kernel (kernels.cu:1641-1870) and, with
+// pos = query index, the two causal prefill kernels (kernels.cu:1071-1158,
+// 1874-1960).  The reference gives one 128-thread block per (sequence, query
+// head), walks every K row byte by byte from a single thread and keeps the
+// scores in an fp32 scratch array in memory.  Here:
+//   - a workgroup owns (sequence, KV head, context chunk): the query heads of a
+//     GQA group share every byte that is loaded, and long contexts are split
+//     over workgroups (split-K) with a log-sum-exp merge;
+//   - four adjacent lanes own one token: each loads 16 bytes (32 codes) of the
+//     64-byte K row, so a wave reads 16 tokens per load instruction, dequantizes
+//     in registers through a 16-entry LDS centroid table and reduces the dot
+//     product over the quad with two cross-lane shuffles;
+//   - softmax is online (running max / running sum per lane), so no score ever
+//     goes to memory; V is accumulated in registers in the rotated basis and
+//     rotated back once per (sequence, head) (kernels.cu:1769-1775).
+// Arithmetic is fp32 throughout like the reference; only summation order differs.
+
+#include "kv_common.hpp"
+#include "kv_kernels.hpp"
+
+namespace twkv {
+
+constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / kWave;
+constexpr int kTokensPerIter = kAttnWaves * 16;  // 16 token quads per wave
+constexpr float kNegBig = -1e30f;                // the reference's max init (kernels.cu:1686)
+
+__device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
+    if (a.pos_mode == kPosArray) return a.positions[g];
+    if (a.pos_mode == kPosScalar) return a.pos_scalar;
+    return g;
+}
+
+// Dimension owned by element e (0..31) of lane-in-quad c.
+template <int MODE>
+__device__ __forceinline__ int lane_dim(int c, int e) {
+    if (MODE == 0) return 32 * (e / 8) + 8 * c + (e % 8);  // four 16-byte pieces, interleaved over the quad
+    return 32 * c + e;                                     // one contiguous piece of codes
+}
+
+// Load and dequantize the lane's 32 values of one cache row (one KV head).
+template <int MODE>
+__device__ __forceinline__ void load_vals(const void* __restrict__ base, long long row, int num_kv_heads,
+                                          int h, int c, const float* __restrict__ cent_s, float* vals) {
+    if (MODE == 0) {
+        const half_t* p = reinterpret_cast<const half_t*>(base) + (row * num_kv_heads + h) * kHeadDim;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            half8_t h8 = *reinterpret_cast<const half8_t*>(p + 32 * j + 8 * c);
+#pragma unroll
+            for (int i = 0; i < 8; i++) vals[8 * j + i] = (float)h8[i];
+        }
+    } else if (MODE == 4) {
+        const uint8_t* p = reinterpret_cast<const uint8_t*>(base) + (row * num_kv_heads + h) * 64 + 16 * c;
+        uint4 w4 = *reinterpret_cast<const uint4*>(p);
+        uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) vals[8 * j + i] = cent_s[(w[j] >> (4 * i)) & 15u];
+        }
+    } else {
+        const uint8_t* p = reinterpret_cast<const uint8_t*>(base) + (row * num_kv_heads + h) * 32 + 8 * c;
+        uint2 w2 = *reinterpret_cast<const uint2*>(p);
+        uint32_t w[2] = {w2.x, w2.y};
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) vals[16 * j + i] = cent_s[(w[j] >> (2 * i)) & 3u];
+        }
+    }
+}
+
+// Normalise, rotate back (compressed cache) and store one head.
+// o_s: 128 floats of LDS holding acc / (l + 1e-8).  Called by threads d < 128
+// of a workgroup after a barrier that made o_s visible.
+__device__ __forceinline__ void store_head(const AttnArgs& a, int g, int head, int d, const float* o_s) {
+    float o;
+    if (a.bits == 0) {
+        o = o_s[d];
+    } else {
+        o = 0.0f;
+        const half_t* rot = a.rotation;
+#pragma unroll 8
+        for (int k = 0; k < kHeadDim; k++) o = __builtin_fmaf((float)rot[k * kHeadDim + d], o_s[k], o);
+    }
+    a.out[(long long)g * a.q_stride + (long long)head * kHeadDim + d] = (half_t)o;
+}
+
+template <int MODE, int RT>
+__global__ void __launch_bounds__(kAttnThreads)
+attention_valu_kernel(AttnArgs a) {
+    __shared__ float q_s[RT][kHeadDim];
+    __shared__ float red_s[kAttnWaves][RT][kHeadDim];
+    __shared__ float ml_s[kAttnWaves][RT][2];
+    __shared__ float cent_s[16];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave, lane = tid % kWave;
+    const int qd = lane / 4, c = lane % 4;
+    const int chunk = blockIdx.x;
+    const int g = blockIdx.z;
+    const int group = a.num_heads / a.num_kv_heads;
+    const int subs = group / RT;                // query-head tiles per KV head
+    const int h = blockIdx.y / subs;
+    const int head0 = h * group + (blockIdx.y % subs) * RT;
+
+    const int n = seq_pos(a, g) + 1;
+    const int t0 = chunk * a.chunk_len;
+    if (t0 >= n) return;                        // uniform for the workgroup
+    const int t1 = min(n, t0 + a.chunk_len);
+
+    if (tid < 16) cent_s[tid] = (MODE == 2) ? kCentroids2[tid & 3] : kCentroids4[tid];
+
+    // Query, rotated for the compressed cache: q_rot = R q (kernels.cu:1671-1681).
+    for (int idx = tid; idx < RT * kHeadDim; idx += kAttnThreads) {
+        int r = idx / kHeadDim, d = idx % kHeadDim;
+        const half_t* qh = a.q + (long long)g * a.q_stride + (long long)(head0 + r) * kHeadDim;
+        float val;
+        if (MODE == 0) {
+            val = (float)qh[d];
+        } else {
+            const half8_t* rot8 = reinterpret_cast<const half8_t*>(a.rotation + d * kHeadDim);
+            const half8_t* q8 = reinterpret_cast<const half8_t*>(qh);
+            val = 0.0f;
+            for (int k8 = 0; k8 < kHeadDim / 8; k8++) {
+                half8_t rr = rot8[k8], qq = q8[k8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) val = __builtin_fmaf((float)rr[i], (float)qq[i], val);
+            }
+        }
+        q_s[r][d] = val;
+    }
+    __syncthreads();
+
+    float qreg[RT][32];
+    float acc[RT][32];
+    float m[RT], l[RT];
+#pragma unroll
+    for (int r = 0; r < RT; r++) {
+        m[r] = kNegBig;
+        l[r] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 32; e++) {
+            qreg[r][e] = q_s[r][lane_dim<MODE>(c, e)];
+            acc[r][e] = 0.0f;
+        }
+    }
+    const float scale = 0.08838834764831845f;   // 1/sqrt(128)
+
+    for (int tb = t0; tb < t1; tb += kTokensPerIter) {
+        const int t = tb + wave * 16 + qd;
+        const bool valid = t < t1;
+        const int tc = valid ? t : (t1 - 1);    // clamp: keep the quad shuffles convergent
+        const long long row = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, g, tc);
+        float kn = 1.0f, vn = 1.0f;
+        if (MODE != 0) {
+            kn = (float)a.k_norms[row * a.num_kv_heads + h];
+            vn = (float)a.v_norms[row * a.num_kv_heads + h];
+        }
+        float vals[32];
+        load_vals<MODE>(a.k, row, a.num_kv_heads, h, c, cent_s, vals);
+        float s[RT];
+#pragma unroll
+        for (int r = 0; r < RT; r++) {
+            float dot = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 32; e++) dot = __builtin_fmaf(qreg[r][e], vals[e], dot);
+            dot += __shfl_xor(dot, 1, 64);
+            dot += __shfl_xor(dot, 2, 64);
+            s[r] = dot * (kn * scale);          // kernels.cu:1707
+        }
+        load_vals<MODE>(a.v, row, a.num_kv_heads, h, c, cent_s, vals);
+        if (valid) {
+#pragma unroll
+            for (int r = 0; r < RT; r++) {
+                if (s[r] > m[r]) {              // rare after the first tokens
+                    float alpha = __expf(m[r] - s[r]);
+                    l[r] *= alpha;
+#pragma unroll
+                    for (int e = 0; e < 32; e++) acc[r][e] *= alpha;
+                    m[r] = s[r];
+                }
+                float p = __expf(s[r] - m[r]);
+                l[r] += p;
+                float pv = p * vn;              // (s * vn) * centroid, kernels.cu:1765
+#pragma unroll
+                for (int e = 0; e < 32; e++) acc[r][e] = __builtin_fmaf(pv, vals[e], acc[r][e]);
+            }
+        }
+    }
+
+    // ---- merge the 64 token streams of the workgroup (16 quads x 4 waves)
+    float mw[RT];
+#pragma unroll
+    for (int r = 0; r < RT; r++) mw[r] = wave_max(m[r]);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; r++) ml_s[wave][r][0] = mw[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RT; r++) {
+        float mg = ml_s[0][r][0];
+#pragma unroll
+        for (int w = 1; w < kAttnWaves; w++) mg = fmaxf(mg, ml_s[w][r][0]);
+        float f = __expf(m[r] - mg);            // streams that saw no token: exp(-1e30 - mg) = 0
+        m[r] = mg;
+        l[r] *= f;
+#pragma unroll
+        for (int e = 0; e < 32; e++) acc[r][e] *= f;
+        // sum over the 16 quads of the wave (lanes with equal c)
+#pragma unroll
+        for (int off = 4; off < 64; off <<= 1) {
+            l[r] += __shfl_xor(l[r], off, 64);
+#pragma unroll
+            for (int e = 0; e < 32; e++) acc[r][e] += __shfl_xor(acc[r][e], off, 64);
+        }
+    }
+    if (qd == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; r++) {
+#pragma unroll
+            for (int e = 0; e < 32; e++) red_s[wave][r][lane_dim<MODE>(c, e)] = acc[r][e];
+            if (c == 0) ml_s[wave][r][1] = l[r];
+        }
+    }
+    __syncthreads();
+
+    for (int idx = tid; idx < RT * kHeadDim; idx += kAttnThreads) {
+        int r = idx / kHeadDim, d = idx % kHeadDim;
+        float av = red_s[0][r][d], lv = ml_s[0][r][1], mg = ml_s[0][r][0];
+#pragma unroll
+        for (int w = 1; w < kAttnWaves; w++) {
+            av += red_s[w][r][d];
+            lv += ml_s[w][r][1];
+            mg = fmaxf(mg, ml_s[w][r][0]);
+        }
+        if (a.nsplit > 1) {
+            float* part = a.ws + ((long long)g * a.num_heads + head0 + r) * a.ws_stride +
+                          (long long)chunk * kPartialFloats;
+            part[d] = av;
+            if (d == 0) {
+                part[kHeadDim] = mg;
+                part[kHeadDim + 1] = lv;
+            }
+        } else {
+            q_s[r][d] = av * (1.0f / (lv + 1e-8f));   // kernels.cu:1746
+        }
+    }
+    if (a.nsplit > 1) return;
+    __syncthreads();
+    for (int idx = tid; idx < RT * kHeadDim; idx += kAttnThreads) {
+        int r = idx / kHeadDim, d = idx % kHeadDim;
+        store_head(a, g, head0 + r, d, q_s[r]);
+    }
+}
+
+// Log-sum-exp merge of the split partials, normalisation, rotate-back, store.
+__global__ void __launch_bounds__(kHeadDim)
+attention_merge_kernel(AttnArgs a) {
+    __shared__ float o_s[kHeadDim];
+    const int head = blockIdx.x, g = blockIdx.y, d = threadIdx.x;
+    const int n = seq_pos(a, g) + 1;
+    int nchunks = (n + a.chunk_len - 1) / a.chunk_len;
+    if (nchunks > a.nsplit) nchunks = a.nsplit;
+    const float* part = a.ws + ((long long)g * a.num_heads + head) * a.ws_stride;
+    float mg = kNegBig;
+    for (int cidx = 0; cidx < nchunks; cidx++) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
+    float lsum = 0.0f, av = 0.0f;
+    for (int cidx = 0; cidx < nchunks; cidx++) {
+        const float* pc = part + (long long)cidx * kPartialFloats;
+        float f = __expf(pc[kHeadDim] - mg);
+        lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);
+        av = __builtin_fmaf(pc[d], f, av);
+    }
+    o_s[d] = av * (1.0f / (lsum + 1e-8f));
+    __syncthreads();
+    store_head(a, g, head, d, o_s);
+}
+
+template <int MODE>
+static void launch_valu_mode(const AttnArgs& a, hipStream_t s) {
+    const int group = a.num_heads / a.num_kv_heads;
+    const int rt = (group % 4 == 0) ? 4 : (group % 2 == 0) ? 2 : 1;
+    dim3 grid(a.nsplit, a.num_kv_heads * (group / rt), a.G);
+    dim3 block(kAttnThreads);
+    if (rt == 4) hipLaunchKernelGGL((attention_valu_kernel<MODE, 4>), grid, block, 0, s, a);
+    else if (rt == 2) hipLaunchKernelGGL((attention_valu_kernel<MODE, 2>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((attention_valu_kernel<MODE, 1>), grid, block, 0, s, a);
+}
+
+void launch_attention_valu(const AttnArgs& a, hipStream_t s) {
+    if (a.G <= 0) return;
+    if (a.bits == 0) launch_valu_mode<0>(a, s);
+    else if (a.bits == 4) launch_valu_mode<4>(a, s);
+    else launch_valu_mode<2>(a, s);
+}
+
+void launch_attention_merge(const AttnArgs& a, hipStream_t s) {
+    if (a.G <= 0 || a.nsplit <= 1) return;
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(a.num_heads, a.G), dim3(kHeadDim), 0, s, a);
+}
+
+}  // namespace twkv

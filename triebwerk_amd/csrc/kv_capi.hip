@@ -1,0 +1,385 @@
+// kv_capi.hip -- the exported C ABI (include/triebwerk_kv.h): the reference's
+// launcher entry points (engine.cpp:105-171) and the paged / fused additions.
+// Argument checks and launch-geometry policy live here; kernels elsewhere.
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "../../include/triebwerk_kv.h"
+#include "kv_kernels.hpp"
+
+using namespace twkv;
+
+// ---------------------------------------------------------------- error state
+namespace {
+thread_local int g_err = 0;
+thread_local char g_err_msg[256] = "";
+std::atomic<int> g_variant{0};
+std::atomic<int> g_nsplit_override{0};
+
+constexpr int kMaxSplits = 64;
+constexpr int kMinChunk = 128;       // tokens
+constexpr int kTargetGroups = 2048;  // workgroups wanted per launch: 8 per CU on 256 CUs
+
+void set_error(int code, const char* fmt, ...) {
+    if (g_err != 0) return;  // keep the first one
+    g_err = code;
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err_msg, sizeof(g_err_msg), fmt, ap);
+    va_end(ap);
+}
+
+void check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) set_error((int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+const half_t* H(const tw_half* p) { return reinterpret_cast<const half_t*>(p); }
+half_t* H(tw_half* p) { return reinterpret_cast<half_t*>(p); }
+
+bool check_shape(const char* fn, int num_heads, int num_kv_heads, int head_dim) {
+    if (head_dim != kHeadDim) {
+        set_error(1, "%s: head_dim=%d, only 128 is supported", fn, head_dim);
+        return false;
+    }
+    if (num_kv_heads <= 0 || num_heads <= 0 || num_heads % num_kv_heads != 0) {
+        set_error(1, "%s: num_heads=%d not a multiple of num_kv_heads=%d", fn, num_heads, num_kv_heads);
+        return false;
+    }
+    return true;
+}
+
+bool check_bits(const char* fn, int bits) {
+    if (bits != 2 && bits != 4) {
+        set_error(1, "%s: bits=%d, expected 2 or 4", fn, bits);
+        return false;
+    }
+    return true;
+}
+
+// Split the context over workgroups.  ctx_bound: upper bound of positions+1
+// known to the host (max_seq_len, or pos+1 for the by-value entry points).
+// ws_floats_per_head: room per (sequence, head) in the caller's workspace.
+void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
+    if (ctx_bound < 1) ctx_bound = 1;
+    const int group = a.num_heads / a.num_kv_heads;
+    const int rt = (group % 4 == 0) ? 4 : (group % 2 == 0) ? 2 : 1;
+    const long long base_groups = (long long)a.G * a.num_kv_heads * (group / rt);
+    int want = g_nsplit_override.load();
+    if (want <= 0) want = (int)((kTargetGroups + base_groups - 1) / base_groups);
+    int max_by_ctx = (ctx_bound + kMinChunk - 1) / kMinChunk;
+    int max_by_ws = a.ws ? (int)(ws_floats_per_head / kPartialFloats) : 1;
+    int nsplit = want;
+    if (nsplit > max_by_ctx) nsplit = max_by_ctx;
+    if (nsplit > max_by_ws) nsplit = max_by_ws;
+    if (nsplit > kMaxSplits) nsplit = kMaxSplits;
+    if (nsplit < 1) nsplit = 1;
+    int chunk = (ctx_bound + nsplit - 1) / nsplit;
+    chunk = (chunk + 63) / 64 * 64;
+    nsplit = (ctx_bound + chunk - 1) / chunk;
+    a.nsplit = nsplit;
+    a.chunk_len = chunk;
+    a.ws_stride = ws_floats_per_head;
+}
+
+void run_attention(AttnArgs& a, hipStream_t s, const char* fn) {
+    bool done = false;
+    int variant = g_variant.load();
+    if (a.bits != 0 && variant != 1) done = launch_attention_mfma(a, s);
+    if (!done) launch_attention_valu(a, s);
+    launch_attention_merge(a, s);
+    check_launch(fn);
+}
+}  // namespace
+
+extern "C" {
+
+int tw_kv_last_error(void) { return g_err; }
+const char* tw_kv_last_error_string(void) { return g_err_msg; }
+void tw_kv_clear_error(void) { g_err = 0; g_err_msg[0] = 0; }
+const char* tw_kv_build_info(void) { return "triebwerk_kv gfx950 " __DATE__ " " __TIME__; }
+void tw_kv_set_attention_variant(int v) { g_variant.store(v); }
+int tw_kv_get_attention_variant(void) { return g_variant.load(); }
+void tw_kv_set_num_splits(int n) { g_nsplit_override.store(n); }
+
+size_t tw_attention_workspace_floats(int G, int num_heads, int max_context) {
+    (void)max_context;
+    return (size_t)G * num_heads * kMaxSplits * kPartialFloats;
+}
+
+// ---------------------------------------------------------------- append
+void launch_kv_cache_write_batch(tw_half* ck, tw_half* cv, const tw_half* k, const tw_half* v,
+                                 const int* pos, int msl, int G, int kv_dim, hipStream_t s) {
+    launch_kv_write(H(ck), H(cv), H(k), H(v), pos, nullptr, 0, msl, G, kv_dim, s);
+    check_launch("launch_kv_cache_write_batch");
+}
+
+void tw_paged_kv_cache_write_batch(tw_half* ck, tw_half* cv, const tw_half* k, const tw_half* v,
+                                   const int* positions, const int* block_table, int bt_stride,
+                                   int G, int kv_dim, hipStream_t s) {
+    if (!block_table) { set_error(1, "tw_paged_kv_cache_write_batch: block_table is NULL"); return; }
+    launch_kv_write(H(ck), H(cv), H(k), H(v), positions, block_table, bt_stride, 0, G, kv_dim, s);
+    check_launch("tw_paged_kv_cache_write_batch");
+}
+
+static void quantize_common(const char* fn, uint8_t* c0, tw_half* n0, const tw_half* s0,
+                            uint8_t* c1, tw_half* n1, const tw_half* s1, int nstreams,
+                            const tw_half* rotation, const int* positions, const int* block_table,
+                            int bt_stride, long long seq_stride_rows, int token_list, int nrows,
+                            int num_kv_heads, int head_dim, int kv_dim, int bits, hipStream_t s) {
+    if (!check_shape(fn, num_kv_heads, num_kv_heads, head_dim) || !check_bits(fn, bits)) return;
+    if (kv_dim < num_kv_heads * head_dim) {
+        set_error(1, "%s: kv_dim=%d smaller than num_kv_heads*head_dim", fn, kv_dim);
+        return;
+    }
+    QuantArgs a;
+    memset(&a, 0, sizeof(a));
+    a.codes[0] = c0; a.norms[0] = H(n0); a.src[0] = H(s0);
+    a.codes[1] = c1; a.norms[1] = H(n1); a.src[1] = H(s1);
+    a.nstreams = nstreams;
+    a.rotation = H(rotation);
+    a.positions = positions;
+    a.block_table = block_table;
+    a.bt_stride = bt_stride;
+    a.seq_stride_rows = seq_stride_rows;
+    a.token_list = token_list;
+    a.nrows = nrows;
+    a.num_kv_heads = num_kv_heads;
+    a.kv_dim = kv_dim;
+    launch_turbo_quantize(a, bits, s);
+    check_launch(fn);
+}
+
+void launch_turbo_kv_quantize(uint8_t* cache_q, tw_half* cache_norms, const tw_half* kv_buf,
+                              const tw_half* rotation, const int* positions, int max_seq_len,
+                              int num_tokens, int num_kv_heads, int head_dim, int kv_dim,
+                              int bits, hipStream_t s) {
+    quantize_common("launch_turbo_kv_quantize", cache_q, cache_norms, kv_buf, nullptr, nullptr,
+                    nullptr, 1, rotation, positions, nullptr, 0, max_seq_len, 1, num_tokens,
+                    num_kv_heads, head_dim, kv_dim, bits, s);
+}
+
+void launch_turbo_kv_quantize_batch(uint8_t* cache_q, tw_half* cache_norms, const tw_half* kv_buf,
+                                    const tw_half* rotation, const int* positions, int max_seq_len,
+                                    int G, int num_kv_heads, int head_dim, int kv_dim,
+                                    int bits, hipStream_t s) {
+    quantize_common("launch_turbo_kv_quantize_batch", cache_q, cache_norms, kv_buf, nullptr,
+                    nullptr, nullptr, 1, rotation, positions, nullptr, 0, max_seq_len, 0, G,
+                    num_kv_heads, head_dim, kv_dim, bits, s);
+}
+
+void tw_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q, tw_half* v_norms,
+                              const tw_half* k_buf, const tw_half* v_buf, const tw_half* rotation,
+                              const int* positions, int max_seq_len, int G, int num_kv_heads,
+                              int head_dim, int kv_dim, int bits, hipStream_t s) {
+    quantize_common("tw_turbo_kv_append_batch", ck_q, k_norms, k_buf, cv_q, v_norms, v_buf, 2,
+                    rotation, positions, nullptr, 0, max_seq_len, 0, G, num_kv_heads, head_dim,
+                    kv_dim, bits, s);
+}
+
+void tw_paged_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q,
+                                    tw_half* v_norms, const tw_half* k_buf, const tw_half* v_buf,
+                                    const tw_half* rotation, const int* positions,
+                                    const int* block_table, int bt_stride, int G,
+                                    int num_kv_heads, int head_dim, int kv_dim, int bits,
+                                    hipStream_t s) {
+    if (!block_table) { set_error(1, "tw_paged_turbo_kv_append_batch: block_table is NULL"); return; }
+    quantize_common("tw_paged_turbo_kv_append_batch", ck_q, k_norms, k_buf, cv_q, v_norms, v_buf,
+                    2, rotation, positions, block_table, bt_stride, 0, 0, G, num_kv_heads,
+                    head_dim, kv_dim, bits, s);
+}
+
+void launch_increment_positions(int* positions, int G, hipStream_t s) {
+    launch_increment(positions, G, s);
+    check_launch("launch_increment_positions");
+}
+
+// ---------------------------------------------------------------- attention
+static void fill_common(AttnArgs& a, tw_half* out, const tw_half* q, int q_stride, const void* k,
+                        const void* v, const tw_half* kn, const tw_half* vn, const tw_half* rot,
+                        int G, int num_heads, int num_kv_heads, int bits, float* ws) {
+    memset(&a, 0, sizeof(a));
+    a.q = H(q); a.out = H(out); a.q_stride = q_stride;
+    a.k = k; a.v = v; a.k_norms = H(kn); a.v_norms = H(vn); a.rotation = H(rot);
+    a.G = G; a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.bits = bits;
+    a.ws = ws;
+}
+
+void launch_gqa_attention(const tw_half* q, const tw_half* k_cache, const tw_half* v_cache,
+                          tw_half* output, float* attn_scratch, int pos, int max_seq_len,
+                          int num_heads, int num_kv_heads, int head_dim, hipStream_t stream) {
+    if (!check_shape("launch_gqa_attention", num_heads, num_kv_heads, head_dim)) return;
+    if (pos < 0) { set_error(1, "launch_gqa_attention: pos=%d", pos); return; }
+    AttnArgs a;
+    fill_common(a, output, q, num_heads * head_dim, k_cache, v_cache, nullptr, nullptr, nullptr, 1,
+                num_heads, num_kv_heads, 0, attn_scratch);
+    a.pos_mode = kPosScalar; a.pos_scalar = pos; a.seq_stride_rows = 0;
+    plan_splits(a, pos + 1, max_seq_len);
+    run_attention(a, stream, "launch_gqa_attention");
+}
+
+void launch_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half* ck,
+                                const tw_half* cv, float* as, const int* pos, int msl, int G,
+                                int num_heads, int num_kv_heads, int head_dim, int q_dim,
+                                int kv_dim, hipStream_t s) {
+    if (!check_shape("launch_gqa_attention_batch", num_heads, num_kv_heads, head_dim)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "launch_gqa_attention_batch: kv_dim=%d != num_kv_heads*head_dim", kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck, cv, nullptr, nullptr, nullptr, G, num_heads, num_kv_heads, 0, as);
+    a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    plan_splits(a, msl, msl);
+    run_attention(a, s, "launch_gqa_attention_batch");
+}
+
+void launch_gqa_prefill_attention(tw_half* out, const tw_half* q, const tw_half* ck,
+                                  const tw_half* cv, float* as, int T, int msl, int num_heads,
+                                  int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                  hipStream_t s) {
+    (void)msl;
+    if (!check_shape("launch_gqa_prefill_attention", num_heads, num_kv_heads, head_dim)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "launch_gqa_prefill_attention: kv_dim=%d != num_kv_heads*head_dim", kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck, cv, nullptr, nullptr, nullptr, T, num_heads, num_kv_heads, 0, as);
+    a.pos_mode = kPosIota; a.seq_stride_rows = 0;
+    plan_splits(a, T, T);   // scratch is T floats per (query, head), kernels.cu:1088
+    run_attention(a, s, "launch_gqa_prefill_attention");
+}
+
+void launch_turbo_gqa_attention(const tw_half* q, const uint8_t* ck_q, const uint8_t* cv_q,
+                                const tw_half* k_norms, const tw_half* v_norms,
+                                const tw_half* rotation, tw_half* output, float* as, int pos,
+                                int msl, int num_heads, int num_kv_heads, int head_dim, int bits,
+                                hipStream_t s) {
+    if (!check_shape("launch_turbo_gqa_attention", num_heads, num_kv_heads, head_dim) ||
+        !check_bits("launch_turbo_gqa_attention", bits)) return;
+    if (pos < 0) { set_error(1, "launch_turbo_gqa_attention: pos=%d", pos); return; }
+    AttnArgs a;
+    fill_common(a, output, q, num_heads * head_dim, ck_q, cv_q, k_norms, v_norms, rotation, 1,
+                num_heads, num_kv_heads, bits, as);
+    a.pos_mode = kPosScalar; a.pos_scalar = pos; a.seq_stride_rows = 0;
+    plan_splits(a, pos + 1, msl);
+    run_attention(a, s, "launch_turbo_gqa_attention");
+}
+
+void launch_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const uint8_t* ck_q,
+                                      const uint8_t* cv_q, const tw_half* k_norms,
+                                      const tw_half* v_norms, const tw_half* rotation, float* as,
+                                      const int* pos, int msl, int G, int num_heads,
+                                      int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                      int bits, hipStream_t s) {
+    if (!check_shape("launch_turbo_gqa_attention_batch", num_heads, num_kv_heads, head_dim) ||
+        !check_bits("launch_turbo_gqa_attention_batch", bits)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "launch_turbo_gqa_attention_batch: kv_dim=%d != num_kv_heads*head_dim", kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads,
+                num_kv_heads, bits, as);
+    a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    plan_splits(a, msl, msl);
+    run_attention(a, s, "launch_turbo_gqa_attention_batch");
+}
+
+void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const uint8_t* ck_q,
+                                        const uint8_t* cv_q, const tw_half* k_norms,
+                                        const tw_half* v_norms, const tw_half* rotation, float* as,
+                                        int T, int msl, int num_heads, int num_kv_heads,
+                                        int head_dim, int q_dim, int kv_dim, int bits,
+                                        hipStream_t s) {
+    (void)msl;
+    if (!check_shape("launch_turbo_gqa_prefill_attention", num_heads, num_kv_heads, head_dim) ||
+        !check_bits("launch_turbo_gqa_prefill_attention", bits)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "launch_turbo_gqa_prefill_attention: kv_dim=%d != num_kv_heads*head_dim", kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, T, num_heads,
+                num_kv_heads, bits, as);
+    a.pos_mode = kPosIota; a.seq_stride_rows = 0;
+    plan_splits(a, T, T);
+    run_attention(a, s, "launch_turbo_gqa_prefill_attention");
+}
+
+void tw_paged_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half* ck,
+                                  const tw_half* cv, float* ws, const int* positions,
+                                  const int* block_table, int bt_stride, int max_context, int G,
+                                  int num_heads, int num_kv_heads, int head_dim, int q_dim,
+                                  int kv_dim, hipStream_t s) {
+    if (!check_shape("tw_paged_gqa_attention_batch", num_heads, num_kv_heads, head_dim)) return;
+    if (!block_table) { set_error(1, "tw_paged_gqa_attention_batch: block_table is NULL"); return; }
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "tw_paged_gqa_attention_batch: kv_dim=%d != num_kv_heads*head_dim", kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck, cv, nullptr, nullptr, nullptr, G, num_heads, num_kv_heads, 0, ws);
+    a.pos_mode = kPosArray; a.positions = positions;
+    a.block_table = block_table; a.bt_stride = bt_stride;
+    plan_splits(a, max_context, (long long)kMaxSplits * kPartialFloats);
+    run_attention(a, s, "tw_paged_gqa_attention_batch");
+}
+
+void tw_paged_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const uint8_t* ck_q,
+                                        const uint8_t* cv_q, const tw_half* k_norms,
+                                        const tw_half* v_norms, const tw_half* rotation, float* ws,
+                                        const int* positions, const int* block_table,
+                                        int bt_stride, int max_context, int G, int num_heads,
+                                        int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                        int bits, hipStream_t s) {
+    if (!check_shape("tw_paged_turbo_gqa_attention_batch", num_heads, num_kv_heads, head_dim) ||
+        !check_bits("tw_paged_turbo_gqa_attention_batch", bits)) return;
+    if (!block_table) { set_error(1, "tw_paged_turbo_gqa_attention_batch: block_table is NULL"); return; }
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "tw_paged_turbo_gqa_attention_batch: kv_dim=%d != num_kv_heads*head_dim", kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads,
+                num_kv_heads, bits, ws);
+    a.pos_mode = kPosArray; a.positions = positions;
+    a.block_table = block_table; a.bt_stride = bt_stride;
+    plan_splits(a, max_context, (long long)kMaxSplits * kPartialFloats);
+    run_attention(a, s, "tw_paged_turbo_gqa_attention_batch");
+}
+
+// ---------------------------------------------------------------- rotation (host)
+// engine.cpp:366-392, same recipe and same library calls so that the matrix is
+// the one the reference engine uploads.
+void tw_make_rotation_host(tw_half* out_host, int d, unsigned seed) {
+    std::mt19937 gen(seed);
+    std::normal_distribution<float> dist(0.0f, 1.0f);
+    std::vector<float> mat((size_t)d * d);
+    for (int i = 0; i < d * d; i++) mat[i] = dist(gen);
+    for (int i = 0; i < d; i++) {
+        for (int j = 0; j < i; j++) {
+            float dot = 0;
+            for (int k = 0; k < d; k++) dot += mat[i * d + k] * mat[j * d + k];
+            for (int k = 0; k < d; k++) mat[i * d + k] -= dot * mat[j * d + k];
+        }
+        float norm = 0;
+        for (int k = 0; k < d; k++) norm += mat[i * d + k] * mat[i * d + k];
+        norm = 1.0f / sqrtf(norm);
+        for (int k = 0; k < d; k++) mat[i * d + k] *= norm;
+    }
+    for (int i = 0; i < d * d; i++) {
+        _Float16 hv = (_Float16)mat[i];
+        memcpy(&out_host[i], &hv, 2);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,86 @@
+// kv_common.hpp -- shared device helpers for the gfx950 KV-cache kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace twkv {
+
+constexpr int kHeadDim = 128;   // the reference kernels hard-size to 128 (kernels.cu:1504)
+constexpr int kWave = 64;       // CDNA wavefront
+constexpr int kPageTokens = 16; // tokens per cache page in the paged layout
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+// Lloyd-Max tables of the reference (kernels.cu:1426-1445).
+__device__ __constant__ const float kCentroids2[4] = {-0.13351f, -0.04003f, 0.04003f, 0.13351f};
+__device__ __constant__ const float kBounds2[3] = {-0.08677f, 0.0f, 0.08677f};
+__device__ __constant__ const float kCentroids4[16] = {
+    -0.24155f, -0.18293f, -0.14304f, -0.11099f, -0.08330f, -0.05806f, -0.03432f, -0.01135f,
+    0.01135f,  0.03432f,  0.05806f,  0.08330f,  0.11099f,  0.14304f,  0.18293f,  0.24155f};
+__device__ __constant__ const float kBounds4[15] = {
+    -0.21224f, -0.16299f, -0.12701f, -0.09715f, -0.07068f, -0.04619f, -0.02284f, 0.00000f,
+    0.02284f,  0.04619f,  0.07068f,  0.09715f,  0.12701f,  0.16299f,  0.21224f};
+
+// Host-side copies for building lookup tables.
+static const float kCentroids2Host[4] = {-0.13351f, -0.04003f, 0.04003f, 0.13351f};
+static const float kCentroids4Host[16] = {
+    -0.24155f, -0.18293f, -0.14304f, -0.11099f, -0.08330f, -0.05806f, -0.03432f, -0.01135f,
+    0.01135f,  0.03432f,  0.05806f,  0.08330f,  0.11099f,  0.14304f,  0.18293f,  0.24155f};
+
+// turbo_quantize of the reference (kernels.cu:1448-1473) with the boundaries as
+// immediates: strict `<` for 4 bits (a value on a boundary goes up, NaN -> 15),
+// a count of `>=` for 2 bits (NaN -> 0).
+__device__ __forceinline__ int turbo_quantize(float val, int bits) {
+    if (bits == 4) {
+        int idx;
+        if (val < 0.00000f) {
+            if (val < -0.09715f) {
+                if (val < -0.16299f) idx = val < -0.21224f ? 0 : 1;
+                else idx = val < -0.12701f ? 2 : 3;
+            } else {
+                if (val < -0.04619f) idx = val < -0.07068f ? 4 : 5;
+                else idx = val < -0.02284f ? 6 : 7;
+            }
+        } else {
+            if (val < 0.09715f) {
+                if (val < 0.04619f) idx = val < 0.02284f ? 8 : 9;
+                else idx = val < 0.07068f ? 10 : 11;
+            } else {
+                if (val < 0.16299f) idx = val < 0.12701f ? 12 : 13;
+                else idx = val < 0.21224f ? 14 : 15;
+            }
+        }
+        return idx;
+    }
+    return (int)(val >= -0.08677f) + (int)(val >= 0.0f) + (int)(val >= 0.08677f);
+}
+
+// Cache row of position p of sequence g: the reference's g*msl + p
+// (kernels.cu:973, 1629, 1690), or the paged indirection.
+__device__ __forceinline__ long long cache_row(const int* __restrict__ block_table, int bt_stride,
+                                               long long seq_stride_rows, int g, int p) {
+    if (block_table) {
+        int page = block_table[(long long)g * bt_stride + (p / kPageTokens)];
+        return (long long)page * kPageTokens + (p % kPageTokens);
+    }
+    return (long long)g * seq_stride_rows + p;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+}  // namespace twkv

@@ -1,0 +1,331 @@
+// kv_engine.hip -- host-side owner of the KV cache: the slice of the reference's
+// InferenceEngine (model.h:373-493, engine.cpp) that the KV-cache path needs.
+//
+//   constructor / kv_bits switch ....... engine.cpp:300-317
+//   rotation matrix .................... engine.cpp:366-392
+//   batch arena, 256-byte bump carve ... engine.cpp:1338-1560, model.h:264-279
+//   external arena ..................... engine.cpp:1609-1620
+//   reset / zero-fill .................. engine.cpp:893-916, 2262-2283
+//   append -> attention per layer ...... engine.cpp:1979-2006
+//   decode-step graph .................. engine.cpp:2369-2412, 2472-2480
+//   prefix broadcast ................... engine.cpp:2173-2214
+//
+// Everything else the reference engine owns (weights, GEMMs, sampling) is not
+// part of this library.
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/triebwerk_kv.h"
+
+namespace {
+constexpr int kMaxLayers = 128;  // model.h:9
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }  // GpuArena::alloc, model.h:270-275
+}  // namespace
+
+struct tw_engine {
+    int max_seq_len = 1024;
+    int kv_bits = 0;
+    tw_model_shape shape{28, 16, 8, 128};  // ModelConfig::qwen3_0_6b(), model.h:66-74
+
+    // batch state (BatchState, model.h:283-330)
+    int G = 0;
+    int batch_msl = 0;
+    char* arena = nullptr;
+    size_t arena_cap = 0;
+    bool arena_owned = false;
+    void* cache[kMaxLayers][4] = {};  // keys, values, key norms, value norms
+    float* attn_scores = nullptr;     // G * num_heads * msl floats, engine.cpp:1371
+    int* d_positions = nullptr;
+    tw_half* d_rotation = nullptr;
+
+    hipStream_t stream = nullptr;     // engine_stream_, engine.cpp:309
+
+    // captured decode step
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    const void* graph_key[4] = {};
+    int graph_G = 0;
+
+    int kv_dim() const { return shape.num_kv_heads * shape.head_dim; }
+    int q_dim() const { return shape.num_heads * shape.head_dim; }
+    // KV_DIM_PACKED, engine.cpp:294
+    size_t kv_dim_packed() const { return kv_bits == 4 ? kv_dim() / 2 : kv_dim() / 4; }
+
+    void drop_graph() {
+        if (graph_exec) { hipGraphExecDestroy(graph_exec); graph_exec = nullptr; }
+        if (graph) { hipGraphDestroy(graph); graph = nullptr; }
+        graph_G = 0;
+    }
+    void drop_arena() {
+        drop_graph();  // the capture holds arena addresses, engine.cpp:1440-1442
+        if (arena && arena_owned) hipFree(arena);
+        arena = nullptr; arena_cap = 0; arena_owned = false;
+        G = 0; batch_msl = 0;
+        memset(cache, 0, sizeof(cache));
+        attn_scores = nullptr; d_positions = nullptr; d_rotation = nullptr;
+    }
+};
+
+namespace {
+
+size_t arena_need(const tw_engine* e, int G, int msl) {
+    size_t need = 0;
+    auto add = [&](size_t bytes) { need = align256(need); need += bytes; };
+    add((size_t)G * e->shape.num_heads * msl * sizeof(float));  // attn_scores
+    for (int i = 0; i < e->shape.num_layers; i++) {
+        if (e->kv_bits == 0) {
+            add((size_t)G * msl * e->kv_dim() * 2);
+            add((size_t)G * msl * e->kv_dim() * 2);
+        } else {
+            add((size_t)G * msl * e->kv_dim_packed());
+            add((size_t)G * msl * e->kv_dim_packed());
+            add((size_t)G * msl * e->shape.num_kv_heads * 2);
+            add((size_t)G * msl * e->shape.num_kv_heads * 2);
+        }
+    }
+    add((size_t)G * sizeof(int));                                                    // positions
+    add((size_t)e->shape.head_dim * e->shape.head_dim * 2);                          // rotation
+    return align256(need);
+}
+
+int carve(tw_engine* e, int G, int msl) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) { off = align256(off); void* p = e->arena + off; off += bytes; return p; };
+    e->attn_scores = (float*)take((size_t)G * e->shape.num_heads * msl * sizeof(float));
+    for (int i = 0; i < e->shape.num_layers; i++) {
+        if (e->kv_bits == 0) {
+            e->cache[i][0] = take((size_t)G * msl * e->kv_dim() * 2);
+            e->cache[i][1] = take((size_t)G * msl * e->kv_dim() * 2);
+            e->cache[i][2] = e->cache[i][3] = nullptr;
+        } else {  // keys_q, values_q, keys_norms, values_norms: engine.cpp:1503-1506
+            e->cache[i][0] = take((size_t)G * msl * e->kv_dim_packed());
+            e->cache[i][1] = take((size_t)G * msl * e->kv_dim_packed());
+            e->cache[i][2] = take((size_t)G * msl * e->shape.num_kv_heads * 2);
+            e->cache[i][3] = take((size_t)G * msl * e->shape.num_kv_heads * 2);
+        }
+    }
+    e->d_positions = (int*)take((size_t)G * sizeof(int));
+    e->d_rotation = (tw_half*)take((size_t)e->shape.head_dim * e->shape.head_dim * 2);
+    if (off > e->arena_cap) return -1;
+    e->G = G;
+    e->batch_msl = msl;
+    if (e->kv_bits > 0) {
+        std::vector<tw_half> rot((size_t)e->shape.head_dim * e->shape.head_dim);
+        tw_make_rotation_host(rot.data(), e->shape.head_dim, 42u);
+        if (hipMemcpy(e->d_rotation, rot.data(), rot.size() * 2, hipMemcpyHostToDevice) != hipSuccess) return -2;
+    }
+    return 0;
+}
+
+hipStream_t pick(tw_engine* e, hipStream_t s) { return s ? s : e->stream; }
+
+// forward_layer_batch steps 4-5, engine.cpp:1979-2006.
+void layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, const tw_half* v,
+                tw_half* out, hipStream_t s) {
+    const tw_model_shape& m = e->shape;
+    if (e->kv_bits == 0) {
+        launch_kv_cache_write_batch((tw_half*)e->cache[layer][0], (tw_half*)e->cache[layer][1], k, v,
+                                    e->d_positions, e->batch_msl, e->G, e->kv_dim(), s);
+        launch_gqa_attention_batch(out, q, (const tw_half*)e->cache[layer][0],
+                                   (const tw_half*)e->cache[layer][1], e->attn_scores, e->d_positions,
+                                   e->batch_msl, e->G, m.num_heads, m.num_kv_heads, m.head_dim,
+                                   e->q_dim(), e->kv_dim(), s);
+    } else {
+        tw_turbo_kv_append_batch((uint8_t*)e->cache[layer][0], (tw_half*)e->cache[layer][2],
+                                 (uint8_t*)e->cache[layer][1], (tw_half*)e->cache[layer][3], k, v,
+                                 e->d_rotation, e->d_positions, e->batch_msl, e->G, m.num_kv_heads,
+                                 m.head_dim, e->kv_dim(), e->kv_bits, s);
+        launch_turbo_gqa_attention_batch(out, q, (const uint8_t*)e->cache[layer][0],
+                                         (const uint8_t*)e->cache[layer][1],
+                                         (const tw_half*)e->cache[layer][2],
+                                         (const tw_half*)e->cache[layer][3], e->d_rotation,
+                                         e->attn_scores, e->d_positions, e->batch_msl, e->G,
+                                         m.num_heads, m.num_kv_heads, m.head_dim, e->q_dim(),
+                                         e->kv_dim(), e->kv_bits, s);
+    }
+}
+
+void all_layers(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v, tw_half* out,
+                hipStream_t s) {
+    const size_t qs = (size_t)e->G * e->q_dim(), ks = (size_t)e->G * e->kv_dim();
+    for (int l = 0; l < e->shape.num_layers; l++)
+        layer_step(e, l, q + l * qs, k + l * ks, v + l * ks, out + l * qs, s);
+    launch_increment_positions(e->d_positions, e->G, s);  // engine.cpp:2394
+}
+
+}  // namespace
+
+extern "C" {
+
+tw_engine* tw_engine_create(int max_seq_len, int kv_bits) {
+    tw_engine* e = new (std::nothrow) tw_engine();
+    if (!e) return nullptr;
+    e->max_seq_len = max_seq_len;
+    e->kv_bits = kv_bits;
+    if (kv_bits != 0 && kv_bits != 2 && kv_bits != 4) {  // engine.cpp:310-313
+        fprintf(stderr, "WARNING: kv_bits=%d not supported, using 0 (fp16)\n", kv_bits);
+        e->kv_bits = 0;
+    }
+    return e;
+}
+
+void tw_engine_destroy(tw_engine* e) {
+    if (!e) return;
+    e->drop_arena();
+    if (e->stream) hipStreamDestroy(e->stream);
+    delete e;
+}
+
+int tw_engine_kv_bits(const tw_engine* e) { return e->kv_bits; }
+int tw_engine_max_seq_len(const tw_engine* e) { return e->max_seq_len; }
+
+int tw_engine_set_shape(tw_engine* e, const tw_model_shape* shape) {
+    if (!shape || shape->num_layers < 1 || shape->num_layers > kMaxLayers || shape->head_dim != 128 ||
+        shape->num_kv_heads < 1 || shape->num_heads % shape->num_kv_heads != 0)
+        return -1;
+    e->drop_arena();
+    e->shape = *shape;
+    return 0;
+}
+
+size_t tw_engine_arena_bytes_needed(const tw_engine* e, int G, int max_seq_len) {
+    return arena_need(e, G, max_seq_len);
+}
+
+int tw_engine_alloc_batch(tw_engine* e, int G, int max_seq_len) {
+    if (G < 1 || max_seq_len < 1) return -1;
+    if (!e->stream && hipStreamCreate(&e->stream) != hipSuccess) return -3;
+    // engine.cpp:1339: keep a batch that is already large enough.
+    if (e->arena && e->G >= G && e->batch_msl >= max_seq_len) return 0;
+    size_t need = arena_need(e, G, max_seq_len);
+    if (!(e->arena && !e->arena_owned && e->arena_cap >= need)) {
+        e->drop_arena();
+        void* p = nullptr;
+        if (hipMalloc(&p, need) != hipSuccess) return -2;
+        e->arena = (char*)p;
+        e->arena_cap = need;
+        e->arena_owned = true;
+    } else {
+        e->drop_graph();
+    }
+    int rc = carve(e, G, max_seq_len);
+    if (rc != 0) return rc;
+    return tw_engine_reset(e);
+}
+
+int tw_engine_set_arena(tw_engine* e, void* device_ptr, size_t bytes) {
+    if (!device_ptr || (reinterpret_cast<uintptr_t>(device_ptr) & 255u)) return -1;
+    e->drop_arena();
+    e->arena = (char*)device_ptr;
+    e->arena_cap = bytes;
+    e->arena_owned = false;
+    return 0;
+}
+
+int tw_engine_reset(tw_engine* e) {
+    if (!e->arena || e->G == 0) return 0;
+    hipStream_t s = e->stream;
+    const size_t rows = (size_t)e->G * e->batch_msl;
+    for (int i = 0; i < e->shape.num_layers; i++) {
+        if (e->kv_bits == 0) {
+            hipMemsetAsync(e->cache[i][0], 0, rows * e->kv_dim() * 2, s);
+            hipMemsetAsync(e->cache[i][1], 0, rows * e->kv_dim() * 2, s);
+        } else {
+            hipMemsetAsync(e->cache[i][0], 0, rows * e->kv_dim_packed(), s);
+            hipMemsetAsync(e->cache[i][1], 0, rows * e->kv_dim_packed(), s);
+            hipMemsetAsync(e->cache[i][2], 0, rows * e->shape.num_kv_heads * 2, s);
+            hipMemsetAsync(e->cache[i][3], 0, rows * e->shape.num_kv_heads * 2, s);
+        }
+    }
+    hipMemsetAsync(e->d_positions, 0, (size_t)e->G * sizeof(int), s);
+    return hipStreamSynchronize(s) == hipSuccess ? 0 : -1;
+}
+
+void* tw_engine_cache_ptr(tw_engine* e, int layer, int which) {
+    if (layer < 0 || layer >= e->shape.num_layers || which < 0 || which > 3) return nullptr;
+    return e->cache[layer][which];
+}
+int* tw_engine_positions(tw_engine* e) { return e->d_positions; }
+const tw_half* tw_engine_rotation(tw_engine* e) { return e->kv_bits > 0 ? e->d_rotation : nullptr; }
+
+int tw_engine_set_positions(tw_engine* e, const int* host_positions, int G) {
+    if (!e->d_positions || G > e->G) return -1;
+    for (int g = 0; g < G; g++)
+        if (host_positions[g] < 0 || host_positions[g] >= e->batch_msl) return -2;
+    // engine.cpp:2364
+    return hipMemcpy(e->d_positions, host_positions, (size_t)G * sizeof(int), hipMemcpyHostToDevice) == hipSuccess ? 0 : -3;
+}
+
+int tw_engine_layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k,
+                         const tw_half* v, tw_half* out, hipStream_t s) {
+    if (!e->arena || layer < 0 || layer >= e->shape.num_layers) return -1;
+    tw_kv_clear_error();
+    layer_step(e, layer, q, k, v, out, pick(e, s));
+    return tw_kv_last_error();
+}
+
+int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v,
+                          tw_half* out, int use_graph, hipStream_t s) {
+    if (!e->arena) return -1;
+    s = pick(e, s);
+    tw_kv_clear_error();
+    if (!use_graph) {
+        all_layers(e, q, k, v, out, s);
+        return tw_kv_last_error();
+    }
+    const void* key[4] = {q, k, v, out};
+    if (!e->graph_exec || e->graph_G != e->G || memcmp(key, e->graph_key, sizeof(key)) != 0) {
+        e->drop_graph();
+        // Capture records the launches without running them, so unlike the
+        // reference (engine.cpp:2414-2444) nothing has to be re-prefilled.
+        if (hipStreamBeginCapture(s, hipStreamCaptureModeRelaxed) != hipSuccess) return -4;
+        all_layers(e, q, k, v, out, s);
+        hipGraph_t g = nullptr;
+        hipError_t err = hipStreamEndCapture(s, &g);
+        if (err != hipSuccess || !g || tw_kv_last_error() != 0) {
+            if (g) hipGraphDestroy(g);
+            (void)hipGetLastError();
+            return -5;
+        }
+        if (hipGraphInstantiate(&e->graph_exec, g, nullptr, nullptr, 0) != hipSuccess) {
+            hipGraphDestroy(g);
+            e->graph_exec = nullptr;
+            return -6;
+        }
+        e->graph = g;
+        e->graph_G = e->G;
+        memcpy(e->graph_key, key, sizeof(key));
+    }
+    return hipGraphLaunch(e->graph_exec, s) == hipSuccess ? 0 : -7;
+}
+
+int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end, int T, hipStream_t s) {
+    if (!e->arena || src < 0 || src >= e->G || dst_begin < 0 || dst_end > e->G || T < 0 || T > e->batch_msl)
+        return -1;
+    s = pick(e, s);
+    const size_t msl = (size_t)e->batch_msl;
+    for (int l = 0; l < e->shape.num_layers; l++) {
+        for (int which = 0; which < 4; which++) {
+            char* base = (char*)e->cache[l][which];
+            if (!base) continue;
+            size_t row_bytes;
+            if (e->kv_bits == 0) row_bytes = (size_t)e->kv_dim() * 2;
+            else row_bytes = which < 2 ? e->kv_dim_packed() : (size_t)e->shape.num_kv_heads * 2;
+            for (int g = dst_begin; g < dst_end; g++) {
+                if (g == src) continue;
+                if (hipMemcpyAsync(base + g * msl * row_bytes, base + src * msl * row_bytes,
+                                   (size_t)T * row_bytes, hipMemcpyDeviceToDevice, s) != hipSuccess)
+                    return -2;
+            }
+        }
+    }
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,68 @@
+// kv_kernels.hpp -- internal launch interface between the C ABI (kv_capi.hip)
+// and the kernel files.  Nothing here is exported.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kv_common.hpp"
+
+namespace twkv {
+
+// ---------------------------------------------------------------- append
+struct QuantArgs {
+    // One or two streams (K, V) quantized by the same launch.
+    uint8_t* codes[2];
+    half_t* norms[2];
+    const half_t* src[2];   // (nrows, kv_dim) fp16
+    int nstreams;
+    const half_t* rotation; // (128,128) fp16 row major
+    const int* positions;   // device int32[nrows]
+    const int* block_table; // NULL = contiguous cache
+    int bt_stride;
+    long long seq_stride_rows;  // max_seq_len for the contiguous batch layout
+    int token_list;         // 1: row r goes to cache row positions[r] of sequence 0
+    int nrows;              // G, or num_tokens
+    int num_kv_heads;
+    int kv_dim;
+};
+
+void launch_kv_write(half_t* ck, half_t* cv, const half_t* k, const half_t* v,
+                     const int* positions, const int* block_table, int bt_stride,
+                     long long seq_stride_rows, int G, int kv_dim, hipStream_t s);
+void launch_turbo_quantize(const QuantArgs& a, int bits, hipStream_t s);
+void launch_increment(int* positions, int G, hipStream_t s);
+
+// ---------------------------------------------------------------- attention
+enum PosMode { kPosArray = 0, kPosScalar = 1, kPosIota = 2 };
+
+struct AttnArgs {
+    const half_t* q;        // (G, q_stride)
+    half_t* out;            // (G, q_stride)
+    int q_stride;
+    const void* k;          // fp16 rows (kv_bits 0) or packed codes
+    const void* v;
+    const half_t* k_norms;  // compressed only: (rows, num_kv_heads)
+    const half_t* v_norms;
+    const half_t* rotation; // compressed only
+    const int* positions;   // kPosArray
+    int pos_scalar;         // kPosScalar
+    int pos_mode;           // kPosIota: sequence g attends rows 0..g (causal prefill)
+    const int* block_table; // NULL = contiguous
+    int bt_stride;
+    long long seq_stride_rows;  // msl (batch), 0 (single sequence / prefill)
+    int G, num_heads, num_kv_heads;
+    int bits;               // 0, 2, 4
+    float* ws;              // split workspace
+    long long ws_stride;    // floats per (g, head)
+    int nsplit;             // >= 1; 1 = no workspace, one workgroup walks the sequence
+    int chunk_len;          // tokens per split, multiple of 64
+};
+
+constexpr int kPartialFloats = kHeadDim + 2;  // acc[128], running max, running sum
+
+void launch_attention_valu(const AttnArgs& a, hipStream_t s);
+void launch_attention_merge(const AttnArgs& a, hipStream_t s);
+bool launch_attention_mfma(const AttnArgs& a, hipStream_t s);  // false = shape not covered
+
+}  // namespace twkv

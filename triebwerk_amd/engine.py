@@ -1,0 +1,127 @@
+"""``Engine(max_seq_len, kv_bits)``: the KV-cache face of the reference's
+``jetson_engine.Engine`` (engine/engine_py.cpp:21-45), backed by the C++ engine
+object behind the C ABI (``tw_engine_*`` in include/triebwerk_kv.h).
+
+The reference class reaches append and attention only through ``generate*``;
+weights, GEMMs and sampling are not part of this library, so the cache calls
+are exposed directly instead: ``alloc_batch``, ``layer_step``, ``decode_step``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from .kvcache import _ptr, _stream
+
+
+class Engine:
+    def __init__(self, max_seq_len: int = 1024, kv_bits: int = 0):
+        # engine_py.cpp:22: py::init<int,int>(), max_seq_len=1024, kv_bits=0
+        self._lib = _lib.load()
+        self._h = self._lib.tw_engine_create(int(max_seq_len), int(kv_bits))
+        if not self._h:
+            raise RuntimeError("tw_engine_create failed")
+        self._arena = None
+        self._shape = (28, 16, 8, 128)
+        self._G = 0
+        self._msl = 0
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.tw_engine_destroy(h)
+
+    # ---- the reference's surface for this path
+    def kv_bits(self) -> int:  # engine_py.cpp:25
+        return self._lib.tw_engine_kv_bits(self._h)
+
+    def reset(self) -> None:  # engine_py.cpp:44
+        rc = self._lib.tw_engine_reset(self._h)
+        if rc != 0:
+            raise RuntimeError(f"reset failed ({rc})")
+
+    # ---- cache management the reference does inside load_config / generate_batch
+    def max_seq_len(self) -> int:
+        return self._lib.tw_engine_max_seq_len(self._h)
+
+    def set_shape(self, num_layers: int, num_heads: int, num_kv_heads: int, head_dim: int = 128) -> None:
+        shape = _lib.ModelShape(num_layers, num_heads, num_kv_heads, head_dim)
+        if self._lib.tw_engine_set_shape(self._h, C.byref(shape)) != 0:
+            raise ValueError("unsupported model shape (head_dim must be 128, heads a multiple of kv heads)")
+        self._shape = (num_layers, num_heads, num_kv_heads, head_dim)
+        self._arena = None
+
+    def alloc_batch(self, G: int, max_seq_len: int, device="cuda") -> None:
+        """Carve the caches for G sequences out of one torch-owned arena
+        (the reference's set_arena + alloc_batch, engine.cpp:1609-1620, 1338)."""
+        need = self._lib.tw_engine_arena_bytes_needed(self._h, G, max_seq_len)
+        arena = torch.empty(need + 256, dtype=torch.uint8, device=device)
+        base = (arena.data_ptr() + 255) & ~255
+        rc = self._lib.tw_engine_set_arena(self._h, base, need)
+        if rc != 0:
+            raise RuntimeError(f"set_arena failed ({rc})")
+        self._arena = arena
+        rc = self._lib.tw_engine_alloc_batch(self._h, G, max_seq_len)
+        if rc != 0:
+            raise RuntimeError(f"alloc_batch failed ({rc})")
+        self._G, self._msl = G, max_seq_len
+
+    def _view(self, ptr: int, nbytes: int, dtype, shape):
+        off = ptr - self._arena.data_ptr()
+        return self._arena[off:off + nbytes].view(dtype).view(shape)
+
+    def cache(self, layer: int):
+        """Torch views of one layer's cache: (keys, values, key_norms, value_norms)."""
+        L, H, Hk, D = self._shape
+        G, msl = self._G, self._msl
+        bits = self.kv_bits()
+        ptrs = [self._lib.tw_engine_cache_ptr(self._h, layer, w) for w in range(4)]
+        if bits == 0:
+            n = G * msl * Hk * D * 2
+            return (self._view(ptrs[0], n, torch.float16, (G, msl, Hk * D)),
+                    self._view(ptrs[1], n, torch.float16, (G, msl, Hk * D)), None, None)
+        kvp = Hk * D * bits // 8
+        return (self._view(ptrs[0], G * msl * kvp, torch.uint8, (G, msl, kvp)),
+                self._view(ptrs[1], G * msl * kvp, torch.uint8, (G, msl, kvp)),
+                self._view(ptrs[2], G * msl * Hk * 2, torch.float16, (G, msl, Hk)),
+                self._view(ptrs[3], G * msl * Hk * 2, torch.float16, (G, msl, Hk)))
+
+    def positions(self) -> torch.Tensor:
+        return self._view(self._lib.tw_engine_positions(self._h), self._G * 4, torch.int32, (self._G,))
+
+    def rotation(self):
+        p = self._lib.tw_engine_rotation(self._h)
+        if not p:
+            return None
+        D = self._shape[3]
+        return self._view(p, D * D * 2, torch.float16, (D, D))
+
+    def set_positions(self, positions) -> None:
+        arr = (C.c_int * len(positions))(*[int(x) for x in positions])
+        rc = self._lib.tw_engine_set_positions(self._h, arr, len(positions))
+        if rc != 0:
+            raise ValueError(f"set_positions failed ({rc})")
+
+    def layer_step(self, layer, q, k, v, out, stream=None) -> None:
+        rc = self._lib.tw_engine_layer_step(self._h, layer, _ptr(q, "f16", "q"), _ptr(k, "f16", "k"),
+                                            _ptr(v, "f16", "v"), _ptr(out, "f16", "out"), _stream(stream))
+        if rc != 0:
+            _lib.check(self._lib)
+            raise RuntimeError(f"layer_step failed ({rc})")
+
+    def decode_step(self, q, k, v, out, use_graph: bool = False, stream=None) -> None:
+        """Append + attention for every layer, then positions += 1.
+        q/out: (L, G, H*D); k/v: (L, G, Hk*D)."""
+        rc = self._lib.tw_engine_decode_step(self._h, _ptr(q, "f16", "q"), _ptr(k, "f16", "k"),
+                                             _ptr(v, "f16", "v"), _ptr(out, "f16", "out"),
+                                             1 if use_graph else 0, _stream(stream))
+        if rc != 0:
+            _lib.check(self._lib)
+            raise RuntimeError(f"decode_step failed ({rc})")
+
+    def broadcast_prefix(self, src: int, dst_begin: int, dst_end: int, T: int, stream=None) -> None:
+        rc = self._lib.tw_engine_broadcast_prefix(self._h, src, dst_begin, dst_end, T, _stream(stream))
+        if rc != 0:
+            raise RuntimeError(f"broadcast_prefix failed ({rc})")

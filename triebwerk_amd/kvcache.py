@@ -1,0 +1,218 @@
+"""Python entry points over the C ABI, one per launcher of ``include/triebwerk_kv.h``.
+
+Argument order and meaning are the launchers' own (reference: engine.cpp:105-171);
+tensors replace raw device pointers and the HIP stream defaults to torch's
+current stream.  torch is used for device memory and streams only.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_DT = {"f16": torch.float16, "u8": torch.uint8, "i32": torch.int32, "f32": torch.float32}
+
+
+def _ptr(t, kind: str, name: str):
+    if t is None:
+        return None
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name}: expected a CUDA/HIP tensor")
+    if t.dtype != _DT[kind]:
+        raise TypeError(f"{name}: expected dtype {_DT[kind]}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: tensor must be contiguous")
+    return t.data_ptr()
+
+
+def _stream(stream):
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, torch.cuda.Stream):
+        return stream.cuda_stream
+    return int(stream)
+
+
+def _done(lib):
+    _lib.check(lib)
+
+
+def launch_kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim, stream=None):
+    lib = _lib.load()
+    lib.launch_kv_cache_write_batch(_ptr(ck, "f16", "ck"), _ptr(cv, "f16", "cv"), _ptr(k, "f16", "k"),
+                                    _ptr(v, "f16", "v"), _ptr(pos, "i32", "pos"), msl, G, kv_dim,
+                                    _stream(stream))
+    _done(lib)
+
+
+def launch_turbo_kv_quantize(cache_q, cache_norms, kv_buf, rotation, positions, max_seq_len,
+                             num_tokens, num_kv_heads, head_dim, kv_dim, bits, stream=None):
+    lib = _lib.load()
+    lib.launch_turbo_kv_quantize(_ptr(cache_q, "u8", "cache_q"), _ptr(cache_norms, "f16", "cache_norms"),
+                                 _ptr(kv_buf, "f16", "kv_buf"), _ptr(rotation, "f16", "rotation"),
+                                 _ptr(positions, "i32", "positions"), max_seq_len, num_tokens,
+                                 num_kv_heads, head_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def launch_turbo_kv_quantize_batch(cache_q, cache_norms, kv_buf, rotation, positions, max_seq_len,
+                                   G, num_kv_heads, head_dim, kv_dim, bits, stream=None):
+    lib = _lib.load()
+    lib.launch_turbo_kv_quantize_batch(_ptr(cache_q, "u8", "cache_q"), _ptr(cache_norms, "f16", "cache_norms"),
+                                       _ptr(kv_buf, "f16", "kv_buf"), _ptr(rotation, "f16", "rotation"),
+                                       _ptr(positions, "i32", "positions"), max_seq_len, G,
+                                       num_kv_heads, head_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def launch_gqa_attention(q, k_cache, v_cache, output, attn_scratch, pos, max_seq_len, num_heads,
+                         num_kv_heads, head_dim, stream=None):
+    lib = _lib.load()
+    lib.launch_gqa_attention(_ptr(q, "f16", "q"), _ptr(k_cache, "f16", "k_cache"),
+                             _ptr(v_cache, "f16", "v_cache"), _ptr(output, "f16", "output"),
+                             _ptr(attn_scratch, "f32", "attn_scratch"), pos, max_seq_len, num_heads,
+                             num_kv_heads, head_dim, _stream(stream))
+    _done(lib)
+
+
+def launch_gqa_attention_batch(out, q, ck, cv, scratch, pos, msl, G, num_heads, num_kv_heads,
+                               head_dim, q_dim, kv_dim, stream=None):
+    lib = _lib.load()
+    lib.launch_gqa_attention_batch(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(ck, "f16", "ck"),
+                                   _ptr(cv, "f16", "cv"), _ptr(scratch, "f32", "as"),
+                                   _ptr(pos, "i32", "pos"), msl, G, num_heads, num_kv_heads, head_dim,
+                                   q_dim, kv_dim, _stream(stream))
+    _done(lib)
+
+
+def launch_gqa_prefill_attention(out, q, ck, cv, scratch, T, msl, num_heads, num_kv_heads, head_dim,
+                                 q_dim, kv_dim, stream=None):
+    lib = _lib.load()
+    lib.launch_gqa_prefill_attention(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(ck, "f16", "ck"),
+                                     _ptr(cv, "f16", "cv"), _ptr(scratch, "f32", "as"), T, msl,
+                                     num_heads, num_kv_heads, head_dim, q_dim, kv_dim, _stream(stream))
+    _done(lib)
+
+
+def launch_turbo_gqa_attention(q, ck_q, cv_q, k_norms, v_norms, rotation, output, scratch, pos, msl,
+                               num_heads, num_kv_heads, head_dim, bits, stream=None):
+    lib = _lib.load()
+    lib.launch_turbo_gqa_attention(_ptr(q, "f16", "q"), _ptr(ck_q, "u8", "ck_q"), _ptr(cv_q, "u8", "cv_q"),
+                                   _ptr(k_norms, "f16", "k_norms"), _ptr(v_norms, "f16", "v_norms"),
+                                   _ptr(rotation, "f16", "rotation"), _ptr(output, "f16", "output"),
+                                   _ptr(scratch, "f32", "as"), pos, msl, num_heads, num_kv_heads,
+                                   head_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def launch_turbo_gqa_attention_batch(out, q, ck_q, cv_q, k_norms, v_norms, rotation, scratch, pos,
+                                     msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits,
+                                     stream=None):
+    lib = _lib.load()
+    lib.launch_turbo_gqa_attention_batch(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"),
+                                         _ptr(ck_q, "u8", "ck_q"), _ptr(cv_q, "u8", "cv_q"),
+                                         _ptr(k_norms, "f16", "k_norms"), _ptr(v_norms, "f16", "v_norms"),
+                                         _ptr(rotation, "f16", "rotation"), _ptr(scratch, "f32", "as"),
+                                         _ptr(pos, "i32", "pos"), msl, G, num_heads, num_kv_heads,
+                                         head_dim, q_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def launch_turbo_gqa_prefill_attention(out, q, ck_q, cv_q, k_norms, v_norms, rotation, scratch, T,
+                                       msl, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits,
+                                       stream=None):
+    lib = _lib.load()
+    lib.launch_turbo_gqa_prefill_attention(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"),
+                                           _ptr(ck_q, "u8", "ck_q"), _ptr(cv_q, "u8", "cv_q"),
+                                           _ptr(k_norms, "f16", "k_norms"), _ptr(v_norms, "f16", "v_norms"),
+                                           _ptr(rotation, "f16", "rotation"), _ptr(scratch, "f32", "as"),
+                                           T, msl, num_heads, num_kv_heads, head_dim, q_dim, kv_dim,
+                                           bits, _stream(stream))
+    _done(lib)
+
+
+def launch_increment_positions(positions, G, stream=None):
+    lib = _lib.load()
+    lib.launch_increment_positions(_ptr(positions, "i32", "positions"), G, _stream(stream))
+    _done(lib)
+
+
+def tw_turbo_kv_append_batch(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotation, positions,
+                             max_seq_len, G, num_kv_heads, head_dim, kv_dim, bits, stream=None):
+    lib = _lib.load()
+    lib.tw_turbo_kv_append_batch(_ptr(ck_q, "u8", "ck_q"), _ptr(k_norms, "f16", "k_norms"),
+                                 _ptr(cv_q, "u8", "cv_q"), _ptr(v_norms, "f16", "v_norms"),
+                                 _ptr(k_buf, "f16", "k_buf"), _ptr(v_buf, "f16", "v_buf"),
+                                 _ptr(rotation, "f16", "rotation"), _ptr(positions, "i32", "positions"),
+                                 max_seq_len, G, num_kv_heads, head_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def tw_paged_kv_cache_write_batch(ck, cv, k, v, positions, block_table, bt_stride, G, kv_dim,
+                                  stream=None):
+    lib = _lib.load()
+    lib.tw_paged_kv_cache_write_batch(_ptr(ck, "f16", "ck"), _ptr(cv, "f16", "cv"), _ptr(k, "f16", "k"),
+                                      _ptr(v, "f16", "v"), _ptr(positions, "i32", "positions"),
+                                      _ptr(block_table, "i32", "block_table"), bt_stride, G, kv_dim,
+                                      _stream(stream))
+    _done(lib)
+
+
+def tw_paged_turbo_kv_append_batch(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotation, positions,
+                                   block_table, bt_stride, G, num_kv_heads, head_dim, kv_dim, bits,
+                                   stream=None):
+    lib = _lib.load()
+    lib.tw_paged_turbo_kv_append_batch(_ptr(ck_q, "u8", "ck_q"), _ptr(k_norms, "f16", "k_norms"),
+                                       _ptr(cv_q, "u8", "cv_q"), _ptr(v_norms, "f16", "v_norms"),
+                                       _ptr(k_buf, "f16", "k_buf"), _ptr(v_buf, "f16", "v_buf"),
+                                       _ptr(rotation, "f16", "rotation"),
+                                       _ptr(positions, "i32", "positions"),
+                                       _ptr(block_table, "i32", "block_table"), bt_stride, G,
+                                       num_kv_heads, head_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def tw_paged_gqa_attention_batch(out, q, ck, cv, ws, positions, block_table, bt_stride, max_context,
+                                 G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, stream=None):
+    lib = _lib.load()
+    lib.tw_paged_gqa_attention_batch(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(ck, "f16", "ck"),
+                                     _ptr(cv, "f16", "cv"), _ptr(ws, "f32", "ws"),
+                                     _ptr(positions, "i32", "positions"),
+                                     _ptr(block_table, "i32", "block_table"), bt_stride, max_context,
+                                     G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim,
+                                     _stream(stream))
+    _done(lib)
+
+
+def tw_paged_turbo_gqa_attention_batch(out, q, ck_q, cv_q, k_norms, v_norms, rotation, ws, positions,
+                                       block_table, bt_stride, max_context, G, num_heads,
+                                       num_kv_heads, head_dim, q_dim, kv_dim, bits, stream=None):
+    lib = _lib.load()
+    lib.tw_paged_turbo_gqa_attention_batch(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"),
+                                           _ptr(ck_q, "u8", "ck_q"), _ptr(cv_q, "u8", "cv_q"),
+                                           _ptr(k_norms, "f16", "k_norms"), _ptr(v_norms, "f16", "v_norms"),
+                                           _ptr(rotation, "f16", "rotation"), _ptr(ws, "f32", "ws"),
+                                           _ptr(positions, "i32", "positions"),
+                                           _ptr(block_table, "i32", "block_table"), bt_stride,
+                                           max_context, G, num_heads, num_kv_heads, head_dim, q_dim,
+                                           kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def attention_workspace_floats(G, num_heads, max_context) -> int:
+    return int(_lib.load().tw_attention_workspace_floats(G, num_heads, max_context))
+
+
+def make_rotation(head_dim: int = 128, seed: int = 42) -> torch.Tensor:
+    """The engine's rotation matrix (engine.cpp:366-392) as a CPU fp16 tensor."""
+    out = torch.empty((head_dim, head_dim), dtype=torch.float16)
+    _lib.load().tw_make_rotation_host(out.data_ptr(), head_dim, seed)
+    return out
+
+
+def set_attention_variant(variant: int) -> None:
+    _lib.load().tw_kv_set_attention_variant(int(variant))
+
+
+def set_num_splits(nsplit: int) -> None:
+    _lib.load().tw_kv_set_num_splits(int(nsplit))
