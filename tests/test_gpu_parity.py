@@ -1,0 +1,550 @@
+"""GPU parity: the HIP library, called through its C ABI, against the CPU oracle
+on the same seeded inputs.
+
+Bars (from the task statement of this path):
+  - packed codes, norms and every piece of cache bookkeeping: bit-exact;
+  - attention outputs: max relative error <= 2e-3 in fp16, measured per head
+    vector as ||gpu - oracle||_inf / ||oracle||_inf.
+"""
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import gen
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+D = 128
+
+
+@pytest.fixture(scope="module")
+def kv():
+    import torch
+    from triebwerk_amd import kvcache
+    assert torch.cuda.is_available()
+    return kvcache
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    import torch
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def rel_err(got, want):
+    got = got.astype(np.float64).reshape(-1, D)
+    want = want.astype(np.float64).reshape(-1, D)
+    return float(np.max(np.max(np.abs(got - want), axis=1) / np.max(np.abs(want), axis=1)))
+
+
+def assert_bytes_equal(got, want, what, margin=None):
+    got = np.ascontiguousarray(got).view(np.uint8)
+    want = np.ascontiguousarray(want).view(np.uint8)
+    if np.array_equal(got, want):
+        return
+    bad = np.argwhere(got != want)
+    msg = f"{what}: {len(bad)} of {got.size} bytes differ; first at {bad[0].tolist()}"
+    if margin is not None:
+        msg += f"; smallest boundary margin in the call: {float(margin.min()):.3e}"
+    raise AssertionError(msg)
+
+
+# ------------------------------------------------------------------ fp16 append
+def test_fp16_append_bit_exact(kv, oracle):
+    r = gen.rng(101)
+    G, msl, kv_dim = 4, 24, 1024
+    ck = np.zeros((G, msl, kv_dim), np.float16); cv = np.zeros_like(ck)
+    d_ck, d_cv = dev(ck), dev(cv)
+    pos = np.array([0, 5, 23, 11], np.int32)
+    for step in range(3):
+        k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+        oracle.kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim)
+        kv.launch_kv_cache_write_batch(d_ck, d_cv, dev(k), dev(v), dev(pos), msl, G, kv_dim)
+        pos = (pos + 7) % msl
+    assert_bytes_equal(host(d_ck), ck, "fp16 K cache")
+    assert_bytes_equal(host(d_cv), cv, "fp16 V cache")
+
+
+def test_fp16_append_unaligned_width(kv, oracle):
+    r = gen.rng(102)
+    G, msl, kv_dim = 3, 5, 132  # not a multiple of 8 halves: scalar path
+    ck = np.zeros((G, msl, kv_dim), np.float16); cv = np.zeros_like(ck)
+    d_ck, d_cv = dev(ck), dev(cv)
+    pos = np.array([4, 0, 2], np.int32)
+    k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    oracle.kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim)
+    kv.launch_kv_cache_write_batch(d_ck, d_cv, dev(k), dev(v), dev(pos), msl, G, kv_dim)
+    assert_bytes_equal(host(d_ck), ck, "fp16 K cache")
+    assert_bytes_equal(host(d_cv), cv, "fp16 V cache")
+
+
+def test_increment_positions(kv):
+    pos = np.array([0, 7, 100, 65535], np.int32)
+    d = dev(pos)
+    for _ in range(3):
+        kv.launch_increment_positions(d, 4)
+    assert np.array_equal(host(d), pos + 3)
+
+
+# ------------------------------------------------------------------ compressed append
+def special_rows(r, G, kv_dim):
+    rows, _ = gen.kv_rows_with_outliers(r, (G, kv_dim), kv_dim)
+    rows[1, :D] = 0
+    rows[2] = (rows[2].astype(np.float32) * 1e-3).astype(np.float16)
+    rows[3] = (rows[3].astype(np.float32) * 30).astype(np.float16)
+    rows[4, D:2 * D] = np.float16(6e-8)  # fp16 subnormals
+    return rows
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_turbo_append_batch_bit_exact(kv, oracle, rotation_fixture, bits):
+    r = gen.rng(110 + bits)
+    G, Hk, msl = 64, 8, 12
+    kv_dim = Hk * D
+    kvp = kv_dim * bits // 8
+    rows = special_rows(r, G, kv_dim)
+    pos = r.integers(0, msl, G).astype(np.int32)
+    cq = np.zeros((G, msl, kvp), np.uint8); cn = np.zeros((G, msl, Hk), np.float16)
+    margin = np.zeros((G, kv_dim), np.float32)
+    oracle.turbo_kv_quantize_batch(cq, cn, rows, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits, None, margin)
+    d_cq, d_cn = dev(np.zeros_like(cq)), dev(np.zeros_like(cn))
+    kv.launch_turbo_kv_quantize_batch(d_cq, d_cn, dev(rows), dev(rotation_fixture), dev(pos), msl, G, Hk, D, kv_dim, bits)
+    assert_bytes_equal(host(d_cq), cq, f"{bits}-bit codes", margin)
+    assert_bytes_equal(host(d_cn), cn, "norms")
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_turbo_append_many_rows_bit_exact(kv, oracle, rotation_fixture, bits):
+    """A few hundred thousand coordinates: the tie set, if any, shows up here."""
+    r = gen.rng(120 + bits)
+    G, Hk, msl = 512, 8, 1
+    kv_dim = Hk * D
+    kvp = kv_dim * bits // 8
+    rows = gen.normal_f16(r, (G, kv_dim))
+    pos = np.zeros(G, np.int32)
+    cq = np.zeros((G, msl, kvp), np.uint8); cn = np.zeros((G, msl, Hk), np.float16)
+    margin = np.zeros((G, kv_dim), np.float32)
+    oracle.turbo_kv_quantize_batch(cq, cn, rows, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits, None, margin)
+    d_cq, d_cn = dev(np.zeros_like(cq)), dev(np.zeros_like(cn))
+    kv.launch_turbo_kv_quantize_batch(d_cq, d_cn, dev(rows), dev(rotation_fixture), dev(pos), msl, G, Hk, D, kv_dim, bits)
+    assert_bytes_equal(host(d_cq), cq, f"{bits}-bit codes", margin)
+    assert_bytes_equal(host(d_cn), cn, "norms")
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_turbo_append_token_list_and_fused(kv, oracle, rotation_fixture, bits):
+    r = gen.rng(130 + bits)
+    T, Hk, msl = 37, 8, 64
+    kv_dim = Hk * D
+    kvp = kv_dim * bits // 8
+    rows = gen.normal_f16(r, (T, kv_dim))
+    positions = r.permutation(msl)[:T].astype(np.int32)
+    cq = np.zeros((msl, kvp), np.uint8); cn = np.zeros((msl, Hk), np.float16)
+    oracle.turbo_kv_quantize(cq, cn, rows, rotation_fixture, positions, msl, T, Hk, D, kv_dim, bits)
+    d_cq, d_cn = dev(np.zeros_like(cq)), dev(np.zeros_like(cn))
+    kv.launch_turbo_kv_quantize(d_cq, d_cn, dev(rows), dev(rotation_fixture), dev(positions), msl, T, Hk, D, kv_dim, bits)
+    assert_bytes_equal(host(d_cq), cq, "token-list codes")
+    assert_bytes_equal(host(d_cn), cn, "token-list norms")
+
+    # K and V through one launch == two reference-style launches
+    G = 9
+    k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    pos = r.integers(0, msl, G).astype(np.int32)
+    want = []
+    for src in (k, v):
+        q_ = np.zeros((G, msl, kvp), np.uint8); n_ = np.zeros((G, msl, Hk), np.float16)
+        oracle.turbo_kv_quantize_batch(q_, n_, src, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+        want += [q_, n_]
+    bufs = [dev(np.zeros_like(w)) for w in want]
+    kv.tw_turbo_kv_append_batch(bufs[0], bufs[1], bufs[2], bufs[3], dev(k), dev(v), dev(rotation_fixture),
+                                dev(pos), msl, G, Hk, D, kv_dim, bits)
+    for b, w, name in zip(bufs, want, ("K codes", "K norms", "V codes", "V norms")):
+        assert_bytes_equal(host(b), w, "fused " + name)
+
+
+# ------------------------------------------------------------------ attention helpers
+def build_fp16_cache(r, G, msl, kv_dim):
+    return gen.normal_f16(r, (G, msl, kv_dim)), gen.normal_f16(r, (G, msl, kv_dim))
+
+
+def build_turbo_cache(oracle, rot, r, G, Hk, msl, lens, bits, outliers=True):
+    """Quantize lens[g] rows per sequence with the oracle's token-list append."""
+    kv_dim = Hk * D
+    kvp = kv_dim * bits // 8
+    ck = np.zeros((G, msl, kvp), np.uint8); cv = np.zeros_like(ck)
+    kn = np.zeros((G, msl, Hk), np.float16); vn = np.zeros_like(kn)
+    for g in range(G):
+        n = int(lens[g])
+        if outliers:
+            k_rows, _ = gen.kv_rows_with_outliers(r, (n, kv_dim), kv_dim)
+            v_rows, _ = gen.kv_rows_with_outliers(r, (n, kv_dim), kv_dim)
+        else:
+            k_rows = gen.normal_f16(r, (n, kv_dim)); v_rows = gen.normal_f16(r, (n, kv_dim))
+        p = np.arange(n, dtype=np.int32)
+        oracle.turbo_kv_quantize(ck[g], kn[g], k_rows, rot, p, msl, n, Hk, D, kv_dim, bits)
+        oracle.turbo_kv_quantize(cv[g], vn[g], v_rows, rot, p, msl, n, Hk, D, kv_dim, bits)
+    return ck, cv, kn, vn
+
+
+# ------------------------------------------------------------------ fp16 attention
+@pytest.mark.parametrize("nsplit", [0, 1, 3])
+def test_fp16_attention_batch_config1(kv, oracle, nsplit):
+    """Single layer, 16 query heads, 8 KV heads, batch 4, context 612 + the appended token."""
+    r = gen.rng(201)
+    G, H, Hk, msl = 4, 16, 8, 640
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+    q = gen.normal_f16(r, (G, q_dim))
+    pos = np.full(G, 612, np.int32)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    import torch
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.set_num_splits(nsplit)
+    try:
+        kv.launch_gqa_attention_batch(out, dev(q), dev(ck), dev(cv), scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim)
+    finally:
+        kv.set_num_splits(0)
+    assert rel_err(host(out), want) <= TOL
+
+
+def test_fp16_attention_ragged_and_strided(kv, oracle):
+    r = gen.rng(202)
+    G, H, Hk, msl = 6, 8, 2, 1500   # GQA group 4
+    kv_dim, q_dim = Hk * D, H * D + 64   # q_dim is a row stride
+    ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+    q = gen.normal_f16(r, (G, q_dim))
+    pos = np.array([0, 1, 63, 64, 777, 1499], np.int32)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    import torch
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.launch_gqa_attention_batch(out, dev(q), dev(ck), dev(cv), scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim)
+    got = host(out)
+    assert rel_err(got[:, :H * D], want[:, :H * D]) <= TOL
+    assert not got[:, H * D:].any()
+
+
+def test_fp16_attention_single_sequence(kv, oracle):
+    r = gen.rng(203)
+    H, Hk, msl = 16, 8, 700
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv = build_fp16_cache(r, 1, msl, kv_dim)
+    q = gen.normal_f16(r, (q_dim,))
+    import torch
+    for pos in (0, 129, 699):
+        want = np.zeros(q_dim, np.float16)
+        oracle.gqa_attention(q, ck[0], cv[0], want, pos, msl, H, Hk, D)
+        out = torch.zeros(q_dim, dtype=torch.float16, device="cuda")
+        scratch = torch.zeros(H * msl, dtype=torch.float32, device="cuda")
+        kv.launch_gqa_attention(dev(q), dev(ck[0]), dev(cv[0]), out, scratch, pos, msl, H, Hk, D)
+        assert rel_err(host(out), want) <= TOL
+
+
+def test_fp16_prefill_attention(kv, oracle):
+    r = gen.rng(204)
+    T, H, Hk, msl = 70, 4, 2, 96
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv = build_fp16_cache(r, 1, msl, kv_dim)
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    oracle.gqa_prefill_attention(want, q, ck[0], cv[0], T, msl, H, Hk, D, q_dim, kv_dim)
+    import torch
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * T, dtype=torch.float32, device="cuda")
+    kv.launch_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), scratch, T, msl, H, Hk, D, q_dim, kv_dim)
+    assert rel_err(host(out), want) <= TOL
+
+
+# ------------------------------------------------------------------ compressed attention
+@pytest.mark.parametrize("variant", [1, 0])
+@pytest.mark.parametrize("bits", [4, 2])
+def test_turbo_attention_batch_config2_layer(kv, oracle, rotation_fixture, bits, variant):
+    """One layer of the 28-layer TurboQuant case: batch 4, context 612 + 1, 1 % outlier channels x8."""
+    r = gen.rng(300 + bits)
+    G, H, Hk, msl = 4, 16, 8, 640
+    kv_dim, q_dim = Hk * D, H * D
+    lens = [613] * G
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits)
+    q = gen.normal_f16(r, (G, q_dim))
+    pos = np.array(lens, np.int32) - 1
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    import torch
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.set_attention_variant(variant)
+    try:
+        kv.launch_turbo_gqa_attention_batch(out, dev(q), dev(ck), dev(cv), dev(kn), dev(vn), dev(rotation_fixture),
+                                            scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    finally:
+        kv.set_attention_variant(0)
+    assert rel_err(host(out), want) <= TOL
+
+
+@pytest.mark.parametrize("variant", [1, 0])
+@pytest.mark.parametrize("bits,H,Hk", [(4, 16, 8), (2, 32, 8), (4, 4, 4)])
+def test_turbo_attention_ragged_splits(kv, oracle, rotation_fixture, bits, H, Hk, variant):
+    """Ragged contexts around every tile / chunk edge, with forced split counts."""
+    r = gen.rng(310 + bits + H)
+    lens = [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 257, 1000, 1535, 1536]
+    G, msl = len(lens), 1536
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits, outliers=False)
+    q = gen.normal_f16(r, (G, q_dim))
+    pos = np.array(lens, np.int32) - 1
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    import torch
+    d = [dev(x) for x in (q, ck, cv, kn, vn, rotation_fixture, pos)]
+    kv.set_attention_variant(variant)
+    try:
+        for nsplit in (0, 1, 2, 7):
+            kv.set_num_splits(nsplit)
+            out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+            scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+            kv.launch_turbo_gqa_attention_batch(out, d[0], d[1], d[2], d[3], d[4], d[5], scratch, d[6], msl, G, H, Hk,
+                                                D, q_dim, kv_dim, bits)
+            err = rel_err(host(out), want)
+            assert err <= TOL, f"nsplit={nsplit}: {err}"
+    finally:
+        kv.set_num_splits(0)
+        kv.set_attention_variant(0)
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_turbo_attention_single_and_tiny_scratch(kv, oracle, rotation_fixture, bits):
+    """Single-sequence entry point; max_seq_len 40 leaves no room for split partials."""
+    r = gen.rng(320 + bits)
+    H, Hk, msl = 4, 2, 40
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, 1, Hk, msl, [37], bits)
+    q = gen.normal_f16(r, (q_dim,))
+    import torch
+    for pos in (0, 36):
+        want = np.zeros(q_dim, np.float16)
+        oracle.turbo_gqa_attention(q, ck[0], cv[0], kn[0], vn[0], rotation_fixture, want, pos, msl, H, Hk, D, bits)
+        out = torch.zeros(q_dim, dtype=torch.float16, device="cuda")
+        scratch = torch.zeros(H * msl, dtype=torch.float32, device="cuda")
+        kv.launch_turbo_gqa_attention(dev(q), dev(ck[0]), dev(cv[0]), dev(kn[0]), dev(vn[0]), dev(rotation_fixture),
+                                      out, scratch, pos, msl, H, Hk, D, bits)
+        assert rel_err(host(out), want) <= TOL
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_turbo_prefill_attention(kv, oracle, rotation_fixture, bits):
+    r = gen.rng(330 + bits)
+    T, H, Hk, msl = 70, 4, 2, 96
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, 1, Hk, msl, [T], bits)
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    oracle.turbo_gqa_prefill_attention(want, q, ck[0], cv[0], kn[0], vn[0], rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+    import torch
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * T, dtype=torch.float32, device="cuda")
+    kv.launch_turbo_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), dev(kn[0]), dev(vn[0]),
+                                          dev(rotation_fixture), scratch, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+    assert rel_err(host(out), want) <= TOL
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_golden_case_on_gpu(kv, rotation_fixture, bits):
+    """Committed vectors: append 37 tokens on the GPU, compare every byte, then attention."""
+    z = np.load(Path(__file__).parent / "golden" / f"case_tq{bits}_g2_h4_ctx37.npz")
+    G, H, Hk, ctx, msl = (int(z[k]) for k in ("G", "H", "Hk", "ctx", "msl"))
+    kv_dim, q_dim = Hk * D, H * D
+    import torch
+    bufs = [dev(np.zeros_like(z[k])) for k in ("ck", "kn", "cv", "vn")]
+    pos = torch.zeros(G, dtype=torch.int32, device="cuda")
+    rot = dev(rotation_fixture)
+    for t in range(ctx + 1):
+        kv.tw_turbo_kv_append_batch(bufs[0], bufs[1], bufs[2], bufs[3], dev(z["k_rows"][t]), dev(z["v_rows"][t]), rot,
+                                    pos, msl, G, Hk, D, kv_dim, bits)
+        if t < ctx:
+            kv.launch_increment_positions(pos, G)
+    for b, k in zip(bufs, ("ck", "kn", "cv", "vn")):
+        assert_bytes_equal(host(b), z[k], k, z["last_margin"])
+    assert np.array_equal(host(pos), z["pos"])
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.launch_turbo_gqa_attention_batch(out, dev(z["q"]), bufs[0], bufs[2], bufs[1], bufs[3], rot, scratch, pos, msl, G,
+                                        H, Hk, D, q_dim, kv_dim, bits)
+    assert rel_err(host(out), z["out"]) <= TOL
+
+
+# ------------------------------------------------------------------ paged cache
+@pytest.mark.parametrize("bits", [4, 2, 0])
+def test_paged_cache_equals_contiguous(kv, oracle, rotation_fixture, bits):
+    """16-token pages in shuffled order: pages gathered in block-table order are the
+    contiguous oracle cache byte for byte, and attention over them is the same."""
+    import torch
+    r = gen.rng(400 + bits)
+    G, H, Hk = 5, 8, 4
+    kv_dim, q_dim = Hk * D, H * D
+    pages_per_seq = 9
+    msl = pages_per_seq * 16
+    lens = np.array([1, 16, 17, 100, 144])
+    steps = 3                                   # append 3 more tokens on the GPU per sequence
+    bt = gen.shuffled_block_table(r, G, pages_per_seq)
+    n_pages = G * pages_per_seq
+    rot = dev(rotation_fixture)
+    if bits == 0:
+        ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+        for g in range(G):
+            ck[g, lens[g] - steps:] = 0; cv[g, lens[g] - steps:] = 0
+        row_bytes = kv_dim * 2
+    else:
+        ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, np.maximum(lens - steps, 0), bits)
+        row_bytes = kv_dim * bits // 8
+
+    def scatter(contig, width, dtype):
+        pool = np.zeros((n_pages, 16, width), dtype)
+        for g in range(G):
+            for i in range(pages_per_seq):
+                pool[bt[g, i]] = contig[g, 16 * i:16 * (i + 1)]
+        return pool
+
+    def gather(pool):
+        return np.stack([np.concatenate([pool[bt[g, i]] for i in range(pages_per_seq)]) for g in range(G)])
+
+    start = np.maximum(lens - steps, 0).astype(np.int32)
+    if bits == 0:
+        p_ck, p_cv = dev(scatter(ck, kv_dim, np.float16)), dev(scatter(cv, kv_dim, np.float16))
+    else:
+        p_ck, p_cv = dev(scatter(ck, row_bytes, np.uint8)), dev(scatter(cv, row_bytes, np.uint8))
+        p_kn, p_vn = dev(scatter(kn, Hk, np.float16)), dev(scatter(vn, Hk, np.float16))
+    d_bt = dev(bt)
+    pos = start.copy()
+    for s in range(steps):
+        live = pos < lens
+        k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+        # sequences shorter than `steps` tokens stay where they are and rewrite the same row
+        wpos = np.where(live, pos, lens - 1).astype(np.int32)
+        if bits == 0:
+            oracle.kv_cache_write_batch(ck, cv, k, v, wpos, msl, G, kv_dim)
+            kv.tw_paged_kv_cache_write_batch(p_ck, p_cv, dev(k), dev(v), dev(wpos), d_bt, pages_per_seq, G, kv_dim)
+        else:
+            oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, wpos, msl, G, Hk, D, kv_dim, bits)
+            oracle.turbo_kv_quantize_batch(cv, vn, v, rotation_fixture, wpos, msl, G, Hk, D, kv_dim, bits)
+            kv.tw_paged_turbo_kv_append_batch(p_ck, p_kn, p_cv, p_vn, dev(k), dev(v), rot, dev(wpos), d_bt,
+                                              pages_per_seq, G, Hk, D, kv_dim, bits)
+        pos = np.where(live, pos + 1, pos)
+    assert_bytes_equal(gather(host(p_ck)), ck, "paged K")
+    assert_bytes_equal(gather(host(p_cv)), cv, "paged V")
+    if bits:
+        assert_bytes_equal(gather(host(p_kn)), kn, "paged K norms")
+        assert_bytes_equal(gather(host(p_vn)), vn, "paged V norms")
+
+    apos = (lens - 1).astype(np.int32)
+    q = gen.normal_f16(r, (G, q_dim))
+    want = np.zeros((G, q_dim), np.float16)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    ws = torch.zeros(kv.attention_workspace_floats(G, H, msl), dtype=torch.float32, device="cuda")
+    if bits == 0:
+        oracle.gqa_attention_batch(want, q, ck, cv, apos, msl, G, H, Hk, D, q_dim, kv_dim)
+        kv.tw_paged_gqa_attention_batch(out, dev(q), p_ck, p_cv, ws, dev(apos), d_bt, pages_per_seq, msl, G, H, Hk, D,
+                                        q_dim, kv_dim)
+    else:
+        oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, apos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+        kv.tw_paged_turbo_gqa_attention_batch(out, dev(q), p_ck, p_cv, p_kn, p_vn, rot, ws, dev(apos), d_bt,
+                                              pages_per_seq, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    assert rel_err(host(out), want) <= TOL
+
+
+# ------------------------------------------------------------------ engine: append -> attention -> positions, eager and graph
+@pytest.mark.parametrize("kv_bits", [0, 4, 2])
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_engine_decode_steps(oracle, kv_bits, use_graph):
+    import torch
+    from triebwerk_amd import Engine
+    r = gen.rng(500 + kv_bits)
+    L, H, Hk, G, msl, steps = 3, 16, 8, 5, 48, 6
+    kv_dim, q_dim = Hk * D, H * D
+    eng = Engine(max_seq_len=1024, kv_bits=kv_bits)
+    assert eng.kv_bits() == kv_bits
+    eng.set_shape(L, H, Hk, D)
+    eng.alloc_batch(G, msl)
+    start = np.array([0, 3, 10, 31, 41], np.int32)
+    eng.set_positions(start)
+    rot = None
+    if kv_bits:
+        rot = host(eng.rotation())
+        assert np.array_equal(rot.view(np.uint16), oracle.make_rotation(128, 42)[0].view(np.uint16))
+    # oracle-side caches
+    if kv_bits == 0:
+        o_k = [np.zeros((G, msl, kv_dim), np.float16) for _ in range(L)]
+        o_v = [np.zeros((G, msl, kv_dim), np.float16) for _ in range(L)]
+    else:
+        kvp = kv_dim * kv_bits // 8
+        o_k = [np.zeros((G, msl, kvp), np.uint8) for _ in range(L)]; o_v = [np.zeros((G, msl, kvp), np.uint8) for _ in range(L)]
+        o_kn = [np.zeros((G, msl, Hk), np.float16) for _ in range(L)]; o_vn = [np.zeros((G, msl, Hk), np.float16) for _ in range(L)]
+    pos = start.copy()
+    # the graph replays fixed buffers: inputs are copied into them before every step
+    d_q = torch.zeros((L, G, q_dim), dtype=torch.float16, device="cuda")
+    d_k = torch.zeros((L, G, kv_dim), dtype=torch.float16, device="cuda")
+    d_v = torch.zeros((L, G, kv_dim), dtype=torch.float16, device="cuda")
+    d_out = torch.zeros((L, G, q_dim), dtype=torch.float16, device="cuda")
+    stream = torch.cuda.Stream()
+    for step in range(steps):
+        q = gen.normal_f16(r, (L, G, q_dim)); k = gen.normal_f16(r, (L, G, kv_dim)); v = gen.normal_f16(r, (L, G, kv_dim))
+        d_q.copy_(dev(q)); d_k.copy_(dev(k)); d_v.copy_(dev(v))
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            eng.decode_step(d_q, d_k, d_v, d_out, use_graph=use_graph, stream=stream)
+        stream.synchronize()
+        got = host(d_out)
+        for l in range(L):
+            want = np.zeros((G, q_dim), np.float16)
+            if kv_bits == 0:
+                oracle.kv_cache_write_batch(o_k[l], o_v[l], k[l], v[l], pos, msl, G, kv_dim)
+                oracle.gqa_attention_batch(want, q[l], o_k[l], o_v[l], pos, msl, G, H, Hk, D, q_dim, kv_dim)
+            else:
+                oracle.turbo_kv_quantize_batch(o_k[l], o_kn[l], k[l], rot, pos, msl, G, Hk, D, kv_dim, kv_bits)
+                oracle.turbo_kv_quantize_batch(o_v[l], o_vn[l], v[l], rot, pos, msl, G, Hk, D, kv_dim, kv_bits)
+                oracle.turbo_gqa_attention_batch(want, q[l], o_k[l], o_v[l], o_kn[l], o_vn[l], rot, pos, msl, G, H, Hk, D,
+                                                 q_dim, kv_dim, kv_bits)
+            err = rel_err(got[l], want)
+            assert err <= TOL, f"step {step} layer {l}: {err}"
+        oracle.increment_positions(pos, G)
+        assert np.array_equal(host(eng.positions()), pos)
+    for l in range(L):
+        c = eng.cache(l)
+        assert_bytes_equal(host(c[0]), o_k[l], f"layer {l} K cache")
+        assert_bytes_equal(host(c[1]), o_v[l], f"layer {l} V cache")
+        if kv_bits:
+            assert_bytes_equal(host(c[2]), o_kn[l], f"layer {l} K norms")
+            assert_bytes_equal(host(c[3]), o_vn[l], f"layer {l} V norms")
+    eng.reset()
+    assert not host(eng.cache(0)[0]).any() and not host(eng.positions()).any()
+
+
+def test_engine_prefix_broadcast(oracle):
+    import torch
+    from triebwerk_amd import Engine
+    r = gen.rng(600)
+    L, H, Hk, G, msl, T = 2, 4, 2, 4, 32, 7
+    kv_dim = Hk * D
+    eng = Engine(kv_bits=4)
+    eng.set_shape(L, H, Hk, D)
+    eng.alloc_batch(G, msl)
+    rot = eng.rotation()
+    rows = gen.normal_f16(r, (T, kv_dim))
+    c = eng.cache(0)
+    from triebwerk_amd import kvcache
+    positions = torch.arange(T, dtype=torch.int32, device="cuda")
+    kvcache.launch_turbo_kv_quantize(c[0][0], c[2][0], dev(rows), rot, positions, msl, T, Hk, D, kv_dim, 4)
+    eng.broadcast_prefix(0, 1, G, T)
+    k = host(c[0]); n = host(c[2])
+    for g in range(1, G):
+        assert np.array_equal(k[g, :T], k[0, :T]) and np.array_equal(n[g, :T], n[0, :T])
+        assert not k[g, T:].any()

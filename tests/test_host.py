@@ -1,0 +1,94 @@
+"""CPU-only checks of the host side: the C ABI library loads and exports every
+symbol the header declares, and the engine's host logic (kv_bits switch, cache
+sizing, rotation matrix) behaves like the reference's.  No kernel is launched."""
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "triebwerk_kv.h"
+
+
+def declared_functions():
+    text = HEADER.read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b((?:launch|tw)_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_declares_the_reference_launchers():
+    names = declared_functions()
+    for fn in ("launch_kv_cache_write_batch", "launch_turbo_kv_quantize", "launch_turbo_kv_quantize_batch",
+               "launch_gqa_attention", "launch_gqa_attention_batch", "launch_turbo_gqa_attention",
+               "launch_turbo_gqa_attention_batch", "launch_gqa_prefill_attention",
+               "launch_turbo_gqa_prefill_attention", "launch_increment_positions"):
+        assert fn in names
+
+
+def test_library_exports_every_declared_symbol():
+    from triebwerk_amd import _lib
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    missing = [n for n in declared_functions() if not hasattr(lib, n)]
+    assert not missing, missing
+    # and the Python binding table covers the same set
+    assert sorted(_lib.SIGNATURES) == declared_functions()
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from triebwerk_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(_lib.LibraryMissing):
+        _lib.load()
+
+
+def test_engine_kv_bits_switch(capfd):
+    """engine.cpp:300-317: 0, 2, 4 are kept; anything else warns and falls back to fp16."""
+    from triebwerk_amd import Engine
+    assert Engine().kv_bits() == 0 and Engine().max_seq_len() == 1024  # engine_py.cpp:22 defaults
+    assert Engine(512, 2).kv_bits() == 2
+    assert Engine(max_seq_len=64, kv_bits=4).kv_bits() == 4
+    capfd.readouterr()
+    assert Engine(64, 3).kv_bits() == 0
+    assert "kv_bits=3 not supported" in capfd.readouterr().err
+    assert Engine(64, 8).kv_bits() == 0
+
+
+def test_cache_sizes_match_the_reference_readme():
+    """README.md:163-168: G=4, 28 layers: 1,024 tokens fp16 448 MiB -> TQ4 ~116 MiB;
+    8,192 tokens TQ4 ~1,005 MiB (1056 bytes per token per layer)."""
+    from triebwerk_amd import _lib
+    lib = _lib.load()
+
+    def cache_bytes(bits, G, msl):
+        e = lib.tw_engine_create(1024, bits)
+        total = lib.tw_engine_arena_bytes_needed(e, G, msl)
+        lib.tw_engine_destroy(e)
+        scratch = G * 16 * msl * 4
+        return total - scratch
+
+    mib = 1024 * 1024
+    assert abs(cache_bytes(0, 4, 1024) / mib - 448) < 0.1
+    assert abs(cache_bytes(4, 4, 1024) / mib - 115.5) < 0.1
+    assert abs(cache_bytes(4, 4, 8192) / mib - 924) < 0.1      # 4*8192*28*1056 B
+    assert abs(cache_bytes(2, 4, 1024) / mib - 59.5) < 0.1     # 544 B per token per layer
+
+
+def test_set_shape_rejects_what_the_kernels_cannot_run():
+    from triebwerk_amd import Engine
+    e = Engine(64, 4)
+    e.set_shape(36, 32, 8, 128)
+    with pytest.raises(ValueError):
+        e.set_shape(2, 16, 8, 64)
+    with pytest.raises(ValueError):
+        e.set_shape(2, 15, 8, 128)
+
+
+def test_host_rotation_is_the_fixture(rotation_fixture):
+    """The matrix the library builds on the host (engine.cpp:366-392) is the committed one."""
+    from triebwerk_amd import kvcache
+    r = kvcache.make_rotation(128, 42).numpy()
+    assert np.array_equal(r.view(np.uint16), rotation_fixture.view(np.uint16))
