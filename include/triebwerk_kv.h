@@ -131,6 +131,14 @@ int tw_kv_get_attention_variant(void);
 /* Split count override for decode attention (0 = automatic). */
 void tw_kv_set_num_splits(int nsplit);
 
+/* Timing of the context-scanning attention kernel alone, with HIP events
+ * recorded on the launch stream around that kernel (not around the merge).
+ * Enable, run eager launches (not under stream capture; at most 4096 are
+ * kept), then read the summed duration and the launch count.  Reading waits
+ * for the recorded launches and resets the counter.  Not thread-safe. */
+void tw_kv_profile_attention(int enable);
+int tw_kv_profile_read(double* total_ms, int* launches);
+
 /* Floats of workspace the *_ws / paged attention entry points need for a
  * (G, num_heads, max_context) problem at the automatic split count.  The
  * reference-signature launchers instead fit their split count to the

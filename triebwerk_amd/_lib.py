@@ -41,6 +41,8 @@ SIGNATURES = {
     "tw_kv_set_attention_variant": (None, [I]),
     "tw_kv_get_attention_variant": (I, []),
     "tw_kv_set_num_splits": (None, [I]),
+    "tw_kv_profile_attention": (None, [I]),
+    "tw_kv_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_attention_workspace_floats": (SZ, [I, I, I]),
     "tw_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_paged_kv_cache_write_batch": (None, [P, P, P, P, P, P, I, I, I, P]),

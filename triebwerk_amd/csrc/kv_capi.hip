@@ -89,11 +89,32 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     a.ws_stride = ws_floats_per_head;
 }
 
+// Optional timing of the dominant (context-scanning) kernel with HIP events on
+// the launch stream; off by default, never active under stream capture.
+constexpr int kProfSlots = 4096;
+struct Profiler {
+    std::atomic<int> enabled{0};
+    hipEvent_t start[kProfSlots];
+    hipEvent_t stop[kProfSlots];
+    int created = 0;
+    int used = 0;
+} g_prof;
+
 void run_attention(AttnArgs& a, hipStream_t s, const char* fn) {
+    bool prof = g_prof.enabled.load() != 0 && g_prof.used < kProfSlots;
+    if (prof) {
+        while (g_prof.created <= g_prof.used) {
+            if (hipEventCreate(&g_prof.start[g_prof.created]) != hipSuccess ||
+                hipEventCreate(&g_prof.stop[g_prof.created]) != hipSuccess) { prof = false; break; }
+            g_prof.created++;
+        }
+    }
+    if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
     bool done = false;
     int variant = g_variant.load();
     if (a.bits != 0 && variant != 1) done = launch_attention_mfma(a, s);
     if (!done) launch_attention_valu(a, s);
+    if (prof) hipEventRecord(g_prof.stop[g_prof.used++], s);
     launch_attention_merge(a, s);
     check_launch(fn);
 }
@@ -108,6 +129,25 @@ const char* tw_kv_build_info(void) { return "triebwerk_kv gfx950 " __DATE__ " " 
 void tw_kv_set_attention_variant(int v) { g_variant.store(v); }
 int tw_kv_get_attention_variant(void) { return g_variant.load(); }
 void tw_kv_set_num_splits(int n) { g_nsplit_override.store(n); }
+
+void tw_kv_profile_attention(int enable) {
+    g_prof.enabled.store(enable);
+    if (enable) g_prof.used = 0;
+}
+
+int tw_kv_profile_read(double* total_ms, int* launches) {
+    double sum = 0.0;
+    for (int i = 0; i < g_prof.used; i++) {
+        if (hipEventSynchronize(g_prof.stop[i]) != hipSuccess) return -1;
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, g_prof.start[i], g_prof.stop[i]) != hipSuccess) return -1;
+        sum += ms;
+    }
+    if (total_ms) *total_ms = sum;
+    if (launches) *launches = g_prof.used;
+    g_prof.used = 0;
+    return 0;
+}
 
 size_t tw_attention_workspace_floats(int G, int num_heads, int max_context) {
     (void)max_context;
