@@ -1,12 +1,409 @@
-// kv_attention_mfma.hip -- MFMA decode attention over the compressed cache.
+// kv_attention_mfma.hip -- GQA decode attention over the 4-bit compressed cache
+// for gfx950: codes are expanded to fp16 centroids in registers and the two
+// contractions (q.K^T and P.V) run on the matrix cores.
+//
+// Same mathematics as turbo_gqa_attention_batch_kernel of the reference
+// (kernels.cu:1641-1776): q_rot = R q; s_p = (q_rot . c(K codes_p)) * kn_p / sqrt(D);
+// softmax over p <= pos with "+1e-8" in the denominator; acc = sum_p w_p vn_p c(V codes_p);
+// out = R^T acc.  Three launches: query_rotate_kernel (q_rot, once per sequence and
+// head), attention_mfma4_kernel (the context scan, below), attention_merge_kernel
+// (split merge, normalisation, rotate-back).
+//
+// Why MFMA for a bandwidth-bound scan: at 5.6 TB/s of 4-bit codes one CU must
+// consume ~18 codes per clock for K and V together, and with two query heads per
+// KV head that is ~4 vector-ALU operations per code (extract, look up, two FMAs)
+// against a budget of 64 lane-operations per clock per CU.  Moving the FMAs to
+// MFMA leaves one v_perm_b32 (LDS address) and one ds_read_b32 per BYTE of codes.
+//
+// Mapping (one wave = one KV head of one sequence, 32 tokens per iteration):
+//   K: lane (t = lane%16, kg = lane/16) loads 16 bytes = dims [32kg, 32kg+32) of
+//      token t.  Dword j of it is the A operand of MFMA j (v_mfma_f32_16x16x32_f16),
+//      rows = tokens; the B operand holds q_rot for the GQA group's heads in the
+//      matching dimension order, columns = heads.  Result S^T[token][head].
+//   softmax: online, per head, in base 2 (q_rot is pre-scaled by log2(e)/sqrt(D));
+//      S^T's register layout (lane: head = lane%16, tokens 4*(lane/16)+r) is exactly
+//      the A-operand layout P[head][token] of the second contraction, so
+//      probabilities never leave registers.
+//   V: lane (n = lane%16, kg = lane/16) loads, for tokens 4kg..4kg+3, the dword
+//      that holds dims 8n..8n+7.  Nibbles of two tokens are interleaved with
+//      v_bfi_b32 so that one table look-up yields the fp16 pair (token, token+1) for
+//      one dim, which is the B-operand order of O[head][dim] += P[head][token] V[token][dim].
+//   dequantization: a 256-entry table byte -> (centroid[lo nibble], centroid[hi nibble])
+//      as packed fp16, replicated per lane in LDS (64 KB) so that every ds_read_b32 of
+//      a wave is bank-conflict free; the address is one v_perm_b32.
+//   addressing: every load is (scalar base of the 16-token sub-tile) + (per-lane
+//      offset fixed for the whole kernel); pages of the paged layout only change
+//      the scalar base.
+//   scheduling: workgroups are persistent (two per CU) and walk a list of
+//      (sequence, chunk, head group) items, so the 64 KB table is built once per
+//      workgroup; waves never synchronise after that.
+//   precision: fp16 operands would cost ~5e-4 relative error each for q_rot and for
+//      the probabilities.  Both are split into hi + lo fp16 parts that ride in MFMA
+//      rows/columns the GQA group leaves empty (head n -> column n and n+8), so the
+//      split costs no extra MFMA; the two halves are added after the contraction.
+//      The centroid table is stored as fp16(alpha * c) with alpha chosen so that all
+//      eight magnitudes round with <= 1.1e-4 relative error (3.6e-4 without it);
+//      1/alpha is folded into q_rot and into the final accumulator.
+// The partial (acc[128], max, sum) per (sequence, head, chunk) goes to the split
+// workspace; attention_merge_kernel combines, normalises and rotates back.
+
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 
 namespace twkv {
 
-bool launch_attention_mfma(const AttnArgs& a, hipStream_t s) {
-    (void)a; (void)s;
-    return false;
+namespace {
+
+constexpr int kMaxWaves = 8;          // KV heads per workgroup
+constexpr int kMaxGroup = 4;          // query heads per KV head handled by this kernel
+constexpr int kTableWords = 256 * 64; // 64 KB
+constexpr float kNegBig = -1e30f;
+// fp16(kAlpha4 * c) has max relative rounding error 1.05e-4 over the 4-bit table
+// (exhaustive search over the fp32 values of one octave).
+constexpr float kAlpha4 = 19.391284942626953f;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kInvSqrtD = 0.08838834764831845f;
+
+__device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
+    if (a.pos_mode == kPosArray) return a.positions[g];
+    if (a.pos_mode == kPosScalar) return a.pos_scalar;
+    return g;
+}
+
+struct TileRegs {
+    uint4 k[2];          // K codes: sub-tile a, b (16 tokens each)
+    uint32_t v[2][4];    // V codes: 4 tokens per sub-tile, 8 dims each
+    uint32_t kn[2];      // fp16 bits of kn of token (lane % 16) of each sub-tile
+    uint32_t vn[2];
+};
+
+// value of the lane 8 places away inside the row of 16 lanes (DPP row_ror:8)
+__device__ __forceinline__ float dpp_ror8(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ float h2f_bits(uint32_t bits16) {
+    union { uint16_t u; half_t h; } cv;
+    cv.u = (uint16_t)bits16;
+    return (float)cv.h;
+}
+
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+typedef uint32_t uint32x4_t __attribute__((ext_vector_type(4)));
+
+// Buffer descriptor over [base, base + bytes).  Every input is forced into scalar
+// registers: a descriptor held in vector registers makes each load a serialising loop.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const char* base, int bytes) {
+    uint64_t p = reinterpret_cast<uint64_t>(base);
+    uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32));
+    char* q = reinterpret_cast<char*>(((uint64_t)hi << 32) | lo);
+    return __builtin_amdgcn_make_buffer_rsrc(q, 0, __builtin_amdgcn_readfirstlane(bytes), 0x00020000);
+}
+
+}  // namespace
+
+// q_rot[g][head][d] = (sum_k R[d][k] q[g][head][k]) * log2(e) / (sqrt(D) * alpha)
+// (kernels.cu:1671-1681, with the score scale of line 1707 and the table scale
+// folded in).  One workgroup of 128 threads per (sequence, head); fp32, k ascending.
+__global__ void __launch_bounds__(kHeadDim)
+query_rotate_kernel(AttnArgs a) {
+    __shared__ float q_s[kHeadDim];
+    const int head = blockIdx.x, g = blockIdx.y, d = threadIdx.x;
+    q_s[d] = (float)a.q[(long long)g * a.q_stride + (long long)head * kHeadDim + d];
+    __syncthreads();
+    const half8_t* rot8 = reinterpret_cast<const half8_t*>(a.rotation + d * kHeadDim);
+    float acc = 0.0f;
+#pragma unroll 4
+    for (int k8 = 0; k8 < kHeadDim / 8; k8++) {
+        half8_t rr = rot8[k8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc = __builtin_fmaf((float)rr[i], q_s[8 * k8 + i], acc);
+    }
+    a.qrot[((long long)g * a.num_heads + head) * a.ws_stride + d] = acc * (kLog2e * kInvSqrtD / kAlpha4);
+}
+
+__global__ void __launch_bounds__(kMaxWaves * kWave, 4)
+attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
+    __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
+
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int wave = uniform(tid / kWave), lane = tid % kWave;   // wave index is wave-uniform: keep it scalar
+    const int ln = lane & 15, kg = lane >> 4;
+    const int waves = nthreads / kWave;
+    const int R = a.num_heads / a.num_kv_heads;
+    const int Hk = a.num_kv_heads;
+
+    // ---- dequantization table, once per workgroup: entry e, 64 identical words
+    for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
+        int e = i >> 6;
+        half2_t p = {(half_t)(kAlpha4 * kCentroids4[e & 15]), (half_t)(kAlpha4 * kCentroids4[e >> 4])};
+        uint32_t w = *reinterpret_cast<uint32_t*>(&p);
+        *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
+    }
+    __syncthreads();
+
+    const char* tab_lane = reinterpret_cast<const char*>(tab_s);
+    const uint32_t lane4 = (uint32_t)lane * 4u;
+    const uint32_t kvp = (uint32_t)Hk * 64u;           // bytes per cache row (all heads)
+    const uint32_t nrow = (uint32_t)Hk * 2u;           // bytes per norm row
+    // per-lane offsets inside a 16-token sub-tile, fixed for the whole kernel
+    const uint32_t koff = (uint32_t)ln * kvp + 16u * (uint32_t)kg;
+    const uint32_t noff = (uint32_t)ln * nrow;
+    uint32_t voff[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(4 * kg + i) * kvp + 4u * (uint32_t)ln;
+
+    for (int item = blockIdx.x; item < total_items; item += gridDim.x) {
+        const int hg = item % hgroups;
+        const int chunk = (item / hgroups) % a.nsplit;
+        const int g = item / (hgroups * a.nsplit);
+        const int h = hg * waves + wave;                      // KV head of this wave
+        const int n = uniform(seq_pos(a, g)) + 1;
+        const int t0 = chunk * a.chunk_len;
+        if (t0 >= n) continue;                                // uniform
+        const int t1 = min(n, t0 + a.chunk_len);
+
+        // B operand of the score MFMAs: q_rot[head][32kg + 8j + i]; column n carries the
+        // fp16 value of head n, column n + 8 what the rounding left over.
+        half8_t bq[4];
+        {
+            const int hq = ln & 7;
+            const bool lo_part = (ln & 8) != 0;
+            const float* qr = a.qrot + ((long long)g * a.num_heads + (long long)h * R + (hq < R ? hq : 0)) * a.ws_stride + 32 * kg;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
+                float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
+                float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float x = (hq < R) ? v[i] : 0.0f;
+                    half_t hi = (half_t)x;
+                    half_t lo = (half_t)(x - (float)hi);
+                    bq[j][i] = lo_part ? lo : hi;
+                }
+            }
+        }
+
+        // scalar bases of this wave's head
+        const char* kseq = reinterpret_cast<const char*>(a.k) + (long long)h * 64;
+        const char* vseq = reinterpret_cast<const char*>(a.v) + (long long)h * 64;
+        const char* knseq = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
+        const char* vnseq = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
+        const int* bt = a.block_table ? a.block_table + (long long)g * a.bt_stride : nullptr;
+        const long long seq_row0 = (long long)g * a.seq_stride_rows;
+
+        // Loads of one 32-token tile.  Each 16-token sub-tile gets buffer descriptors whose
+        // base is the sub-tile's first cache row (a scalar) and whose extent is the rows that
+        // exist, so lanes past the end of the sequence read zeros instead of foreign memory.
+        auto issue = [&](TileRegs& L, int tile_start) {
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                const int ts = tile_start + 16 * sub;
+                long long row;
+                int rows;
+                if (bt) {   // a page always holds 16 rows; past the end re-read the last page (masked)
+                    row = (long long)uniform(bt[min(ts, t1 - 1) >> 4]) * kPageTokens;
+                    rows = kPageTokens;
+                } else {
+                    row = seq_row0 + ts;
+                    rows = max(min(n - ts, 16), 0);
+                }
+                __amdgpu_buffer_rsrc_t rk = make_rsrc(kseq + row * kvp, rows * (int)kvp);
+                __amdgpu_buffer_rsrc_t rv = make_rsrc(vseq + row * kvp, rows * (int)kvp);
+                __amdgpu_buffer_rsrc_t rkn = make_rsrc(knseq + row * nrow, rows * (int)nrow);
+                __amdgpu_buffer_rsrc_t rvn = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
+                uint32x4_t kq = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff, 0, 0);
+                L.k[sub] = uint4{kq[0], kq[1], kq[2], kq[3]};
+                L.kn[sub] = __builtin_amdgcn_raw_buffer_load_b16(rkn, (int)noff, 0, 0);
+                L.vn[sub] = __builtin_amdgcn_raw_buffer_load_b16(rvn, (int)noff, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; i++) L.v[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)voff[i], 0, 0);
+            }
+        };
+
+        float4_t o[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        float m_run = kNegBig, l_run = 0.0f;
+
+        // one 32-token tile: scores, online softmax, weighted V sum
+        auto compute = [&](const TileRegs& cur, int tile, bool masked) {
+            // ---- scores: S^T[token][head] for both sub-tiles
+            float4_t s[2];
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+                const uint32_t w[4] = {cur.k[sub].x, cur.k[sub].y, cur.k[sub].z, cur.k[sub].w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    union { uint32_t u[4]; half8_t h; } av;
+                    av.u[0] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
+                    av.u[1] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
+                    av.u[2] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
+                    av.u[3] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
+                    s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av.h, bq[j], s[sub], 0, 0, 0);
+                }
+            }
+            // ---- online softmax (base 2) for head ln over the 8 tokens this lane holds
+            float sv[8], vnv[8];
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float knr = h2f_bits((uint32_t)__shfl((int)cur.kn[sub], 4 * kg + r, 64));
+                    vnv[4 * sub + r] = h2f_bits((uint32_t)__shfl((int)cur.vn[sub], 4 * kg + r, 64));
+                    float sc = s[sub][r] + dpp_ror8(s[sub][r]);         // hi + lo parts of q_rot
+                    sv[4 * sub + r] = sc * knr;                         // kernels.cu:1707
+                }
+            }
+            if (masked) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    int t = tile + 16 * (i >> 2) + 4 * kg + (i & 3);
+                    sv[i] = (t < t1) ? sv[i] : kNegBig;
+                }
+            }
+            float mt = sv[0];
+#pragma unroll
+            for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
+            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m_run, mt);
+            if (__any(m_new > m_run)) {                                 // rare after the first tiles
+                float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+                m_run = m_new;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float ar = __shfl(alpha, 4 * kg + r, 64);           // O rows are heads 4kg + r
+#pragma unroll
+                    for (int j = 0; j < 8; j++) o[j][r] *= ar;
+                }
+            }
+            union { half_t e[8]; uint32_t u[4]; half8_t h; } pv, plo;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float p = __builtin_amdgcn_exp2f(sv[i] - m_run);
+                l_run += p;
+                float pf = p * vnv[i];                                  // (s * vn) * centroid, kernels.cu:1765
+                half_t hi = (half_t)pf;
+                pv.e[i] = hi;
+                plo.e[i] = (half_t)(pf - (float)hi);
+            }
+            // rows 8..15 of P carry the rounding remainder of rows 0..7
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                uint32_t moved = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)plo.u[q4], 0x128, 0xf, 0xf, false);
+                pv.u[q4] = (ln & 8) ? moved : pv.u[q4];
+            }
+            // ---- O[head][dim 8ln + j] += P[head][token] V[token][dim]
+            uint32_t xe[4], xo[4];   // [2*sub + pair]: index bytes for even / odd dims
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                for (int pr = 0; pr < 2; pr++) {
+                    uint32_t wa = cur.v[sub][2 * pr], wb = cur.v[sub][2 * pr + 1];
+                    xe[2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                    xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t sel = 0x0c0c0400u + ((uint32_t)(j >> 1) << 8);
+                union { uint32_t u[4]; half8_t h; } bv;
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    uint32_t x = (j & 1) ? xo[q4] : xe[q4];
+                    bv.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(x, lane4, sel));
+                }
+                o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv.h, bv.h, o[j], 0, 0, 0);
+            }
+        };
+
+        // loads run one tile ahead of the arithmetic
+        const int ntiles = (t1 - t0 + 31) >> 5;
+        TileRegs cur, nxt;
+        issue(cur, t0);
+        for (int it = 0; it < ntiles; it++) {
+            const int tile = t0 + 32 * it;
+            if (it + 1 < ntiles) issue(nxt, tile + 32);
+            compute(cur, tile, tile + 32 > t1);
+            if (it + 1 < ntiles) cur = nxt;
+        }
+
+        // ---- partial result of this (sequence, KV head, chunk)
+        l_run += __shfl_xor(l_run, 16, 64);
+        l_run += __shfl_xor(l_run, 32, 64);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) o[j][r] += __shfl_xor(o[j][r], 32, 64);   // row hm + row hm+8 (lo part of P)
+        }
+        if (kg == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (r < R) {
+                    float* part = a.ws + ((long long)g * a.num_heads + (long long)h * R + r) * a.ws_stride +
+                                  (long long)chunk * kPartialFloats;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) part[8 * ln + j] = o[j][r] * (1.0f / kAlpha4);
+                }
+            }
+            if (ln < R) {
+                float* part = a.ws + ((long long)g * a.num_heads + (long long)h * R + ln) * a.ws_stride +
+                              (long long)chunk * kPartialFloats;
+                part[kHeadDim] = m_run;
+                part[kHeadDim + 1] = l_run;
+            }
+        }
+    }
+}
+
+static int resident_groups() {
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        cached = 2 * cus;   // 64 KB of LDS and <= 128 VGPRs per workgroup of 8 waves: two per CU
+    }
+    return cached;
+}
+
+static int scan_waves(const AttnArgs& a) {
+    int waves = a.num_kv_heads < kMaxWaves ? a.num_kv_heads : kMaxWaves;
+    while (a.num_kv_heads % waves != 0) waves--;
+    return waves;
+}
+
+bool prepare_attention_mfma(AttnArgs& a, hipStream_t s) {
+    const int R = a.num_heads / a.num_kv_heads;
+    if (a.bits != 4) return false;
+    if (R > kMaxGroup) return false;
+    if (a.chunk_len % 32 != 0) return false;
+    // needs the split workspace with room for q_rot behind each block's partials
+    if (!a.ws || !a.qrot) return false;
+    if ((reinterpret_cast<uintptr_t>(a.qrot) & 15u) != 0 || (a.ws_stride & 3) != 0) return false;
+    const long long items = (long long)a.G * a.nsplit * (a.num_kv_heads / scan_waves(a));
+    if (items <= 0 || items > 0x7fffffff) return false;
+    a.force_merge = 1;
+    a.m_log2 = 1;
+    hipLaunchKernelGGL(query_rotate_kernel, dim3(a.num_heads, a.G), dim3(kHeadDim), 0, s, a);
+    return true;
+}
+
+void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
+    const int waves = scan_waves(a);
+    const int hgroups = a.num_kv_heads / waves;
+    const int items = a.G * a.nsplit * hgroups;
+    int grid = resident_groups();
+    if (items < grid) grid = items;
+    hipLaunchKernelGGL(attention_mfma4_kernel, dim3(grid), dim3(waves * kWave), 0, s, a, items, hgroups);
 }
 
 }  // namespace twkv

@@ -274,7 +274,7 @@ attention_merge_kernel(AttnArgs a) {
     float lsum = 0.0f, av = 0.0f;
     for (int cidx = 0; cidx < nchunks; cidx++) {
         const float* pc = part + (long long)cidx * kPartialFloats;
-        float f = __expf(pc[kHeadDim] - mg);
+        float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
         lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);
         av = __builtin_fmaf(pc[d], f, av);
     }
@@ -302,7 +302,7 @@ void launch_attention_valu(const AttnArgs& a, hipStream_t s) {
 }
 
 void launch_attention_merge(const AttnArgs& a, hipStream_t s) {
-    if (a.G <= 0 || a.nsplit <= 1) return;
+    if (a.G <= 0 || (a.nsplit <= 1 && !a.force_merge)) return;
     hipLaunchKernelGGL(attention_merge_kernel, dim3(a.num_heads, a.G), dim3(kHeadDim), 0, s, a);
 }
 

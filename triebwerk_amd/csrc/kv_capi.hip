@@ -24,8 +24,10 @@ std::atomic<int> g_variant{0};
 std::atomic<int> g_nsplit_override{0};
 
 constexpr int kMaxSplits = 64;
+constexpr long long kPagedBlockFloats = 64 * 130 + 128 + 4;  // per (sequence, head): partials + rotated query
 constexpr int kMinChunk = 128;       // tokens
 constexpr int kTargetGroups = 2048;  // workgroups wanted per launch: 8 per CU on 256 CUs
+constexpr int kTargetItems = 1024;   // (sequence, chunk) items wanted by the persistent MFMA scan
 
 void set_error(int code, const char* fmt, ...) {
     if (g_err != 0) return;  // keep the first one
@@ -69,24 +71,43 @@ bool check_bits(const char* fn, int bits) {
 // ws_floats_per_head: room per (sequence, head) in the caller's workspace.
 void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     if (ctx_bound < 1) ctx_bound = 1;
-    const int group = a.num_heads / a.num_kv_heads;
-    const int rt = (group % 4 == 0) ? 4 : (group % 2 == 0) ? 2 : 1;
-    const long long base_groups = (long long)a.G * a.num_kv_heads * (group / rt);
+    const bool mfma = a.bits == 4 && g_variant.load() != 1 && a.num_heads / a.num_kv_heads <= 4;
+    // workgroups per split: the MFMA scan takes up to 8 KV heads per workgroup,
+    // the vector-ALU kernel one (KV head, tile of query heads) each
+    long long base_groups;
+    if (mfma) {
+        base_groups = (long long)a.G * ((a.num_kv_heads + 7) / 8);
+    } else {
+        const int group = a.num_heads / a.num_kv_heads;
+        const int rt = (group % 4 == 0) ? 4 : (group % 2 == 0) ? 2 : 1;
+        base_groups = (long long)a.G * a.num_kv_heads * (group / rt);
+    }
     int want = g_nsplit_override.load();
-    if (want <= 0) want = (int)((kTargetGroups + base_groups - 1) / base_groups);
+    if (want <= 0) want = (int)(((mfma ? kTargetItems : kTargetGroups) + base_groups - 1) / base_groups);
     int max_by_ctx = (ctx_bound + kMinChunk - 1) / kMinChunk;
-    int max_by_ws = a.ws ? (int)(ws_floats_per_head / kPartialFloats) : 1;
+    // a block holds nsplit partials, then (16-byte aligned) the rotated query
+    int max_by_ws = a.ws ? (int)((ws_floats_per_head - kHeadDim - 3) / kPartialFloats) : 0;
     int nsplit = want;
     if (nsplit > max_by_ctx) nsplit = max_by_ctx;
-    if (nsplit > max_by_ws) nsplit = max_by_ws;
     if (nsplit > kMaxSplits) nsplit = kMaxSplits;
     if (nsplit < 1) nsplit = 1;
+    bool have_ws = max_by_ws >= 1;
+    if (have_ws && nsplit > max_by_ws) nsplit = max_by_ws;
+    if (!have_ws) nsplit = 1;
     int chunk = (ctx_bound + nsplit - 1) / nsplit;
     chunk = (chunk + 63) / 64 * 64;
     nsplit = (ctx_bound + chunk - 1) / chunk;
     a.nsplit = nsplit;
     a.chunk_len = chunk;
-    a.ws_stride = ws_floats_per_head;
+    if (have_ws) {
+        long long qoff = ((long long)nsplit * kPartialFloats + 3) & ~3LL;
+        a.ws_stride = qoff + kHeadDim;
+        a.qrot = a.ws + qoff;
+    } else {
+        a.ws = nullptr;          // too small to hold anything: single pass, no workspace
+        a.ws_stride = 0;
+        a.qrot = nullptr;
+    }
 }
 
 // Optional timing of the dominant (context-scanning) kernel with HIP events on
@@ -109,11 +130,11 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn) {
             g_prof.created++;
         }
     }
+    const int variant = g_variant.load();
+    const bool mfma = a.bits != 0 && variant != 1 && prepare_attention_mfma(a, s);
     if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
-    bool done = false;
-    int variant = g_variant.load();
-    if (a.bits != 0 && variant != 1) done = launch_attention_mfma(a, s);
-    if (!done) launch_attention_valu(a, s);
+    if (mfma) launch_attention_mfma_scan(a, s);
+    else launch_attention_valu(a, s);
     if (prof) hipEventRecord(g_prof.stop[g_prof.used++], s);
     launch_attention_merge(a, s);
     check_launch(fn);
@@ -151,7 +172,7 @@ int tw_kv_profile_read(double* total_ms, int* launches) {
 
 size_t tw_attention_workspace_floats(int G, int num_heads, int max_context) {
     (void)max_context;
-    return (size_t)G * num_heads * kMaxSplits * kPartialFloats;
+    return (size_t)G * num_heads * kPagedBlockFloats;
 }
 
 // ---------------------------------------------------------------- append
@@ -370,7 +391,7 @@ void tw_paged_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half*
     fill_common(a, out, q, q_dim, ck, cv, nullptr, nullptr, nullptr, G, num_heads, num_kv_heads, 0, ws);
     a.pos_mode = kPosArray; a.positions = positions;
     a.block_table = block_table; a.bt_stride = bt_stride;
-    plan_splits(a, max_context, (long long)kMaxSplits * kPartialFloats);
+    plan_splits(a, max_context, kPagedBlockFloats);
     run_attention(a, s, "tw_paged_gqa_attention_batch");
 }
 
@@ -393,7 +414,7 @@ void tw_paged_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const ui
                 num_kv_heads, bits, ws);
     a.pos_mode = kPosArray; a.positions = positions;
     a.block_table = block_table; a.bt_stride = bt_stride;
-    plan_splits(a, max_context, (long long)kMaxSplits * kPartialFloats);
+    plan_splits(a, max_context, kPagedBlockFloats);
     run_attention(a, s, "tw_paged_turbo_gqa_attention_batch");
 }
 

@@ -53,16 +53,22 @@ struct AttnArgs {
     long long seq_stride_rows;  // msl (batch), 0 (single sequence / prefill)
     int G, num_heads, num_kv_heads;
     int bits;               // 0, 2, 4
-    float* ws;              // split workspace
-    long long ws_stride;    // floats per (g, head)
+    float* ws;              // split workspace: per (g, head) block, nsplit partials then q_rot
+    long long ws_stride;    // floats per (g, head) block
+    float* qrot;            // ws + offset of q_rot inside a block (128 floats), or NULL
     int nsplit;             // >= 1; 1 = no workspace, one workgroup walks the sequence
     int chunk_len;          // tokens per split, multiple of 64
+    int force_merge;        // the scan kernel wrote partials even though nsplit == 1
+    int m_log2;             // partial maxima are in base-2 units
 };
 
 constexpr int kPartialFloats = kHeadDim + 2;  // acc[128], running max, running sum
 
 void launch_attention_valu(const AttnArgs& a, hipStream_t s);
 void launch_attention_merge(const AttnArgs& a, hipStream_t s);
-bool launch_attention_mfma(const AttnArgs& a, hipStream_t s);  // false = shape not covered
+// MFMA path, two steps so that the scan kernel can be timed alone:
+// prepare = shape check + query rotation (false = shape not covered), then the scan.
+bool prepare_attention_mfma(AttnArgs& a, hipStream_t s);
+void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);
 
 }  // namespace twkv
