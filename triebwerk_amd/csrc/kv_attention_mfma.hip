@@ -70,12 +70,6 @@ __device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
     return g;
 }
 
-struct TileRegs {
-    uint4 k[2];          // K codes: sub-tile a, b (16 tokens each)
-    uint32_t v[2][4];    // V codes: 4 tokens per sub-tile, 8 dims each
-    uint32_t kn[2];      // fp16 bits of kn of token (lane % 16) of each sub-tile
-    uint32_t vn[2];
-};
 
 // value of the lane 8 places away inside the row of 16 lanes (DPP row_ror:8)
 __device__ __forceinline__ float dpp_ror8(float v) {
@@ -124,9 +118,11 @@ query_rotate_kernel(AttnArgs a) {
     a.qrot[((long long)g * a.num_heads + head) * a.ws_stride + d] = acc * (kLog2e * kInvSqrtD / kAlpha4);
 }
 
+template <bool PAGED>
 __global__ void __launch_bounds__(kMaxWaves * kWave, 4)
 attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
+    __shared__ __attribute__((aligned(16))) uint32_t nrm_s[kMaxWaves][32];   // per wave: kn | vn << 16 of 32 tokens
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
@@ -149,12 +145,17 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     const uint32_t lane4 = (uint32_t)lane * 4u;
     const uint32_t kvp = (uint32_t)Hk * 64u;           // bytes per cache row (all heads)
     const uint32_t nrow = (uint32_t)Hk * 2u;           // bytes per norm row
-    // per-lane offsets inside a 16-token sub-tile, fixed for the whole kernel
+    // per-lane byte offsets inside a 16-token sub-tile, fixed for the whole kernel
     const uint32_t koff = (uint32_t)ln * kvp + 16u * (uint32_t)kg;
-    const uint32_t noff = (uint32_t)ln * nrow;
     uint32_t voff[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(4 * kg + i) * kvp + 4u * (uint32_t)ln;
+    const uint32_t sub_bytes = 16u * kvp;              // sub-tile b follows sub-tile a when contiguous
+    // norms: lane (ln, kg) fetches token ln of sub-tile (kg & 1)
+    const uint32_t noff = (uint32_t)ln * nrow + (PAGED ? 0u : (uint32_t)(kg & 1) * 16u * nrow);
+    uint32_t* nrm_w = &nrm_s[wave][(kg & 1) * 16 + ln];
+    const uint4* nrm_r0 = reinterpret_cast<const uint4*>(&nrm_s[wave][4 * kg]);
+    const uint4* nrm_r1 = reinterpret_cast<const uint4*>(&nrm_s[wave][16 + 4 * kg]);
 
     for (int item = blockIdx.x; item < total_items; item += gridDim.x) {
         const int hg = item % hgroups;
@@ -193,36 +194,73 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
         const char* vseq = reinterpret_cast<const char*>(a.v) + (long long)h * 64;
         const char* knseq = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
         const char* vnseq = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
-        const int* bt = a.block_table ? a.block_table + (long long)g * a.bt_stride : nullptr;
+        const int* bt = PAGED ? a.block_table + (long long)g * a.bt_stride : nullptr;
         const long long seq_row0 = (long long)g * a.seq_stride_rows;
 
-        // Loads of one 32-token tile.  Each 16-token sub-tile gets buffer descriptors whose
-        // base is the sub-tile's first cache row (a scalar) and whose extent is the rows that
-        // exist, so lanes past the end of the sequence read zeros instead of foreign memory.
-        auto issue = [&](TileRegs& L, int tile_start) {
+        // Buffer descriptors: base = first cache row of the tile (contiguous cache) or of the
+        // 16-token page (paged cache), extent = the rows that exist, so lanes past the end
+        // of the sequence read zeros instead of foreign memory.  All scalar.
+        auto page_row = [&](int ts) -> long long {   // paged: past the end re-read the last page (masked)
+            return (long long)uniform(bt[min(ts, t1 - 1) >> 4]) * kPageTokens;
+        };
+        auto issue_k = [&](uint4 (&kreg)[2], int tile) {
+            if (PAGED) {
 #pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
-                const int ts = tile_start + 16 * sub;
-                long long row;
-                int rows;
-                if (bt) {   // a page always holds 16 rows; past the end re-read the last page (masked)
-                    row = (long long)uniform(bt[min(ts, t1 - 1) >> 4]) * kPageTokens;
-                    rows = kPageTokens;
-                } else {
-                    row = seq_row0 + ts;
-                    rows = max(min(n - ts, 16), 0);
+                for (int sub = 0; sub < 2; sub++) {
+                    __amdgpu_buffer_rsrc_t r = make_rsrc(kseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp);
+                    uint32x4_t q = __builtin_amdgcn_raw_buffer_load_b128(r, (int)koff, 0, 0);
+                    kreg[sub] = uint4{q[0], q[1], q[2], q[3]};
                 }
-                __amdgpu_buffer_rsrc_t rk = make_rsrc(kseq + row * kvp, rows * (int)kvp);
-                __amdgpu_buffer_rsrc_t rv = make_rsrc(vseq + row * kvp, rows * (int)kvp);
-                __amdgpu_buffer_rsrc_t rkn = make_rsrc(knseq + row * nrow, rows * (int)nrow);
-                __amdgpu_buffer_rsrc_t rvn = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
-                uint32x4_t kq = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff, 0, 0);
-                L.k[sub] = uint4{kq[0], kq[1], kq[2], kq[3]};
-                L.kn[sub] = __builtin_amdgcn_raw_buffer_load_b16(rkn, (int)noff, 0, 0);
-                L.vn[sub] = __builtin_amdgcn_raw_buffer_load_b16(rvn, (int)noff, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; i++) L.v[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)voff[i], 0, 0);
+            } else {
+                __amdgpu_buffer_rsrc_t r = make_rsrc(kseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
+                uint32x4_t q0 = __builtin_amdgcn_raw_buffer_load_b128(r, (int)koff, 0, 0);
+                uint32x4_t q1 = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + sub_bytes), 0, 0);
+                kreg[0] = uint4{q0[0], q0[1], q0[2], q0[3]};
+                kreg[1] = uint4{q1[0], q1[1], q1[2], q1[3]};
             }
+        };
+        auto issue_v = [&](uint32_t (&vreg)[2][4], int tile) {
+            if (PAGED) {
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+                    __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff[i], 0, 0);
+                }
+            } else {
+                __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)(voff[i] + sub * sub_bytes), 0, 0);
+                }
+            }
+        };
+        // packed norms kn | vn << 16 of token (sub = kg & 1, ln)
+        auto issue_n = [&](int tile) -> uint32_t {
+            long long row;
+            int rows;
+            if (PAGED) {
+                // both pages' rows are needed; lanes pick theirs by kg & 1
+                long long r0 = page_row(tile), r1 = page_row(tile + 16);
+                __amdgpu_buffer_rsrc_t ka = make_rsrc(knseq + r0 * nrow, kPageTokens * (int)nrow);
+                __amdgpu_buffer_rsrc_t kb = make_rsrc(knseq + r1 * nrow, kPageTokens * (int)nrow);
+                __amdgpu_buffer_rsrc_t va = make_rsrc(vnseq + r0 * nrow, kPageTokens * (int)nrow);
+                __amdgpu_buffer_rsrc_t vb = make_rsrc(vnseq + r1 * nrow, kPageTokens * (int)nrow);
+                uint32_t k0 = __builtin_amdgcn_raw_buffer_load_b16(ka, (int)noff, 0, 0);
+                uint32_t k1 = __builtin_amdgcn_raw_buffer_load_b16(kb, (int)noff, 0, 0);
+                uint32_t v0 = __builtin_amdgcn_raw_buffer_load_b16(va, (int)noff, 0, 0);
+                uint32_t v1 = __builtin_amdgcn_raw_buffer_load_b16(vb, (int)noff, 0, 0);
+                return (kg & 1) ? (k1 | (v1 << 16)) : (k0 | (v0 << 16));
+            }
+            row = seq_row0 + tile;
+            rows = max(min(n - tile, 32), 0);
+            __amdgpu_buffer_rsrc_t rk = make_rsrc(knseq + row * nrow, rows * (int)nrow);
+            __amdgpu_buffer_rsrc_t rv = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
+            uint32_t kk = __builtin_amdgcn_raw_buffer_load_b16(rk, (int)noff, 0, 0);
+            uint32_t vv = __builtin_amdgcn_raw_buffer_load_b16(rv, (int)noff, 0, 0);
+            return kk | (vv << 16);
         };
 
         float4_t o[8];
@@ -230,35 +268,55 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
         for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
         float m_run = kNegBig, l_run = 0.0f;
 
-        // one 32-token tile: scores, online softmax, weighted V sum
-        auto compute = [&](const TileRegs& cur, int tile, bool masked) {
+        // Loads are re-issued into the same registers as soon as their contents have been
+        // expanded, which leaves about two thirds of an iteration to cover their latency.
+        const int ntiles = (t1 - t0 + 31) >> 5;
+        uint4 kreg[2];
+        uint32_t vreg[2][4];
+        uint32_t nreg;
+        issue_k(kreg, t0);
+        nreg = issue_n(t0);
+        issue_v(vreg, t0);
+
+        for (int it = 0; it < ntiles; it++) {
+            const int tile = t0 + 32 * it;
+            const bool more = it + 1 < ntiles;
+            const bool masked = tile + 32 > t1;
+
+            // norms: through LDS into the layout of the scores (tokens 4kg..4kg+3 of each sub-tile)
+            *nrm_w = nreg;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const uint4 na = *nrm_r0, nb = *nrm_r1;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (more) nreg = issue_n(tile + 32);
+
             // ---- scores: S^T[token][head] for both sub-tiles
             float4_t s[2];
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
-                s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
-                const uint32_t w[4] = {cur.k[sub].x, cur.k[sub].y, cur.k[sub].z, cur.k[sub].w};
+                const uint32_t w[4] = {kreg[sub].x, kreg[sub].y, kreg[sub].z, kreg[sub].w};
+                union { uint32_t u[4]; half8_t h; } av[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    union { uint32_t u[4]; half8_t h; } av;
-                    av.u[0] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
-                    av.u[1] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
-                    av.u[2] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
-                    av.u[3] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
-                    s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av.h, bq[j], s[sub], 0, 0, 0);
+                    av[j].u[0] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
+                    av[j].u[1] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
+                    av[j].u[2] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
+                    av[j].u[3] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
                 }
+                s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[j].h, bq[j], s[sub], 0, 0, 0);
             }
+            if (more) issue_k(kreg, tile + 32);
+
             // ---- online softmax (base 2) for head ln over the 8 tokens this lane holds
-            float sv[8], vnv[8];
+            const uint32_t nrm[8] = {na.x, na.y, na.z, na.w, nb.x, nb.y, nb.z, nb.w};
+            float sv[8];
 #pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    float knr = h2f_bits((uint32_t)__shfl((int)cur.kn[sub], 4 * kg + r, 64));
-                    vnv[4 * sub + r] = h2f_bits((uint32_t)__shfl((int)cur.vn[sub], 4 * kg + r, 64));
-                    float sc = s[sub][r] + dpp_ror8(s[sub][r]);         // hi + lo parts of q_rot
-                    sv[4 * sub + r] = sc * knr;                         // kernels.cu:1707
-                }
+            for (int i = 0; i < 8; i++) {
+                float sc = s[i >> 2][i & 3] + dpp_ror8(s[i >> 2][i & 3]);   // hi + lo parts of q_rot
+                sv[i] = sc * h2f_bits(nrm[i] & 0xffffu);                     // kernels.cu:1707
             }
             if (masked) {
 #pragma unroll
@@ -289,7 +347,7 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
             for (int i = 0; i < 8; i++) {
                 float p = __builtin_amdgcn_exp2f(sv[i] - m_run);
                 l_run += p;
-                float pf = p * vnv[i];                                  // (s * vn) * centroid, kernels.cu:1765
+                float pf = p * h2f_bits(nrm[i] >> 16);                  // (s * vn) * centroid, kernels.cu:1765
                 half_t hi = (half_t)pf;
                 pv.e[i] = hi;
                 plo.e[i] = (half_t)(pf - (float)hi);
@@ -306,33 +364,24 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
             for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
                 for (int pr = 0; pr < 2; pr++) {
-                    uint32_t wa = cur.v[sub][2 * pr], wb = cur.v[sub][2 * pr + 1];
+                    uint32_t wa = vreg[sub][2 * pr], wb = vreg[sub][2 * pr + 1];
                     xe[2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
                     xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
                 }
             }
+            if (more) issue_v(vreg, tile + 32);
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const uint32_t sel = 0x0c0c0400u + ((uint32_t)(j >> 1) << 8);
-                union { uint32_t u[4]; half8_t h; } bv;
+            for (int jp = 0; jp < 4; jp++) {         // two dims (even, odd) per step: 8 look-ups, 2 MFMAs
+                const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
+                union { uint32_t u[4]; half8_t h; } be, bo;
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
-                    uint32_t x = (j & 1) ? xo[q4] : xe[q4];
-                    bv.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(x, lane4, sel));
+                    be.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(xe[q4], lane4, sel));
+                    bo.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(xo[q4], lane4, sel));
                 }
-                o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv.h, bv.h, o[j], 0, 0, 0);
+                o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv.h, be.h, o[2 * jp], 0, 0, 0);
+                o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv.h, bo.h, o[2 * jp + 1], 0, 0, 0);
             }
-        };
-
-        // loads run one tile ahead of the arithmetic
-        const int ntiles = (t1 - t0 + 31) >> 5;
-        TileRegs cur, nxt;
-        issue(cur, t0);
-        for (int it = 0; it < ntiles; it++) {
-            const int tile = t0 + 32 * it;
-            if (it + 1 < ntiles) issue(nxt, tile + 32);
-            compute(cur, tile, tile + 32 > t1);
-            if (it + 1 < ntiles) cur = nxt;
         }
 
         // ---- partial result of this (sequence, KV head, chunk)
@@ -403,7 +452,10 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     const int items = a.G * a.nsplit * hgroups;
     int grid = resident_groups();
     if (items < grid) grid = items;
-    hipLaunchKernelGGL(attention_mfma4_kernel, dim3(grid), dim3(waves * kWave), 0, s, a, items, hgroups);
+    if (a.block_table)
+        hipLaunchKernelGGL(attention_mfma4_kernel<true>, dim3(grid), dim3(waves * kWave), 0, s, a, items, hgroups);
+    else
+        hipLaunchKernelGGL(attention_mfma4_kernel<false>, dim3(grid), dim3(waves * kWave), 0, s, a, items, hgroups);
 }
 
 }  // namespace twkv
