@@ -17,13 +17,17 @@
 //
 // Mapping (one wave = one KV head of one sequence, 32 tokens per iteration):
 //   K: lane (t = lane%16, kg = lane/16) loads 16 bytes = dims [32kg, 32kg+32) of
-//      token t.  Dword j of it is the A operand of MFMA j (v_mfma_f32_16x16x32_f16),
-//      rows = tokens; the B operand holds q_rot for the GQA group's heads in the
-//      matching dimension order, columns = heads.  Result S^T[token][head].
-//   softmax: online, per head, in base 2 (q_rot is pre-scaled by log2(e)/sqrt(D));
-//      S^T's register layout (lane: head = lane%16, tokens 4*(lane/16)+r) is exactly
-//      the A-operand layout P[head][token] of the second contraction, so
-//      probabilities never leave registers.
+//      token t.  Dword j of it is the B operand of MFMA j (v_mfma_f32_16x16x32_f16),
+//      columns = tokens; the A operand holds q_rot for the GQA group's heads in the
+//      matching dimension order, rows = heads.  Result S[head][token]: a lane holds
+//      the scores of ONE token (its lane%16) for the group's heads.
+//   softmax: online, per head, in base 2 (q_rot is pre-scaled by log2(e)/sqrt(D)).
+//      One v_permlane32_swap per head brings the two 16-token sub-tiles into the two
+//      halves of the wave, so a lane does the exponentials of exactly one token; the
+//      running maximum is only raised when a score exceeds it by more than 2^5
+//      (then every accumulator is rescaled), which keeps it uniform over the wave.
+//      The probabilities go through a 1 KB LDS tile into the A-operand layout
+//      P[head][token] of the second contraction (4 ds_write_b16 + 1 ds_read_b128).
 //   V: lane (n = lane%16, kg = lane/16) loads, for tokens 4kg..4kg+3, the dword
 //      that holds dims 8n..8n+7.  Nibbles of two tokens are interleaved with
 //      v_bfi_b32 so that one table look-up yields the fp16 pair (token, token+1) for
@@ -39,8 +43,8 @@
 //      workgroup; waves never synchronise after that.
 //   precision: fp16 operands would cost ~5e-4 relative error each for q_rot and for
 //      the probabilities.  Both are split into hi + lo fp16 parts that ride in MFMA
-//      rows/columns the GQA group leaves empty (head n -> column n and n+8), so the
-//      split costs no extra MFMA; the two halves are added after the contraction.
+//      rows the GQA group leaves empty (head n -> row n and n+8), so the split costs
+//      no extra MFMA; the two halves are added after the contraction.
 //      The centroid table is stored as fp16(alpha * c) with alpha chosen so that all
 //      eight magnitudes round with <= 1.1e-4 relative error (3.6e-4 without it);
 //      1/alpha is folded into q_rot and into the final accumulator.
@@ -71,11 +75,6 @@ __device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
 }
 
 
-// value of the lane 8 places away inside the row of 16 lanes (DPP row_ror:8)
-__device__ __forceinline__ float dpp_ror8(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
-}
-
 __device__ __forceinline__ float h2f_bits(uint32_t bits16) {
     union { uint16_t u; half_t h; } cv;
     cv.u = (uint16_t)bits16;
@@ -85,6 +84,7 @@ __device__ __forceinline__ float h2f_bits(uint32_t bits16) {
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
 typedef uint32_t uint32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint32x2_t __attribute__((ext_vector_type(2)));
 
 // Buffer descriptor over [base, base + bytes).  Every input is forced into scalar
 // registers: a descriptor held in vector registers makes each load a serialising loop.
@@ -118,18 +118,18 @@ query_rotate_kernel(AttnArgs a) {
     a.qrot[((long long)g * a.num_heads + head) * a.ws_stride + d] = acc * (kLog2e * kInvSqrtD / kAlpha4);
 }
 
-template <bool PAGED>
+template <bool PAGED, int R>
 __global__ void __launch_bounds__(kMaxWaves * kWave, 4)
 attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
-    __shared__ __attribute__((aligned(16))) uint32_t nrm_s[kMaxWaves][32];   // per wave: kn | vn << 16 of 32 tokens
+    // per wave: P[row][k] as fp16, rows 0..R-1 = heads, rows 8..8+R-1 = rounding remainders
+    __shared__ __attribute__((aligned(16))) half_t p_s[kMaxWaves][16][32];
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int wave = uniform(tid / kWave), lane = tid % kWave;   // wave index is wave-uniform: keep it scalar
     const int ln = lane & 15, kg = lane >> 4;
     const int waves = nthreads / kWave;
-    const int R = a.num_heads / a.num_kv_heads;
     const int Hk = a.num_kv_heads;
 
     // ---- dequantization table, once per workgroup: entry e, 64 identical words
@@ -139,6 +139,7 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
         uint32_t w = *reinterpret_cast<uint32_t*>(&p);
         *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
     }
+    for (int i = tid; i < kMaxWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
     __syncthreads();
 
     const char* tab_lane = reinterpret_cast<const char*>(tab_s);
@@ -151,11 +152,14 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
 #pragma unroll
     for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(4 * kg + i) * kvp + 4u * (uint32_t)ln;
     const uint32_t sub_bytes = 16u * kvp;              // sub-tile b follows sub-tile a when contiguous
-    // norms: lane (ln, kg) fetches token ln of sub-tile (kg & 1)
-    const uint32_t noff = (uint32_t)ln * nrow + (PAGED ? 0u : (uint32_t)(kg & 1) * 16u * nrow);
-    uint32_t* nrm_w = &nrm_s[wave][(kg & 1) * 16 + ln];
-    const uint4* nrm_r0 = reinterpret_cast<const uint4*>(&nrm_s[wave][4 * kg]);
-    const uint4* nrm_r1 = reinterpret_cast<const uint4*>(&nrm_s[wave][16 + 4 * kg]);
+    // After the sub-tile swap a lane owns token ln of sub-tile (kg >> 1); lanes with odd kg idle.
+    const int my_sub = kg >> 1;
+    const bool useful = (kg & 1) == 0;
+    const uint32_t noff = (uint32_t)ln * nrow + (PAGED ? 0u : (uint32_t)my_sub * 16u * nrow);
+    // slot of that token in the k order of the P.V contraction: k = 8*(t/4) + 4*sub + t%4
+    half_t* p_w = &p_s[wave][0][8 * (ln >> 2) + 4 * my_sub + (ln & 3)];
+    const uint4* p_r = reinterpret_cast<const uint4*>(&p_s[wave][ln][8 * kg]);
+    constexpr float kRaise = 5.0f;                     // raise the running max only past 2^5
 
     for (int item = blockIdx.x; item < total_items; item += gridDim.x) {
         const int hg = item % hgroups;
@@ -167,9 +171,9 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
         if (t0 >= n) continue;                                // uniform
         const int t1 = min(n, t0 + a.chunk_len);
 
-        // B operand of the score MFMAs: q_rot[head][32kg + 8j + i]; column n carries the
-        // fp16 value of head n, column n + 8 what the rounding left over.
-        half8_t bq[4];
+        // A operand of the score MFMAs: q_rot[head][32kg + 8j + i]; row m carries the
+        // fp16 value of head m, row m + 8 what the rounding left over.
+        half8_t aq[4];
         {
             const int hq = ln & 7;
             const bool lo_part = (ln & 8) != 0;
@@ -184,7 +188,7 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                     float x = (hq < R) ? v[i] : 0.0f;
                     half_t hi = (half_t)x;
                     half_t lo = (half_t)(x - (float)hi);
-                    bq[j][i] = lo_part ? lo : hi;
+                    aq[j][i] = lo_part ? lo : hi;
                 }
             }
         }
@@ -237,12 +241,9 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                 }
             }
         };
-        // packed norms kn | vn << 16 of token (sub = kg & 1, ln)
+        // fp16 bits of kn (low half) and vn (high half) of this lane's token
         auto issue_n = [&](int tile) -> uint32_t {
-            long long row;
-            int rows;
             if (PAGED) {
-                // both pages' rows are needed; lanes pick theirs by kg & 1
                 long long r0 = page_row(tile), r1 = page_row(tile + 16);
                 __amdgpu_buffer_rsrc_t ka = make_rsrc(knseq + r0 * nrow, kPageTokens * (int)nrow);
                 __amdgpu_buffer_rsrc_t kb = make_rsrc(knseq + r1 * nrow, kPageTokens * (int)nrow);
@@ -252,10 +253,10 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                 uint32_t k1 = __builtin_amdgcn_raw_buffer_load_b16(kb, (int)noff, 0, 0);
                 uint32_t v0 = __builtin_amdgcn_raw_buffer_load_b16(va, (int)noff, 0, 0);
                 uint32_t v1 = __builtin_amdgcn_raw_buffer_load_b16(vb, (int)noff, 0, 0);
-                return (kg & 1) ? (k1 | (v1 << 16)) : (k0 | (v0 << 16));
+                return my_sub ? (k1 | (v1 << 16)) : (k0 | (v0 << 16));
             }
-            row = seq_row0 + tile;
-            rows = max(min(n - tile, 32), 0);
+            const long long row = seq_row0 + tile;
+            const int rows = max(min(n - tile, 32), 0);
             __amdgpu_buffer_rsrc_t rk = make_rsrc(knseq + row * nrow, rows * (int)nrow);
             __amdgpu_buffer_rsrc_t rv = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
             uint32_t kk = __builtin_amdgcn_raw_buffer_load_b16(rk, (int)noff, 0, 0);
@@ -266,7 +267,9 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
         float4_t o[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-        float m_run = kNegBig, l_run = 0.0f;
+        float m_run[R], l_run[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
 
         // Loads are re-issued into the same registers as soon as their contents have been
         // expanded, which leaves about two thirds of an iteration to cover their latency.
@@ -281,83 +284,72 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
         for (int it = 0; it < ntiles; it++) {
             const int tile = t0 + 32 * it;
             const bool more = it + 1 < ntiles;
-            const bool masked = tile + 32 > t1;
 
-            // norms: through LDS into the layout of the scores (tokens 4kg..4kg+3 of each sub-tile)
-            *nrm_w = nreg;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            const uint4 na = *nrm_r0, nb = *nrm_r1;
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            if (more) nreg = issue_n(tile + 32);
-
-            // ---- scores: S^T[token][head] for both sub-tiles
+            // ---- scores S[head][token] for both sub-tiles
             float4_t s[2];
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
                 const uint32_t w[4] = {kreg[sub].x, kreg[sub].y, kreg[sub].z, kreg[sub].w};
-                union { uint32_t u[4]; half8_t h; } av[4];
+                union { uint32_t u[4]; half8_t h; } kv[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    av[j].u[0] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
-                    av[j].u[1] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
-                    av[j].u[2] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
-                    av[j].u[3] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
+                    kv[j].u[0] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
+                    kv[j].u[1] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
+                    kv[j].u[2] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
+                    kv[j].u[3] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
                 }
                 s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[j].h, bq[j], s[sub], 0, 0, 0);
+                for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[sub], 0, 0, 0);
             }
             if (more) issue_k(kreg, tile + 32);
 
-            // ---- online softmax (base 2) for head ln over the 8 tokens this lane holds
-            const uint32_t nrm[8] = {na.x, na.y, na.z, na.w, nb.x, nb.y, nb.z, nb.w};
-            float sv[8];
+            // ---- online softmax (base 2): this lane owns token ln of sub-tile my_sub
+            const float kn = h2f_bits(nreg & 0xffffu), vn = h2f_bits(nreg >> 16);
+            if (more) nreg = issue_n(tile + 32);
+            const bool valid = useful && (tile + 16 * my_sub + ln < t1);
+            float raw[R], x[R];
+            bool raise = false;
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                float sc = s[i >> 2][i & 3] + dpp_ror8(s[i >> 2][i & 3]);   // hi + lo parts of q_rot
-                sv[i] = sc * h2f_bits(nrm[i] & 0xffffu);                     // kernels.cu:1707
+            for (int r = 0; r < R; r++) {
+                // rows r (hi part of q_rot) and r + 8 (lo part) sit 32 lanes apart; the swap also
+                // moves sub-tile b into the upper half of the wave
+                uint32x2_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(s[0][r]), __float_as_uint(s[1][r]), false, false);
+                raw[r] = (__uint_as_float(sw[0]) + __uint_as_float(sw[1])) * kn;    // kernels.cu:1707
+                x[r] = valid ? raw[r] - m_run[r] : kNegBig;
+                raise = raise || (x[r] > kRaise);
             }
-            if (masked) {
+            if (__any(raise)) {                                         // rare after the first tiles
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    int t = tile + 16 * (i >> 2) + 4 * kg + (i & 3);
-                    sv[i] = (t < t1) ? sv[i] : kNegBig;
+                for (int r = 0; r < R; r++) {
+                    float m_new = fmaxf(m_run[r], wave_max(valid ? raw[r] : kNegBig));
+                    float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                    m_run[r] = m_new;
+                    l_run[r] *= alpha;
+                    x[r] = valid ? raw[r] - m_new : kNegBig;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) o[j][r] *= alpha;       // rows r and r + 8 live in register r
                 }
             }
-            float mt = sv[0];
 #pragma unroll
-            for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
-            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-            const float m_new = fmaxf(m_run, mt);
-            if (__any(m_new > m_run)) {                                 // rare after the first tiles
-                float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                l_run *= alpha;
-                m_run = m_new;
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    float ar = __shfl(alpha, 4 * kg + r, 64);           // O rows are heads 4kg + r
-#pragma unroll
-                    for (int j = 0; j < 8; j++) o[j][r] *= ar;
-                }
-            }
-            union { half_t e[8]; uint32_t u[4]; half8_t h; } pv, plo;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                float p = __builtin_amdgcn_exp2f(sv[i] - m_run);
-                l_run += p;
-                float pf = p * h2f_bits(nrm[i] >> 16);                  // (s * vn) * centroid, kernels.cu:1765
+            for (int r = 0; r < R; r++) {
+                float p = __builtin_amdgcn_exp2f(x[r]);
+                l_run[r] += p;
+                float pf = p * vn;                                      // (s * vn) * centroid, kernels.cu:1765
                 half_t hi = (half_t)pf;
-                pv.e[i] = hi;
-                plo.e[i] = (half_t)(pf - (float)hi);
+                half_t lo = (half_t)(pf - (float)hi);
+                if (useful) {
+                    p_w[r * 32] = hi;
+                    p_w[(r + 8) * 32] = lo;
+                }
             }
-            // rows 8..15 of P carry the rounding remainder of rows 0..7
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                uint32_t moved = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)plo.u[q4], 0x128, 0xf, 0xf, false);
-                pv.u[q4] = (ln & 8) ? moved : pv.u[q4];
-            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            union { uint4 q; half8_t h; } pa;
+            pa.q = *p_r;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+
             // ---- O[head][dim 8ln + j] += P[head][token] V[token][dim]
             uint32_t xe[4], xo[4];   // [2*sub + pair]: index bytes for even / odd dims
 #pragma unroll
@@ -379,34 +371,29 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                     be.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(xe[q4], lane4, sel));
                     bo.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(xo[q4], lane4, sel));
                 }
-                o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv.h, be.h, o[2 * jp], 0, 0, 0);
-                o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv.h, bo.h, o[2 * jp + 1], 0, 0, 0);
+                o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * jp], 0, 0, 0);
+                o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * jp + 1], 0, 0, 0);
             }
         }
 
         // ---- partial result of this (sequence, KV head, chunk)
-        l_run += __shfl_xor(l_run, 16, 64);
-        l_run += __shfl_xor(l_run, 32, 64);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
+        for (int r = 0; r < R; r++) {
+            l_run[r] = wave_sum(l_run[r]);                                        // idle and masked lanes hold 0
 #pragma unroll
-            for (int j = 0; j < 8; j++) o[j][r] += __shfl_xor(o[j][r], 32, 64);   // row hm + row hm+8 (lo part of P)
+            for (int j = 0; j < 8; j++) o[j][r] += __shfl_xor(o[j][r], 32, 64);   // row r + row r+8 (lo part of P)
         }
         if (kg == 0) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                if (r < R) {
-                    float* part = a.ws + ((long long)g * a.num_heads + (long long)h * R + r) * a.ws_stride +
-                                  (long long)chunk * kPartialFloats;
-#pragma unroll
-                    for (int j = 0; j < 8; j++) part[8 * ln + j] = o[j][r] * (1.0f / kAlpha4);
-                }
-            }
-            if (ln < R) {
-                float* part = a.ws + ((long long)g * a.num_heads + (long long)h * R + ln) * a.ws_stride +
+            for (int r = 0; r < R; r++) {
+                float* part = a.ws + ((long long)g * a.num_heads + (long long)h * R + r) * a.ws_stride +
                               (long long)chunk * kPartialFloats;
-                part[kHeadDim] = m_run;
-                part[kHeadDim + 1] = l_run;
+#pragma unroll
+                for (int j = 0; j < 8; j++) part[8 * ln + j] = o[j][r] * (1.0f / kAlpha4);
+                if (ln == 0) {
+                    part[kHeadDim] = m_run[r];
+                    part[kHeadDim + 1] = l_run[r];
+                }
             }
         }
     }
@@ -433,7 +420,7 @@ static int scan_waves(const AttnArgs& a) {
 bool prepare_attention_mfma(AttnArgs& a, hipStream_t s) {
     const int R = a.num_heads / a.num_kv_heads;
     if (a.bits != 4) return false;
-    if (R > kMaxGroup) return false;
+    if (R != 1 && R != 2 && R != 4) return false;
     if (a.chunk_len % 32 != 0) return false;
     // needs the split workspace with room for q_rot behind each block's partials
     if (!a.ws || !a.qrot) return false;
@@ -452,10 +439,15 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     const int items = a.G * a.nsplit * hgroups;
     int grid = resident_groups();
     if (items < grid) grid = items;
-    if (a.block_table)
-        hipLaunchKernelGGL(attention_mfma4_kernel<true>, dim3(grid), dim3(waves * kWave), 0, s, a, items, hgroups);
-    else
-        hipLaunchKernelGGL(attention_mfma4_kernel<false>, dim3(grid), dim3(waves * kWave), 0, s, a, items, hgroups);
+    const int R = a.num_heads / a.num_kv_heads;
+    const dim3 g3(grid), b3(waves * kWave);
+#define TW_LAUNCH(P, RR) hipLaunchKernelGGL((attention_mfma4_kernel<P, RR>), g3, b3, 0, s, a, items, hgroups)
+    if (a.block_table) {
+        if (R == 1) TW_LAUNCH(true, 1); else if (R == 2) TW_LAUNCH(true, 2); else TW_LAUNCH(true, 4);
+    } else {
+        if (R == 1) TW_LAUNCH(false, 1); else if (R == 2) TW_LAUNCH(false, 2); else TW_LAUNCH(false, 4);
+    }
+#undef TW_LAUNCH
 }
 
 }  // namespace twkv
