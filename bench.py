@@ -134,6 +134,9 @@ def main():
     ap.add_argument("--nsplit", type=int, default=0)
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--ctx", type=int, default=None, help="override the workload's context length")
+    ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
+    ap.add_argument("--layers", type=int, default=None, help="override the workload's layer count")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; sharding is by sequence or KV head with no exchange "
@@ -145,6 +148,13 @@ def main():
 
     w = dict(WORKLOADS[args.workload])
     kv_bits = w["kv_bits"] if args.kv_bits is None else args.kv_bits
+    overridden = []
+    for key, val in (("ctx", args.ctx), ("G", args.batch), ("L", args.layers)):
+        if val is not None:
+            w[key] = val
+            overridden.append(f"{key}={val}")
+    if overridden:
+        w["desc"] += " [override " + ",".join(overridden) + "]"
     L, H, Hk, G, D = w["L"], w["H"], w["Hk"], w["G"], 128
     K, W = args.steps, args.warmup
     kv_dim, q_dim = Hk * D, H * D

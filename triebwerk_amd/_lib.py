@@ -8,7 +8,10 @@ from __future__ import annotations
 import ctypes as C
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriebwerk_kv.so"
+import os
+
+# TRIEBWERK_KV_LIB selects another build of the same library (e.g. an experiment).
+LIB_PATH = Path(os.environ.get("TRIEBWERK_KV_LIB") or Path(__file__).resolve().parent / "lib" / "libtriebwerk_kv.so")
 
 P = C.c_void_p
 I = C.c_int

@@ -54,6 +54,16 @@
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 
+#ifndef TW_EXP
+#define TW_EXP 0
+#endif
+#ifndef TW_DEPTH
+#define TW_DEPTH 1
+#endif
+#define TW_LUT(addr) ((TW_EXP == 3 || TW_EXP == 4) ? ((uint32_t)(addr) & 0x33ffu) : *reinterpret_cast<const uint32_t*>(tab_lane + (addr)))
+#define TW_LUTK(addr) ((TW_EXP == 1) ? ((uint32_t)(addr) & 0x33ffu) : TW_LUT(addr))
+#define TW_LUTV(addr) ((TW_EXP == 2) ? ((uint32_t)(addr) & 0x33ffu) : TW_LUT(addr))
+
 namespace twkv {
 
 namespace {
@@ -118,8 +128,8 @@ query_rotate_kernel(AttnArgs a) {
     a.qrot[((long long)g * a.num_heads + head) * a.ws_stride + d] = acc * (kLog2e * kInvSqrtD / kAlpha4);
 }
 
-template <bool PAGED, int R>
-__global__ void __launch_bounds__(kMaxWaves * kWave, 4)
+template <bool PAGED, int R, int DEPTH>
+__global__ void __launch_bounds__(kMaxWaves * kWave, (DEPTH <= 1 ? 4 : 2))
 attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
     // per wave: P[row][k] as fp16, rows 0..R-1 = heads, rows 8..8+R-1 = rounding remainders
@@ -131,16 +141,6 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     const int ln = lane & 15, kg = lane >> 4;
     const int waves = nthreads / kWave;
     const int Hk = a.num_kv_heads;
-
-    // ---- dequantization table, once per workgroup: entry e, 64 identical words
-    for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
-        int e = i >> 6;
-        half2_t p = {(half_t)(kAlpha4 * kCentroids4[e & 15]), (half_t)(kAlpha4 * kCentroids4[e >> 4])};
-        uint32_t w = *reinterpret_cast<uint32_t*>(&p);
-        *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
-    }
-    for (int i = tid; i < kMaxWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
-    __syncthreads();
 
     const char* tab_lane = reinterpret_cast<const char*>(tab_s);
     const uint32_t lane4 = (uint32_t)lane * 4u;
@@ -161,37 +161,16 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     const uint4* p_r = reinterpret_cast<const uint4*>(&p_s[wave][ln][8 * kg]);
     constexpr float kRaise = 5.0f;                     // raise the running max only past 2^5
 
+    bool table_ready = false;
     for (int item = blockIdx.x; item < total_items; item += gridDim.x) {
         const int hg = item % hgroups;
         const int chunk = (item / hgroups) % a.nsplit;
         const int g = item / (hgroups * a.nsplit);
         const int h = hg * waves + wave;                      // KV head of this wave
         const int n = uniform(seq_pos(a, g)) + 1;
-        const int t0 = chunk * a.chunk_len;
-        if (t0 >= n) continue;                                // uniform
-        const int t1 = min(n, t0 + a.chunk_len);
-
-        // A operand of the score MFMAs: q_rot[head][32kg + 8j + i]; row m carries the
-        // fp16 value of head m, row m + 8 what the rounding left over.
-        half8_t aq[4];
-        {
-            const int hq = ln & 7;
-            const bool lo_part = (ln & 8) != 0;
-            const float* qr = a.qrot + ((long long)g * a.num_heads + (long long)h * R + (hq < R ? hq : 0)) * a.ws_stride + 32 * kg;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
-                float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
-                float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    float x = (hq < R) ? v[i] : 0.0f;
-                    half_t hi = (half_t)x;
-                    half_t lo = (half_t)(x - (float)hi);
-                    aq[j][i] = lo_part ? lo : hi;
-                }
-            }
-        }
+        int t0, t1;
+        chunk_range(n, chunk, a.nsplit, t0, t1);
+        if (t0 >= t1) continue;                               // uniform
 
         // scalar bases of this wave's head
         const char* kseq = reinterpret_cast<const char*>(a.k) + (long long)h * 64;
@@ -241,22 +220,48 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                 }
             }
         };
-        // fp16 bits of kn (low half) and vn (high half) of this lane's token
+        // fp16 bits of kn (low half) and vn (high half) of this lane's token.  When a norm row
+        // (all KV heads of one token) is a multiple of 16 bytes the lane fetches the 16 bytes
+        // that hold its head with one b128 load (rows of consecutive tokens are contiguous, so
+        // the 32 useful lanes read one contiguous run) and picks its half-word; a 2-byte gather
+        // over the same rows costs ~15 % of the whole scan's bandwidth.
+        auto pick = [&](const uint32x4_t& q) -> uint32_t {
+            const int dw = (h & 7) >> 1;
+            uint32_t w = dw == 0 ? q[0] : dw == 1 ? q[1] : dw == 2 ? q[2] : q[3];
+            return (h & 1) ? (w >> 16) : (w & 0xffffu);
+        };
         auto issue_n = [&](int tile) -> uint32_t {
+            const bool wide = (nrow & 15u) == 0;
+            const uint32_t hgrp = (uint32_t)(h >> 3) * 16u;          // 16-byte group of this head inside a row
             if (PAGED) {
                 long long r0 = page_row(tile), r1 = page_row(tile + 16);
-                __amdgpu_buffer_rsrc_t ka = make_rsrc(knseq + r0 * nrow, kPageTokens * (int)nrow);
-                __amdgpu_buffer_rsrc_t kb = make_rsrc(knseq + r1 * nrow, kPageTokens * (int)nrow);
-                __amdgpu_buffer_rsrc_t va = make_rsrc(vnseq + r0 * nrow, kPageTokens * (int)nrow);
-                __amdgpu_buffer_rsrc_t vb = make_rsrc(vnseq + r1 * nrow, kPageTokens * (int)nrow);
-                uint32_t k0 = __builtin_amdgcn_raw_buffer_load_b16(ka, (int)noff, 0, 0);
-                uint32_t k1 = __builtin_amdgcn_raw_buffer_load_b16(kb, (int)noff, 0, 0);
-                uint32_t v0 = __builtin_amdgcn_raw_buffer_load_b16(va, (int)noff, 0, 0);
-                uint32_t v1 = __builtin_amdgcn_raw_buffer_load_b16(vb, (int)noff, 0, 0);
-                return my_sub ? (k1 | (v1 << 16)) : (k0 | (v0 << 16));
+                const long long rr = my_sub ? r1 : r0;
+                if (wide) {
+                    uint32x4_t kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
+                    if (useful) {
+                        const char* kp = reinterpret_cast<const char*>(a.k_norms) + (rr + ln) * nrow + hgrp;
+                        const char* vp = reinterpret_cast<const char*>(a.v_norms) + (rr + ln) * nrow + hgrp;
+                        kq = *reinterpret_cast<const uint32x4_t*>(kp);
+                        vq = *reinterpret_cast<const uint32x4_t*>(vp);
+                    }
+                    return pick(kq) | (pick(vq) << 16);
+                }
+                uint32_t kk = *reinterpret_cast<const uint16_t*>(knseq + (rr + ln) * nrow);
+                uint32_t vv = *reinterpret_cast<const uint16_t*>(vnseq + (rr + ln) * nrow);
+                return kk | (vv << 16);
             }
             const long long row = seq_row0 + tile;
             const int rows = max(min(n - tile, 32), 0);
+            if (wide) {
+                __amdgpu_buffer_rsrc_t rk = make_rsrc(reinterpret_cast<const char*>(a.k_norms) + row * nrow, rows * (int)nrow);
+                __amdgpu_buffer_rsrc_t rv = make_rsrc(reinterpret_cast<const char*>(a.v_norms) + row * nrow, rows * (int)nrow);
+                uint32x4_t kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
+                if (useful) {
+                    kq = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)(noff + hgrp), 0, 0);
+                    vq = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)(noff + hgrp), 0, 0);
+                }
+                return pick(kq) | (pick(vq) << 16);
+            }
             __amdgpu_buffer_rsrc_t rk = make_rsrc(knseq + row * nrow, rows * (int)nrow);
             __amdgpu_buffer_rsrc_t rv = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
             uint32_t kk = __builtin_amdgcn_raw_buffer_load_b16(rk, (int)noff, 0, 0);
@@ -271,20 +276,104 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
 #pragma unroll
         for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
 
-        // Loads are re-issued into the same registers as soon as their contents have been
-        // expanded, which leaves about two thirds of an iteration to cover their latency.
+        // DEPTH tiles of loads are in flight per wave; a slot is re-issued (for the tile DEPTH
+        // further on) as soon as its contents have been expanded.
         const int ntiles = (t1 - t0 + 31) >> 5;
-        uint4 kreg[2];
-        uint32_t vreg[2][4];
-        uint32_t nreg;
-        issue_k(kreg, t0);
-        nreg = issue_n(t0);
-        issue_v(vreg, t0);
+        uint4 kring[DEPTH][2];
+        uint32_t vring[DEPTH][2][4];
+        uint32_t nring[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (d < ntiles && TW_EXP != 5) {
+                issue_k(kring[d], t0 + 32 * d);
+                nring[d] = issue_n(t0 + 32 * d);
+                issue_v(vring[d], t0 + 32 * d);
+            }
+        }
 
-        for (int it = 0; it < ntiles; it++) {
+        // The first loads are already in flight while the workgroup builds its table.
+        if (!table_ready) {
+        // ---- dequantization table, once per workgroup: entry e, 64 identical words
+        for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
+            int e = i >> 6;
+            half2_t p = {(half_t)(kAlpha4 * kCentroids4[e & 15]), (half_t)(kAlpha4 * kCentroids4[e >> 4])};
+            uint32_t w = *reinterpret_cast<uint32_t*>(&p);
+            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
+        }
+        for (int i = tid; i < kMaxWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
+        __syncthreads();
+            table_ready = true;
+        }
+
+        // A operand of the score MFMAs: q_rot[head][32kg + 8j + i]; row m carries the
+        // fp16 value of head m, row m + 8 what the rounding left over.
+        half8_t aq[4];
+        {
+            const int hq = ln & 7;
+            const bool lo_part = (ln & 8) != 0;
+            const float* qr = a.qrot + ((long long)g * a.num_heads + (long long)h * R + (hq < R ? hq : 0)) * a.ws_stride + 32 * kg;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
+                float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
+                float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float x = (hq < R) ? v[i] : 0.0f;
+                    half_t hi = (half_t)x;
+                    half_t lo = (half_t)(x - (float)hi);
+                    aq[j][i] = lo_part ? lo : hi;
+                }
+            }
+        }
+
+
+        for (int it0 = 0; it0 < ntiles; it0 += DEPTH) {
+#pragma unroll
+          for (int d = 0; d < DEPTH; d++) {
+            const int it = it0 + d;
+            if (it >= ntiles) break;
+            uint4 (&kreg)[2] = kring[d];
+            uint32_t (&vreg)[2][4] = vring[d];
+            uint32_t& nreg = nring[d];
             const int tile = t0 + 32 * it;
-            const bool more = it + 1 < ntiles;
+            const int next_tile = tile + 32 * DEPTH;
+            const bool more = it + DEPTH < ntiles;
 
+#if TW_EXP == 5
+            {   // loads only, plain global loads with per-lane 64-bit pointers
+                const char* kp = kseq + (seq_row0 + tile) * kvp + koff;
+                const char* vp = vseq + (seq_row0 + tile) * kvp;
+                uint4 ka = *reinterpret_cast<const uint4*>(kp);
+                uint4 kb2 = *reinterpret_cast<const uint4*>(kp + sub_bytes);
+                uint32_t f = ka.x ^ ka.w ^ kb2.y ^ kb2.z;
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) f ^= *reinterpret_cast<const uint32_t*>(vp + voff[i] + sub * sub_bytes);
+                if (useful) {
+                    const char* np_ = reinterpret_cast<const char*>(a.k_norms) + (seq_row0 + tile) * nrow + noff;
+                    const char* nq_ = reinterpret_cast<const char*>(a.v_norms) + (seq_row0 + tile) * nrow + noff;
+                    uint4 n1 = *reinterpret_cast<const uint4*>(np_);
+                    uint4 n2 = *reinterpret_cast<const uint4*>(nq_);
+                    f ^= n1.x ^ n2.w;
+                }
+                o[0][0] += __uint_as_float(f & 0x3fffffu);
+                continue;
+            }
+#endif
+#if TW_EXP == 4
+            {   // loads only: fold the loaded words into one accumulator and re-issue
+                uint32_t f = kreg[0].x ^ kreg[0].y ^ kreg[0].z ^ kreg[0].w ^ kreg[1].x ^ kreg[1].y ^ kreg[1].z ^ kreg[1].w ^ nreg;
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) f ^= vreg[sub][i];
+                o[0][0] += __uint_as_float(f & 0x3fffffu);
+                if (more) { issue_k(kreg, next_tile); nreg = issue_n(next_tile); issue_v(vreg, next_tile); }
+                continue;
+            }
+#endif
             // ---- scores S[head][token] for both sub-tiles
             float4_t s[2];
 #pragma unroll
@@ -293,20 +382,20 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                 union { uint32_t u[4]; half8_t h; } kv[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    kv[j].u[0] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
-                    kv[j].u[1] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
-                    kv[j].u[2] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
-                    kv[j].u[3] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
+                    kv[j].u[0] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
+                    kv[j].u[1] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
+                    kv[j].u[2] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
+                    kv[j].u[3] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
                 }
                 s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[sub], 0, 0, 0);
             }
-            if (more) issue_k(kreg, tile + 32);
+            if (more) issue_k(kreg, next_tile);
 
             // ---- online softmax (base 2): this lane owns token ln of sub-tile my_sub
             const float kn = h2f_bits(nreg & 0xffffu), vn = h2f_bits(nreg >> 16);
-            if (more) nreg = issue_n(tile + 32);
+            if (more) nreg = issue_n(next_tile);
             const bool valid = useful && (tile + 16 * my_sub + ln < t1);
             float raw[R], x[R];
             bool raise = false;
@@ -361,19 +450,20 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                     xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
                 }
             }
-            if (more) issue_v(vreg, tile + 32);
+            if (more) issue_v(vreg, next_tile);
 #pragma unroll
             for (int jp = 0; jp < 4; jp++) {         // two dims (even, odd) per step: 8 look-ups, 2 MFMAs
                 const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
                 union { uint32_t u[4]; half8_t h; } be, bo;
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
-                    be.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(xe[q4], lane4, sel));
-                    bo.u[q4] = *reinterpret_cast<const uint32_t*>(tab_lane + __builtin_amdgcn_perm(xo[q4], lane4, sel));
+                    be.u[q4] = TW_LUTV(__builtin_amdgcn_perm(xe[q4], lane4, sel));
+                    bo.u[q4] = TW_LUTV(__builtin_amdgcn_perm(xo[q4], lane4, sel));
                 }
                 o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * jp], 0, 0, 0);
                 o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * jp + 1], 0, 0, 0);
             }
+          }
         }
 
         // ---- partial result of this (sequence, KV head, chunk)
@@ -406,7 +496,7 @@ static int resident_groups() {
         if (hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             cus = 256;
-        cached = 2 * cus;   // 64 KB of LDS and <= 128 VGPRs per workgroup of 8 waves: two per CU
+        cached = (TW_DEPTH <= 1 ? 2 : 1) * cus;   // 64 KB of LDS and <= 128 VGPRs per workgroup of 8 waves: two per CU
     }
     return cached;
 }
@@ -421,7 +511,6 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s) {
     const int R = a.num_heads / a.num_kv_heads;
     if (a.bits != 4) return false;
     if (R != 1 && R != 2 && R != 4) return false;
-    if (a.chunk_len % 32 != 0) return false;
     // needs the split workspace with room for q_rot behind each block's partials
     if (!a.ws || !a.qrot) return false;
     if ((reinterpret_cast<uintptr_t>(a.qrot) & 15u) != 0 || (a.ws_stride & 3) != 0) return false;
@@ -441,7 +530,10 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     if (items < grid) grid = items;
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3(grid), b3(waves * kWave);
-#define TW_LAUNCH(P, RR) hipLaunchKernelGGL((attention_mfma4_kernel<P, RR>), g3, b3, 0, s, a, items, hgroups)
+#ifndef TW_DEPTH
+#define TW_DEPTH 1
+#endif
+#define TW_LAUNCH(P, RR) hipLaunchKernelGGL((attention_mfma4_kernel<P, RR, TW_DEPTH>), g3, b3, 0, s, a, items, hgroups)
     if (a.block_table) {
         if (R == 1) TW_LAUNCH(true, 1); else if (R == 2) TW_LAUNCH(true, 2); else TW_LAUNCH(true, 4);
     } else {

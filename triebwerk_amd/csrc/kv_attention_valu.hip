@@ -110,9 +110,9 @@ attention_valu_kernel(AttnArgs a) {
     const int head0 = h * group + (blockIdx.y % subs) * RT;
 
     const int n = seq_pos(a, g) + 1;
-    const int t0 = chunk * a.chunk_len;
-    if (t0 >= n) return;                        // uniform for the workgroup
-    const int t1 = min(n, t0 + a.chunk_len);
+    int t0, t1;
+    chunk_range(n, chunk, a.nsplit, t0, t1);
+    if (t0 >= t1) return;                       // uniform for the workgroup
 
     if (tid < 16) cent_s[tid] = (MODE == 2) ? kCentroids2[tid & 3] : kCentroids4[tid];
 
@@ -266,13 +266,18 @@ attention_merge_kernel(AttnArgs a) {
     __shared__ float o_s[kHeadDim];
     const int head = blockIdx.x, g = blockIdx.y, d = threadIdx.x;
     const int n = seq_pos(a, g) + 1;
-    int nchunks = (n + a.chunk_len - 1) / a.chunk_len;
-    if (nchunks > a.nsplit) nchunks = a.nsplit;
     const float* part = a.ws + ((long long)g * a.num_heads + head) * a.ws_stride;
     float mg = kNegBig;
-    for (int cidx = 0; cidx < nchunks; cidx++) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
+    for (int cidx = 0; cidx < a.nsplit; cidx++) {
+        int t0, t1;
+        chunk_range(n, cidx, a.nsplit, t0, t1);
+        if (t0 < t1) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
+    }
     float lsum = 0.0f, av = 0.0f;
-    for (int cidx = 0; cidx < nchunks; cidx++) {
+    for (int cidx = 0; cidx < a.nsplit; cidx++) {
+        int t0, t1;
+        chunk_range(n, cidx, a.nsplit, t0, t1);
+        if (t0 >= t1) continue;                 // no workgroup wrote this slot
         const float* pc = part + (long long)cidx * kPartialFloats;
         float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
         lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);

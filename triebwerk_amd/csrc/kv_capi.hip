@@ -27,7 +27,7 @@ constexpr int kMaxSplits = 64;
 constexpr long long kPagedBlockFloats = 64 * 130 + 128 + 4;  // per (sequence, head): partials + rotated query
 constexpr int kMinChunk = 128;       // tokens
 constexpr int kTargetGroups = 2048;  // workgroups wanted per launch: 8 per CU on 256 CUs
-constexpr int kTargetItems = 1024;   // (sequence, chunk) items wanted by the persistent MFMA scan
+constexpr int kTargetItems = 512;    // (sequence, chunk) items wanted by the persistent MFMA scan: one per resident workgroup
 
 void set_error(int code, const char* fmt, ...) {
     if (g_err != 0) return;  // keep the first one
@@ -94,11 +94,8 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     bool have_ws = max_by_ws >= 1;
     if (have_ws && nsplit > max_by_ws) nsplit = max_by_ws;
     if (!have_ws) nsplit = 1;
-    int chunk = (ctx_bound + nsplit - 1) / nsplit;
-    chunk = (chunk + 63) / 64 * 64;
-    nsplit = (ctx_bound + chunk - 1) / chunk;
     a.nsplit = nsplit;
-    a.chunk_len = chunk;
+    a.chunk_len = 0;   // chunks are cut per sequence on the device (chunk_range)
     if (have_ws) {
         long long qoff = ((long long)nsplit * kPartialFloats + 3) & ~3LL;
         a.ws_stride = qoff + kHeadDim;

@@ -72,6 +72,17 @@ __device__ __forceinline__ long long cache_row(const int* __restrict__ block_tab
     return (long long)g * seq_stride_rows + p;
 }
 
+// Chunk c of nsplit of a sequence of n tokens: the sequence's 32-token tiles are dealt
+// out evenly, so every chunk of one sequence has the same length to within one tile
+// whatever max_seq_len the caller allocated.  Empty (t0 >= t1) when n has fewer tiles
+// than nsplit.
+__device__ __forceinline__ void chunk_range(int n, int c, int nsplit, int& t0, int& t1) {
+    const long long tiles = (n + 31) >> 5;
+    t0 = 32 * (int)((c * tiles) / nsplit);
+    int e = 32 * (int)(((c + 1) * tiles) / nsplit);
+    t1 = e < n ? e : n;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
