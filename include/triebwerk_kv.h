@@ -152,6 +152,18 @@ void tw_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q, tw
                               const int* positions, int max_seq_len, int G, int num_kv_heads,
                               int head_dim, int kv_dim, int bits, hipStream_t s);
 
+/* One decode step of one layer in a single call: append K and V at positions[g],
+ * then attention over 0..positions[g] (forward_layer_batch steps 4-5,
+ * engine.cpp:1979-2006).  Same results as tw_turbo_kv_append_batch followed by
+ * launch_turbo_gqa_attention_batch; the rotation of the appended rows and of the
+ * query share one launch. */
+void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf,
+                                     const tw_half* v_buf, uint8_t* ck_q, uint8_t* cv_q,
+                                     tw_half* k_norms, tw_half* v_norms, const tw_half* rotation,
+                                     float* as, const int* pos, int msl, int G, int num_heads,
+                                     int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                     int bits, hipStream_t s);
+
 /* Paged cache.  A page holds TW_PAGE_TOKENS consecutive positions of one
  * sequence in the same row layout the contiguous cache uses, so
  *   row(g, p) = block_table[g*bt_stride + p/16]*16 + p%16

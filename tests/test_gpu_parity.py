@@ -120,9 +120,11 @@ def test_turbo_append_batch_bit_exact(kv, oracle, rotation_fixture, bits):
     assert_bytes_equal(host(d_cn), cn, "norms")
 
 
+@pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("bits", [4, 2])
-def test_turbo_append_many_rows_bit_exact(kv, oracle, rotation_fixture, bits):
-    """A few hundred thousand coordinates: the tie set, if any, shows up here."""
+def test_turbo_append_many_rows_bit_exact(kv, oracle, rotation_fixture, bits, variant):
+    """A few hundred thousand coordinates: the tie set, if any, shows up here.
+    variant 0 = MFMA rotation kernel, 1 = vector-ALU kernel; both must give the oracle's bytes."""
     r = gen.rng(120 + bits)
     G, Hk, msl = 512, 8, 1
     kv_dim = Hk * D
@@ -133,7 +135,11 @@ def test_turbo_append_many_rows_bit_exact(kv, oracle, rotation_fixture, bits):
     margin = np.zeros((G, kv_dim), np.float32)
     oracle.turbo_kv_quantize_batch(cq, cn, rows, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits, None, margin)
     d_cq, d_cn = dev(np.zeros_like(cq)), dev(np.zeros_like(cn))
-    kv.launch_turbo_kv_quantize_batch(d_cq, d_cn, dev(rows), dev(rotation_fixture), dev(pos), msl, G, Hk, D, kv_dim, bits)
+    kv.set_attention_variant(variant)
+    try:
+        kv.launch_turbo_kv_quantize_batch(d_cq, d_cn, dev(rows), dev(rotation_fixture), dev(pos), msl, G, Hk, D, kv_dim, bits)
+    finally:
+        kv.set_attention_variant(0)
     assert_bytes_equal(host(d_cq), cq, f"{bits}-bit codes", margin)
     assert_bytes_equal(host(d_cn), cn, "norms")
 
@@ -319,6 +325,31 @@ def test_turbo_attention_ragged_splits(kv, oracle, rotation_fixture, bits, H, Hk
     finally:
         kv.set_num_splits(0)
         kv.set_attention_variant(0)
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_fused_append_attention_equals_two_calls(kv, oracle, rotation_fixture, bits):
+    """append + attention in one call == oracle append, then oracle attention."""
+    r = gen.rng(340 + bits)
+    G, H, Hk, msl = 7, 16, 8, 320
+    kv_dim, q_dim = Hk * D, H * D
+    lens = [1, 33, 64, 100, 257, 300, 319]
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits)
+    pos = np.array(lens, np.int32)            # the appended token goes right behind the cache
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    import torch
+    d_ck, d_cv, d_kn, d_vn = dev(ck), dev(cv), dev(kn), dev(vn)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.tw_turbo_append_attention_batch(out, dev(q), dev(k), dev(v), d_ck, d_cv, d_kn, d_vn, dev(rotation_fixture),
+                                       scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(cv, vn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    assert_bytes_equal(host(d_ck), ck, "K codes"); assert_bytes_equal(host(d_cv), cv, "V codes")
+    assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+    assert rel_err(host(out), want) <= TOL
 
 
 @pytest.mark.parametrize("bits", [4, 2])

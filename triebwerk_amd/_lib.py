@@ -48,6 +48,7 @@ SIGNATURES = {
     "tw_kv_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_attention_workspace_floats": (SZ, [I, I, I]),
     "tw_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
+    "tw_turbo_append_attention_batch": (None, [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
     "tw_paged_kv_cache_write_batch": (None, [P, P, P, P, P, P, I, I, I, P]),
     "tw_paged_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_paged_gqa_attention_batch": (None, [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),

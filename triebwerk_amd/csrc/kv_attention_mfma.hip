@@ -5,7 +5,7 @@
 // Same mathematics as turbo_gqa_attention_batch_kernel of the reference
 // (kernels.cu:1641-1776): q_rot = R q; s_p = (q_rot . c(K codes_p)) * kn_p / sqrt(D);
 // softmax over p <= pos with "+1e-8" in the denominator; acc = sum_p w_p vn_p c(V codes_p);
-// out = R^T acc.  Three launches: query_rotate_kernel (q_rot, once per sequence and
+// out = R^T acc.  Three launches: rotate_kernel in kv_rotate.hip (q_rot, once per sequence and
 // head), attention_mfma4_kernel (the context scan, below), attention_merge_kernel
 // (split merge, normalisation, rotate-back).
 //
@@ -53,6 +53,8 @@
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
+
+#include <cstring>
 
 #ifndef TW_EXP
 #define TW_EXP 0
@@ -107,26 +109,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const char* base, in
 }
 
 }  // namespace
-
-// q_rot[g][head][d] = (sum_k R[d][k] q[g][head][k]) * log2(e) / (sqrt(D) * alpha)
-// (kernels.cu:1671-1681, with the score scale of line 1707 and the table scale
-// folded in).  One workgroup of 128 threads per (sequence, head); fp32, k ascending.
-__global__ void __launch_bounds__(kHeadDim)
-query_rotate_kernel(AttnArgs a) {
-    __shared__ float q_s[kHeadDim];
-    const int head = blockIdx.x, g = blockIdx.y, d = threadIdx.x;
-    q_s[d] = (float)a.q[(long long)g * a.q_stride + (long long)head * kHeadDim + d];
-    __syncthreads();
-    const half8_t* rot8 = reinterpret_cast<const half8_t*>(a.rotation + d * kHeadDim);
-    float acc = 0.0f;
-#pragma unroll 4
-    for (int k8 = 0; k8 < kHeadDim / 8; k8++) {
-        half8_t rr = rot8[k8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) acc = __builtin_fmaf((float)rr[i], q_s[8 * k8 + i], acc);
-    }
-    a.qrot[((long long)g * a.num_heads + head) * a.ws_stride + d] = acc * (kLog2e * kInvSqrtD / kAlpha4);
-}
 
 template <bool PAGED, int R, int DEPTH>
 __global__ void __launch_bounds__(kMaxWaves * kWave, (DEPTH <= 1 ? 4 : 2))
@@ -507,7 +489,13 @@ static int scan_waves(const AttnArgs& a) {
     return waves;
 }
 
-bool prepare_attention_mfma(AttnArgs& a, hipStream_t s) {
+float attention_mfma_q_scale(int bits) {
+    (void)bits;
+    return kLog2e * kInvSqrtD / kAlpha4;   // score scale of kernels.cu:1707 in base 2, table scale undone
+}
+
+// Shape check; with rotate_query also q_rot = R q (kernels.cu:1671-1681) into the workspace.
+bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     const int R = a.num_heads / a.num_kv_heads;
     if (a.bits != 4) return false;
     if (R != 1 && R != 2 && R != 4) return false;
@@ -518,7 +506,22 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s) {
     if (items <= 0 || items > 0x7fffffff) return false;
     a.force_merge = 1;
     a.m_log2 = 1;
-    hipLaunchKernelGGL(query_rotate_kernel, dim3(a.num_heads, a.G), dim3(kHeadDim), 0, s, a);
+    if (rotate_query) {
+        RotArgs r;
+        memset(&r, 0, sizeof(r));
+        r.nseg = 1;
+        r.seg_src[0] = a.q;
+        r.seg_stride[0] = a.q_stride;
+        r.seg_heads[0] = a.num_heads;
+        r.seg_nvec[0] = a.G * a.num_heads;
+        r.seg_units[0] = (r.seg_nvec[0] + 15) / 16 * 8;
+        r.seg_kind[0] = 1;
+        r.rotation = a.rotation;
+        r.qrot = a.qrot;
+        r.qrot_stride = a.ws_stride;
+        r.q_scale = attention_mfma_q_scale(a.bits);
+        launch_rotate(r, a.bits, s);
+    }
     return true;
 }
 

@@ -24,7 +24,7 @@ std::atomic<int> g_variant{0};
 std::atomic<int> g_nsplit_override{0};
 
 constexpr int kMaxSplits = 64;
-constexpr long long kPagedBlockFloats = 64 * 130 + 128 + 4;  // per (sequence, head): partials + rotated query
+constexpr long long kPagedBlockFloats = 64 * (long long)kPartialFloats + 128 + 4;  // per (sequence, head): partials + rotated query
 constexpr int kMinChunk = 128;       // tokens
 constexpr int kTargetGroups = 2048;  // workgroups wanted per launch: 8 per CU on 256 CUs
 constexpr int kTargetItems = 512;    // (sequence, chunk) items wanted by the persistent MFMA scan: one per resident workgroup
@@ -118,7 +118,11 @@ struct Profiler {
     int used = 0;
 } g_prof;
 
-void run_attention(AttnArgs& a, hipStream_t s, const char* fn) {
+// query_done: q_rot is already in the workspace (the fused append + attention entry
+// rotates the query together with the appended rows).
+bool mfma_wanted(const AttnArgs& a) { return a.bits != 0 && g_variant.load() != 1; }
+
+void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done = false) {
     bool prof = g_prof.enabled.load() != 0 && g_prof.used < kProfSlots;
     if (prof) {
         while (g_prof.created <= g_prof.used) {
@@ -127,13 +131,14 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn) {
             g_prof.created++;
         }
     }
-    const int variant = g_variant.load();
-    const bool mfma = a.bits != 0 && variant != 1 && prepare_attention_mfma(a, s);
+    const bool mfma = mfma_wanted(a) && prepare_attention_mfma(a, s, !query_done);
     if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
     if (mfma) launch_attention_mfma_scan(a, s);
     else launch_attention_valu(a, s);
     if (prof) hipEventRecord(g_prof.stop[g_prof.used++], s);
-    launch_attention_merge(a, s);
+    if (a.nsplit > 1 || a.force_merge) {
+        if (!(g_variant.load() != 1 && launch_merge_rotate(a, s))) launch_attention_merge(a, s);
+    }
     check_launch(fn);
 }
 }  // namespace
@@ -187,6 +192,25 @@ void tw_paged_kv_cache_write_batch(tw_half* ck, tw_half* cv, const tw_half* k, c
     check_launch("tw_paged_kv_cache_write_batch");
 }
 
+static void fill_quant_segments(RotArgs& r, uint8_t* c0, tw_half* n0, const tw_half* s0, uint8_t* c1,
+                                tw_half* n1, const tw_half* s1, int nstreams, int nrows,
+                                int num_kv_heads, int kv_dim) {
+    uint8_t* c[2] = {c0, c1};
+    tw_half* n[2] = {n0, n1};
+    const tw_half* src[2] = {s0, s1};
+    for (int i = 0; i < nstreams; i++) {
+        int k = r.nseg++;
+        r.seg_src[k] = H(src[i]);
+        r.seg_stride[k] = kv_dim;
+        r.seg_heads[k] = num_kv_heads;
+        r.seg_nvec[k] = nrows * num_kv_heads;
+        r.seg_units[k] = (r.seg_nvec[k] + 15) / 16 * 8;
+        r.seg_kind[k] = 0;
+        r.seg_codes[k] = c[i];
+        r.seg_norms[k] = H(n[i]);
+    }
+}
+
 static void quantize_common(const char* fn, uint8_t* c0, tw_half* n0, const tw_half* s0,
                             uint8_t* c1, tw_half* n1, const tw_half* s1, int nstreams,
                             const tw_half* rotation, const int* positions, const int* block_table,
@@ -197,21 +221,36 @@ static void quantize_common(const char* fn, uint8_t* c0, tw_half* n0, const tw_h
         set_error(1, "%s: kv_dim=%d smaller than num_kv_heads*head_dim", fn, kv_dim);
         return;
     }
-    QuantArgs a;
-    memset(&a, 0, sizeof(a));
-    a.codes[0] = c0; a.norms[0] = H(n0); a.src[0] = H(s0);
-    a.codes[1] = c1; a.norms[1] = H(n1); a.src[1] = H(s1);
-    a.nstreams = nstreams;
-    a.rotation = H(rotation);
-    a.positions = positions;
-    a.block_table = block_table;
-    a.bt_stride = bt_stride;
-    a.seq_stride_rows = seq_stride_rows;
-    a.token_list = token_list;
-    a.nrows = nrows;
-    a.num_kv_heads = num_kv_heads;
-    a.kv_dim = kv_dim;
-    launch_turbo_quantize(a, bits, s);
+    if (g_variant.load() == 1) {   // vector-ALU kernel, kept for cross-checks
+        QuantArgs a;
+        memset(&a, 0, sizeof(a));
+        a.codes[0] = c0; a.norms[0] = H(n0); a.src[0] = H(s0);
+        a.codes[1] = c1; a.norms[1] = H(n1); a.src[1] = H(s1);
+        a.nstreams = nstreams;
+        a.rotation = H(rotation);
+        a.positions = positions;
+        a.block_table = block_table;
+        a.bt_stride = bt_stride;
+        a.seq_stride_rows = seq_stride_rows;
+        a.token_list = token_list;
+        a.nrows = nrows;
+        a.num_kv_heads = num_kv_heads;
+        a.kv_dim = kv_dim;
+        launch_turbo_quantize(a, bits, s);
+        check_launch(fn);
+        return;
+    }
+    RotArgs r;
+    memset(&r, 0, sizeof(r));
+    fill_quant_segments(r, c0, n0, s0, c1, n1, s1, nstreams, nrows, num_kv_heads, kv_dim);
+    r.rotation = H(rotation);
+    r.positions = positions;
+    r.block_table = block_table;
+    r.bt_stride = bt_stride;
+    r.seq_stride_rows = seq_stride_rows;
+    r.token_list = token_list;
+    r.num_kv_heads = num_kv_heads;
+    launch_rotate(r, bits, s);
     check_launch(fn);
 }
 
@@ -350,6 +389,55 @@ void launch_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const uint
     a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
     plan_splits(a, msl, msl);
     run_attention(a, s, "launch_turbo_gqa_attention_batch");
+}
+
+void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf,
+                                     const tw_half* v_buf, uint8_t* ck_q, uint8_t* cv_q,
+                                     tw_half* k_norms, tw_half* v_norms, const tw_half* rotation,
+                                     float* as, const int* pos, int msl, int G, int num_heads,
+                                     int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                     int bits, hipStream_t s) {
+    const char* fn = "tw_turbo_append_attention_batch";
+    if (!check_shape(fn, num_heads, num_kv_heads, head_dim) || !check_bits(fn, bits)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads,
+                num_kv_heads, bits, as);
+    a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    plan_splits(a, msl, msl);
+    // one rotation launch for the appended K and V rows and, when the MFMA scan will run,
+    // for the query as well
+    const int R = num_heads / num_kv_heads;
+    const bool fuse_q = mfma_wanted(a) && a.qrot && (R == 1 || R == 2 || R == 4) && bits == 4 &&
+                        (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0;
+    if (g_variant.load() == 1 || !fuse_q) {
+        tw_turbo_kv_append_batch(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotation, pos, msl, G,
+                                 num_kv_heads, head_dim, kv_dim, bits, s);
+        run_attention(a, s, fn);
+        return;
+    }
+    RotArgs r;
+    memset(&r, 0, sizeof(r));
+    fill_quant_segments(r, ck_q, k_norms, k_buf, cv_q, v_norms, v_buf, 2, G, num_kv_heads, kv_dim);
+    int k = r.nseg++;
+    r.seg_src[k] = H(q);
+    r.seg_stride[k] = q_dim;
+    r.seg_heads[k] = num_heads;
+    r.seg_nvec[k] = G * num_heads;
+    r.seg_units[k] = (r.seg_nvec[k] + 15) / 16 * 8;
+    r.seg_kind[k] = 1;
+    r.rotation = H(rotation);
+    r.positions = pos;
+    r.seq_stride_rows = msl;
+    r.num_kv_heads = num_kv_heads;
+    r.qrot = a.qrot;
+    r.qrot_stride = a.ws_stride;
+    r.q_scale = attention_mfma_q_scale(bits);
+    launch_rotate(r, bits, s);
+    run_attention(a, s, fn, /*query_done=*/true);
 }
 
 void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const uint8_t* ck_q,

@@ -137,17 +137,12 @@ void layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, con
                                    e->batch_msl, e->G, m.num_heads, m.num_kv_heads, m.head_dim,
                                    e->q_dim(), e->kv_dim(), s);
     } else {
-        tw_turbo_kv_append_batch((uint8_t*)e->cache[layer][0], (tw_half*)e->cache[layer][2],
-                                 (uint8_t*)e->cache[layer][1], (tw_half*)e->cache[layer][3], k, v,
-                                 e->d_rotation, e->d_positions, e->batch_msl, e->G, m.num_kv_heads,
-                                 m.head_dim, e->kv_dim(), e->kv_bits, s);
-        launch_turbo_gqa_attention_batch(out, q, (const uint8_t*)e->cache[layer][0],
-                                         (const uint8_t*)e->cache[layer][1],
-                                         (const tw_half*)e->cache[layer][2],
-                                         (const tw_half*)e->cache[layer][3], e->d_rotation,
-                                         e->attn_scores, e->d_positions, e->batch_msl, e->G,
-                                         m.num_heads, m.num_kv_heads, m.head_dim, e->q_dim(),
-                                         e->kv_dim(), e->kv_bits, s);
+        tw_turbo_append_attention_batch(out, q, k, v, (uint8_t*)e->cache[layer][0],
+                                        (uint8_t*)e->cache[layer][1], (tw_half*)e->cache[layer][2],
+                                        (tw_half*)e->cache[layer][3], e->d_rotation, e->attn_scores,
+                                        e->d_positions, e->batch_msl, e->G, m.num_heads,
+                                        m.num_kv_heads, m.head_dim, e->q_dim(), e->kv_dim(),
+                                        e->kv_bits, s);
     }
 }
 

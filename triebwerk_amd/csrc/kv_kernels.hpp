@@ -33,6 +33,31 @@ void launch_kv_write(half_t* ck, half_t* cv, const half_t* k, const half_t* v,
 void launch_turbo_quantize(const QuantArgs& a, int bits, hipStream_t s);
 void launch_increment(int* positions, int G, hipStream_t s);
 
+// ---------------------------------------------------------------- rotation on the matrix cores
+struct RotArgs {
+    int nseg;                    // up to 3 segments: K rows, V rows (quantize), Q rows (rotate only)
+    const half_t* seg_src[3];    // fp16 source, row r at src + r * stride
+    long long seg_stride[3];     // halves per source row
+    int seg_heads[3];            // head vectors per source row
+    int seg_nvec[3];             // rows * heads
+    int seg_units[3];            // work units = ceil(nvec / 16) * 8
+    int seg_kind[3];             // 0 = quantize into the cache, 1 = query rotation
+    uint8_t* seg_codes[3];
+    half_t* seg_norms[3];
+    const half_t* rotation;
+    const int* positions;
+    const int* block_table;
+    int bt_stride;
+    long long seq_stride_rows;
+    int token_list;              // 1: source row r goes to cache row positions[r] of sequence 0
+    int num_kv_heads;
+    float* qrot;                 // query output: vector v at qrot + v * qrot_stride (fp32)
+    long long qrot_stride;
+    float q_scale;
+};
+
+void launch_rotate(const RotArgs& a, int bits, hipStream_t s);
+
 // ---------------------------------------------------------------- attention
 enum PosMode { kPosArray = 0, kPosScalar = 1, kPosIota = 2 };
 
@@ -62,13 +87,15 @@ struct AttnArgs {
     int m_log2;             // partial maxima are in base-2 units
 };
 
-constexpr int kPartialFloats = kHeadDim + 2;  // acc[128], running max, running sum
+constexpr int kPartialFloats = kHeadDim + 4;  // acc[128], running max, running sum, 2 pad (16-byte rows)
 
 void launch_attention_valu(const AttnArgs& a, hipStream_t s);
 void launch_attention_merge(const AttnArgs& a, hipStream_t s);
+bool launch_merge_rotate(const AttnArgs& a, hipStream_t s);   // MFMA merge + rotate-back; false = not applicable
 // MFMA path, two steps so that the scan kernel can be timed alone:
 // prepare = shape check + query rotation (false = shape not covered), then the scan.
-bool prepare_attention_mfma(AttnArgs& a, hipStream_t s);
+bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query);
+float attention_mfma_q_scale(int bits);
 void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);
 
 }  // namespace twkv

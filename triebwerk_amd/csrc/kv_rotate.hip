@@ -1,0 +1,247 @@
+// kv_rotate.hip -- the 128x128 rotation on the matrix cores (gfx950), for
+//   - the TurboQuant compressed append: y = R (x / |x|), bin search, pack, norm
+//     (turbo_kv_quantize{,_batch}_kernel, kernels.cu:1482-1636), K and V rows, and
+//   - the query rotation q_rot = R q of the compressed attention (kernels.cu:1671-1681),
+// all in one launch (any subset).
+//
+// Bit-exactness of the append.  The reference accumulates each output coordinate as
+// one fp32 fused-multiply-add chain over k = 0..127.  v_mfma_f32_16x16x4_f32 chained
+// over k-blocks of 4 produces the same bits: inside one instruction the four k of the
+// block are accumulated in ascending order with fused multiply-adds, and blocks chain
+// through the accumulator (checked on hardware against a host fmaf chain: 0 of 4096
+// outputs differ).  The sum of squares keeps the reference's reduction tree
+// (kernels.cu:1509-1520): offsets 16, 8 and 4 of the 32-lane shuffle tree only combine
+// coordinates that are congruent mod 4, which one lane owns; offsets 2 and 1 and the
+// combination of the four 32-coordinate groups, (s0+s2)+(s1+s3), are done across lanes.
+//
+// Mapping.  One wave = one work unit = (16 vectors) x (16 output coordinates):
+//   A operand = R rows   : lane (i = lane%16, kk = lane/16) holds R[d0+i][4s+kk], s = 0..31
+//   B operand = vectors  : the same lane holds u[v0+i][4s+kk]
+//   D[16 x 16]           : lane holds y[d0 + 4*(lane/16) + r][v0 + lane%16], r = 0..3
+// A wave needs nothing from any other wave (no LDS, no barrier), so a launch is
+// ceil(vectors/16) * 8 independent single-wave workgroups that spread over the chip;
+// that matters because these launches are small (a few thousand vectors) and
+// latency-bound.
+
+#include "kv_common.hpp"
+#include "kv_kernels.hpp"
+
+namespace twkv {
+
+namespace {
+
+// fp16 at index (4s + kk) of a row held as 16 x (8 halves): s = 2*q + e picks dword
+// (2e + kk/2) of 16-byte piece q, half kk%2.
+__device__ __forceinline__ float pick_half(const uint4& piece, int e, int kk) {
+    uint32_t lo = e ? piece.z : piece.x;
+    uint32_t hi = e ? piece.w : piece.y;
+    uint32_t w = (kk & 2) ? hi : lo;
+    w = (kk & 1) ? (w >> 16) : (w & 0xffffu);
+    union { uint16_t u; half_t h; } cv;
+    cv.u = (uint16_t)w;
+    return (float)cv.h;
+}
+
+}  // namespace
+
+template <int BITS>
+__global__ void __launch_bounds__(kWave)
+rotate_kernel(RotArgs a) {
+    const int lane = threadIdx.x;
+    const int i16 = lane & 15, kk = lane >> 4;
+
+    // ---- which unit
+    int unit = blockIdx.x;
+    int seg = 0;
+    while (seg < a.nseg - 1 && unit >= a.seg_units[seg]) { unit -= a.seg_units[seg]; seg++; }
+    const int dblk = unit & 7;
+    const int vtile = unit >> 3;
+    const int nvec = a.seg_nvec[seg];
+    const int heads = a.seg_heads[seg];                  // head vectors per source row
+    const bool is_query = a.seg_kind[seg] != 0;
+    const int v = vtile * 16 + i16;
+    const int vc = v < nvec ? v : nvec - 1;              // clamp loads, mask stores
+    const int row = vc / heads, head = vc - row * heads;
+
+    // ---- operands: R row d0 + i16 and source vector v, both as 16 pieces of 8 halves
+    const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (dblk * 16 + i16) * kHeadDim);
+    const uint4* xsrc = reinterpret_cast<const uint4*>(a.seg_src[seg] + (long long)row * a.seg_stride[seg] +
+                                                       (long long)head * kHeadDim);
+    float rv[32], xv[32];
+#pragma unroll
+    for (int q = 0; q < 16; q++) {
+        uint4 rp = rsrc[q], xp = xsrc[q];
+        rv[2 * q] = pick_half(rp, 0, kk);
+        rv[2 * q + 1] = pick_half(rp, 1, kk);
+        xv[2 * q] = pick_half(xp, 0, kk);
+        xv[2 * q + 1] = pick_half(xp, 1, kk);
+    }
+
+    float n2 = 0.0f;
+    if (!is_query) {
+        // sum of squares in the reference's order: xv[s] is coordinate 4s + kk; group w holds s = 8w..8w+7
+        float sgrp[4];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            float t[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) t[j] = xv[8 * w + j] * xv[8 * w + j];
+            // offset 16: positions i and i+16 are local j and j+4; offset 8: j and j+2; offset 4: j and j+1
+            float a0 = t[0] + t[4], a1 = t[1] + t[5], a2 = t[2] + t[6], a3 = t[3] + t[7];
+            float b0 = a0 + a2, b1 = a1 + a3;
+            float c = b0 + b1;                                   // c_kk of the tree
+            float d = c + __shfl_xor(c, 32, 64);                 // offset 2: c0+c2 | c1+c3
+            sgrp[w] = d + __shfl_xor(d, 16, 64);                 // offset 1: d0+d1
+        }
+        n2 = (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
+        const float inv = 1.0f / sqrtf(n2 + 1e-12f);
+#pragma unroll
+        for (int s = 0; s < 32; s++) xv[s] *= inv;
+    }
+
+    // ---- y[d][v] = sum_k R[d][k] u[v][k], k ascending
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 32; s++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(rv[s], xv[s], acc, 0, 0, 0);
+
+    if (is_query) {
+        if (v < nvec) {
+            float* dst = a.qrot + (long long)v * a.qrot_stride + dblk * 16 + 4 * kk;
+            float4 o = {acc[0] * a.q_scale, acc[1] * a.q_scale, acc[2] * a.q_scale, acc[3] * a.q_scale};
+            *reinterpret_cast<float4*>(dst) = o;
+        }
+        return;
+    }
+
+    // ---- quantize the lane's 4 consecutive coordinates d0 + 4kk .. +3 and pack (low field first)
+    uint32_t packed = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) packed |= (uint32_t)turbo_quantize(acc[r], BITS) << (r * BITS);
+    // gather the four lanes of a vector (kk = 0..3) into the kk == 0 lane
+    constexpr int PB = 4 * BITS;                                  // bits per lane
+    uint32_t p1 = (uint32_t)__shfl((int)packed, i16 + 16, 64);
+    uint32_t p2 = (uint32_t)__shfl((int)packed, i16 + 32, 64);
+    uint32_t p3 = (uint32_t)__shfl((int)packed, i16 + 48, 64);
+    if (kk == 0 && v < nvec) {
+        long long crow;
+        if (a.token_list) crow = a.positions[row];               // sequence 0, kernels.cu:1499, 1553
+        else crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, a.positions[row]);
+        constexpr int BPH = kHeadDim * BITS / 8;                  // bytes per head: 64 or 32
+        uint8_t* dst = a.seg_codes[seg] + (crow * a.num_kv_heads + head) * BPH + dblk * (2 * BITS);
+        if (BITS == 4) {
+            uint2 o = {packed | (p1 << PB), p2 | (p3 << PB)};
+            *reinterpret_cast<uint2*>(dst) = o;                   // 16 codes = 8 bytes
+        } else {
+            *reinterpret_cast<uint32_t*>(dst) = packed | (p1 << PB) | (p2 << (2 * PB)) | (p3 << (3 * PB));
+        }
+        if (dblk == 0) a.seg_norms[seg][crow * a.num_kv_heads + head] = (half_t)sqrtf(n2 + 1e-12f);
+    }
+}
+
+void launch_rotate(const RotArgs& a, int bits, hipStream_t s) {
+    int units = 0;
+    for (int i = 0; i < a.nseg; i++) units += a.seg_units[i];
+    if (units <= 0) return;
+    if (bits == 4) hipLaunchKernelGGL(rotate_kernel<4>, dim3(units), dim3(kWave), 0, s, a);
+    else hipLaunchKernelGGL(rotate_kernel<2>, dim3(units), dim3(kWave), 0, s, a);
+}
+
+// ---------------------------------------------------------------- split merge + rotate-back
+// out[g][head][d] = sum_k R[k][d] * o[k],  o = (sum_c f_c acc_c) / (sum_c f_c l_c + 1e-8),
+// f_c = exp(m_c - max_c m_c): the log-sum-exp merge of the split partials, the
+// normalisation of kernels.cu:1746 and the rotate-back of kernels.cu:1769-1775.
+// A workgroup of 8 waves takes 16 (sequence, head) vectors: all threads merge into LDS,
+// then wave w produces output coordinates [16w, 16w+16) with 32 fp32 MFMAs
+// (v_mfma_f32_16x16x4_f32; A = merged vectors from LDS, B = a column block of R).
+constexpr int kMergeVecs = 16;
+constexpr int kMergeStride = kHeadDim + 4;     // floats per LDS row: conflict-free 16-byte reads
+
+__global__ void __launch_bounds__(8 * kWave)
+merge_rotate_kernel(AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) float o_s[kMergeVecs][kMergeStride];
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave, lane = tid % kWave;
+    const int i16 = lane & 15, kk = lane >> 4;
+    const int total = a.G * a.num_heads;
+    const int v0 = blockIdx.x * kMergeVecs;
+
+    // B operand first (its loads overlap the merge): R[32kk + s][16*wave + i16], s = 0..31
+    uint16_t rb[32];
+    {
+        const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.rotation) + (32 * kk) * kHeadDim + 16 * wave + i16;
+#pragma unroll
+        for (int s = 0; s < 32; s++) rb[s] = rp[s * kHeadDim];
+    }
+
+    // ---- merge: thread -> (vector tid/32, coordinates 4*(tid%32) .. +3)
+    {
+        const int vl = tid >> 5, k4 = (tid & 31) * 4;
+        const int vv = min(v0 + vl, total - 1);
+        const int g = vv / a.num_heads;
+        int n;
+        if (a.pos_mode == kPosArray) n = a.positions[g] + 1;
+        else if (a.pos_mode == kPosScalar) n = a.pos_scalar + 1;
+        else n = g + 1;
+        const float* part = a.ws + (long long)vv * a.ws_stride;
+        float mg = -1e30f;
+        for (int c = 0; c < a.nsplit; c++) {
+            int t0, t1;
+            chunk_range(n, c, a.nsplit, t0, t1);
+            if (t0 < t1) mg = fmaxf(mg, part[(long long)c * kPartialFloats + kHeadDim]);
+        }
+        float lsum = 0.0f;
+        float4 av = {0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < a.nsplit; c++) {
+            int t0, t1;
+            chunk_range(n, c, a.nsplit, t0, t1);
+            if (t0 >= t1) continue;
+            const float* pc = part + (long long)c * kPartialFloats;
+            float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
+            lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);
+            float4 p4 = *reinterpret_cast<const float4*>(pc + k4);
+            av.x = __builtin_fmaf(p4.x, f, av.x);
+            av.y = __builtin_fmaf(p4.y, f, av.y);
+            av.z = __builtin_fmaf(p4.z, f, av.z);
+            av.w = __builtin_fmaf(p4.w, f, av.w);
+        }
+        const float inv = 1.0f / (lsum + 1e-8f);
+        float4 o4 = {av.x * inv, av.y * inv, av.z * inv, av.w * inv};
+        *reinterpret_cast<float4*>(&o_s[vl][k4]) = o4;
+    }
+    __syncthreads();
+
+    // ---- out[vector][d] = sum_k o[vector][k] R[k][d]; lane group kk owns k in [32kk, 32kk+32)
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const float* orow = &o_s[i16][32 * kk];
+#pragma unroll
+    for (int s4 = 0; s4 < 8; s4++) {
+        float4 o4 = *reinterpret_cast<const float4*>(orow + 4 * s4);
+        const float ov[4] = {o4.x, o4.y, o4.z, o4.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            union { uint16_t u; half_t h; } cv;
+            cv.u = rb[4 * s4 + j];
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ov[j], (float)cv.h, acc, 0, 0, 0);
+        }
+    }
+    // lane holds out[vector 4kk + r][d = 16*wave + i16]
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int vv = v0 + 4 * kk + r;
+        if (vv < total) {
+            const int g = vv / a.num_heads, head = vv - g * a.num_heads;
+            a.out[(long long)g * a.q_stride + (long long)head * kHeadDim + 16 * wave + i16] = (half_t)acc[r];
+        }
+    }
+}
+
+bool launch_merge_rotate(const AttnArgs& a, hipStream_t s) {
+    if (a.bits == 0 || !a.ws) return false;
+    if ((reinterpret_cast<uintptr_t>(a.ws) & 15u) != 0 || (a.ws_stride & 3) != 0) return false;
+    const int total = a.G * a.num_heads;
+    if (total <= 0) return true;
+    hipLaunchKernelGGL(merge_rotate_kernel, dim3((total + kMergeVecs - 1) / kMergeVecs), dim3(8 * kWave), 0, s, a);
+    return true;
+}
+
+}  // namespace twkv

@@ -148,6 +148,20 @@ def tw_turbo_kv_append_batch(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotatio
     _done(lib)
 
 
+def tw_turbo_append_attention_batch(out, q, k_buf, v_buf, ck_q, cv_q, k_norms, v_norms, rotation, scratch,
+                                    pos, msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits,
+                                    stream=None):
+    lib = _lib.load()
+    lib.tw_turbo_append_attention_batch(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(k_buf, "f16", "k_buf"),
+                                        _ptr(v_buf, "f16", "v_buf"), _ptr(ck_q, "u8", "ck_q"),
+                                        _ptr(cv_q, "u8", "cv_q"), _ptr(k_norms, "f16", "k_norms"),
+                                        _ptr(v_norms, "f16", "v_norms"), _ptr(rotation, "f16", "rotation"),
+                                        _ptr(scratch, "f32", "as"), _ptr(pos, "i32", "pos"), msl, G,
+                                        num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits,
+                                        _stream(stream))
+    _done(lib)
+
+
 def tw_paged_kv_cache_write_batch(ck, cv, k, v, positions, block_table, bt_stride, G, kv_dim,
                                   stream=None):
     lib = _lib.load()
