@@ -269,15 +269,11 @@ attention_merge_kernel(AttnArgs a) {
     const float* part = a.ws + ((long long)g * a.num_heads + head) * a.ws_stride;
     float mg = kNegBig;
     for (int cidx = 0; cidx < a.nsplit; cidx++) {
-        int t0, t1;
-        chunk_range(n, cidx, a.nsplit, t0, t1);
-        if (t0 < t1) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
+        if (chunk_nonempty(n, cidx, a.nsplit)) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
     }
     float lsum = 0.0f, av = 0.0f;
     for (int cidx = 0; cidx < a.nsplit; cidx++) {
-        int t0, t1;
-        chunk_range(n, cidx, a.nsplit, t0, t1);
-        if (t0 >= t1) continue;                 // no workgroup wrote this slot
+        if (!chunk_nonempty(n, cidx, a.nsplit)) continue;   // no workgroup wrote this slot
         const float* pc = part + (long long)cidx * kPartialFloats;
         float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
         lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);

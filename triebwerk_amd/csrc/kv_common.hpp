@@ -77,10 +77,16 @@ __device__ __forceinline__ long long cache_row(const int* __restrict__ block_tab
 // whatever max_seq_len the caller allocated.  Empty (t0 >= t1) when n has fewer tiles
 // than nsplit.
 __device__ __forceinline__ void chunk_range(int n, int c, int nsplit, int& t0, int& t1) {
-    const long long tiles = (n + 31) >> 5;
-    t0 = 32 * (int)((c * tiles) / nsplit);
-    int e = 32 * (int)(((c + 1) * tiles) / nsplit);
+    const unsigned tiles = (unsigned)(n + 31) >> 5;             // tiles * nsplit < 2^32 (nsplit <= 64)
+    t0 = 32 * (int)(((unsigned)c * tiles) / (unsigned)nsplit);
+    int e = 32 * (int)(((unsigned)(c + 1) * tiles) / (unsigned)nsplit);
     t1 = e < n ? e : n;
+}
+// Does chunk c hold any token?  Always when the sequence has at least nsplit tiles.
+__device__ __forceinline__ bool chunk_nonempty(int n, int c, int nsplit) {
+    const unsigned tiles = (unsigned)(n + 31) >> 5;
+    if (tiles >= (unsigned)nsplit) return true;
+    return ((unsigned)(c + 1) * tiles) / (unsigned)nsplit > ((unsigned)c * tiles) / (unsigned)nsplit;
 }
 
 __device__ __forceinline__ float wave_max(float v) {

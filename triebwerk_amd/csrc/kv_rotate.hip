@@ -185,16 +185,12 @@ merge_rotate_kernel(AttnArgs a) {
         const float* part = a.ws + (long long)vv * a.ws_stride;
         float mg = -1e30f;
         for (int c = 0; c < a.nsplit; c++) {
-            int t0, t1;
-            chunk_range(n, c, a.nsplit, t0, t1);
-            if (t0 < t1) mg = fmaxf(mg, part[(long long)c * kPartialFloats + kHeadDim]);
+            if (chunk_nonempty(n, c, a.nsplit)) mg = fmaxf(mg, part[(long long)c * kPartialFloats + kHeadDim]);
         }
         float lsum = 0.0f;
         float4 av = {0.f, 0.f, 0.f, 0.f};
         for (int c = 0; c < a.nsplit; c++) {
-            int t0, t1;
-            chunk_range(n, c, a.nsplit, t0, t1);
-            if (t0 >= t1) continue;
+            if (!chunk_nonempty(n, c, a.nsplit)) continue;
             const float* pc = part + (long long)c * kPartialFloats;
             float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
             lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);
