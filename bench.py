@@ -44,6 +44,11 @@ WORKLOADS = {
 }
 BYTES_HEAD = {0: 256, 4: 66, 2: 34}  # per (token, kv head): fp16 row | codes + fp16 norm
 
+# HBM bytes per launch of the context-scanning kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# on this file's own run (counter KiB scaled by what `--copy-calibration` reads for a copy of
+# known size); the summaries are profiles/scan_kv{4,2,16}_target_pmc.txt.  Keyed by (workload, kv_bits).
+MEASURED_TRAFFIC_BYTES = {}
+
 
 def algorithmic_bytes(n_tokens_total: int, G: int, L: int, H: int, Hk: int, kv_bits: int, with_append: bool) -> int:
     """Bytes one step must move, each cache byte counted once per step (not once per query head)."""
@@ -77,7 +82,7 @@ def fill_caches(eng, L, kv_bits, seed):
                 t.copy_((11.3 + 0.7 * torch.randn(t.shape, generator=gen, device="cuda")).to(torch.float16))
 
 
-def cpu_baseline(w, kv_bits, seconds_budget=20.0):
+def cpu_baseline(w, kv_bits, seconds_budget=15.0):
     """The CPU oracle (a restatement of the reference kernels, oracle/kv_oracle.cpp) on a
     bounded sample of the workload: one layer, as many sequences as fit the time budget."""
     import gen
@@ -116,9 +121,14 @@ def cpu_baseline(w, kv_bits, seconds_budget=20.0):
     S2 = int(max(S, min(w["G"], seconds_budget / max(per_seq, 1e-9))))
     if S2 > S:
         t, S = run(S2), S2
-    tokens_per_s = S / (t * w["L"])   # one layer measured; a step needs L of them
+    # more layers of the same sample until the budget is used (never more than the workload has)
+    layers = 1
+    while layers < w["L"] and t + t / layers < seconds_budget:
+        t += run(S)
+        layers += 1
+    tokens_per_s = S * layers / (t * w["L"])   # `layers` layers measured; a step needs L of them
     return dict(value=tokens_per_s, unit="tokens/s", cores=threads, kind="port",
-                sample=f"1 of {w['L']} layers x {S} of {w['G']} sequences at context {ctx}, "
+                sample=f"{layers} of {w['L']} layers x {S} of {w['G']} sequences at context {ctx}, "
                        f"{t:.2f} s of CPU time, scaled linearly; OpenMP over (sequence, head), "
                        f"{os.cpu_count()} logical CPUs visible")
 
@@ -137,7 +147,20 @@ def main():
     ap.add_argument("--ctx", type=int, default=None, help="override the workload's context length")
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--layers", type=int, default=None, help="override the workload's layer count")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="only run a plain device-to-device copy of this many MiB five times (reference for the "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
+    if args.copy_calibration:
+        import torch
+        n = args.copy_calibration << 20
+        src = torch.full((n,), 7, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": n, "copies": 5, "reads_bytes_each": n, "writes_bytes_each": n}))
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; sharding is by sequence or KV head with no exchange "
               "inside the path, and is not implemented. Use --gpus 1.", file=sys.stderr)
@@ -261,7 +284,7 @@ def main():
             "frac": achieved / HBM_PEAK_GBS,
             "launch_ms": kern_ms,
             "launch_algorithmic_MB": launch_bytes * 1e-6,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, kv_bits)) if not overridden else None,
         },
     }
     if not args.no_cpu:

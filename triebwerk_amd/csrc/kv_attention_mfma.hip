@@ -1,13 +1,14 @@
-// kv_attention_mfma.hip -- GQA decode attention over the 4-bit compressed cache
-// for gfx950: codes are expanded to fp16 centroids in registers and the two
+// kv_attention_mfma.hip -- GQA decode attention over the 4-bit and 2-bit compressed
+// caches for gfx950: codes are expanded to fp16 centroids in registers and the two
 // contractions (q.K^T and P.V) run on the matrix cores.
 //
 // Same mathematics as turbo_gqa_attention_batch_kernel of the reference
 // (kernels.cu:1641-1776): q_rot = R q; s_p = (q_rot . c(K codes_p)) * kn_p / sqrt(D);
 // softmax over p <= pos with "+1e-8" in the denominator; acc = sum_p w_p vn_p c(V codes_p);
 // out = R^T acc.  Three launches: rotate_kernel in kv_rotate.hip (q_rot, once per sequence and
-// head), attention_mfma4_kernel (the context scan, below), attention_merge_kernel
-// (split merge, normalisation, rotate-back).
+// head), attention_mfma_kernel (the context scan, below), merge_rotate_kernel
+// (split merge, normalisation, rotate-back).  The mapping is described for 4-bit codes;
+// the 2-bit differences follow it.
 //
 // Why MFMA for a bandwidth-bound scan: at 5.6 TB/s of 4-bit codes one CU must
 // consume ~18 codes per clock for K and V together, and with two query heads per
@@ -16,8 +17,9 @@
 // MFMA leaves one v_perm_b32 (LDS address) and one ds_read_b32 per BYTE of codes.
 //
 // Mapping (one wave = one KV head of one sequence, 32 tokens per iteration):
-//   K: lane (t = lane%16, kg = lane/16) loads 16 bytes = dims [32kg, 32kg+32) of
-//      token t.  Dword j of it is the B operand of MFMA j (v_mfma_f32_16x16x32_f16),
+//   K: lane (t = lane%16, kg = lane/16) holds 16 bytes = dims [32kg, 32kg+32) of
+//      token t (loaded by lane 4t + kg, so that adjacent lanes read adjacent bytes, and
+//      moved with ds_bpermute).  Dword j of it is the B operand of MFMA j (v_mfma_f32_16x16x32_f16),
 //      columns = tokens; the A operand holds q_rot for the GQA group's heads in the
 //      matching dimension order, rows = heads.  Result S[head][token]: a lane holds
 //      the scores of ONE token (its lane%16) for the group's heads.
@@ -38,9 +40,12 @@
 //   addressing: every load is (scalar base of the 16-token sub-tile) + (per-lane
 //      offset fixed for the whole kernel); pages of the paged layout only change
 //      the scalar base.
-//   scheduling: workgroups are persistent (two per CU) and walk a list of
-//      (sequence, chunk, head group) items, so the 64 KB table is built once per
-//      workgroup; waves never synchronise after that.
+//   scheduling: one persistent workgroup of 16 waves per CU.  Its waves form two groups of
+//      8 (one KV head per wave); each group walks its own list of (sequence, chunk, head
+//      group) items, so the 64 KB table is built once per CU and waves never synchronise
+//      after that.  Measured: the waves in the upper wave slots of a CU (the second group,
+//      or a second workgroup) run ~5 % slower than the lower ones whatever their s_setprio,
+//      so the kernel ends with half of each CU idle for the last ~5 % of its time.
 //   precision: fp16 operands would cost ~5e-4 relative error each for q_rot and for
 //      the probabilities.  Both are split into hi + lo fp16 parts that ride in MFMA
 //      rows the GQA group leaves empty (head n -> row n and n+8), so the split costs
@@ -48,37 +53,47 @@
 //      The centroid table is stored as fp16(alpha * c) with alpha chosen so that all
 //      eight magnitudes round with <= 1.1e-4 relative error (3.6e-4 without it);
 //      1/alpha is folded into q_rot and into the final accumulator.
+//   2-bit codes: a cache row of one head is 32 bytes.  K: a lane loads 8 bytes (the same 32
+//      dims).  The table maps a byte (4 codes) to 4 fp16 centroids, 8 bytes per entry and 32
+//      replicas, read with ds_read_b64 (conflict free per half wave); entry order is
+//      (code0, code2, code1, code3), matched by the order of q_rot in the A operand, because
+//      that order is what V needs.  V: the 8 dims of a lane are 2 bytes per token; lanes n and
+//      n^1 share dwords, so each loads the dword of two of the four tokens and they trade
+//      halves with one DPP move.  Index bytes hold (token a dims d,d+1 | token b dims d,d+1),
+//      so one look-up returns the B-operand dwords (a,b) of dim d and of dim d+1.
 // The partial (acc[128], max, sum) per (sequence, head, chunk) goes to the split
-// workspace; attention_merge_kernel combines, normalises and rotates back.
+// workspace; merge_rotate_kernel combines, normalises and rotates back.
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 
 #include <cstring>
 
-#ifndef TW_EXP
-#define TW_EXP 0
-#endif
-#ifndef TW_DEPTH
-#define TW_DEPTH 1
-#endif
-#define TW_LUT(addr) ((TW_EXP == 3 || TW_EXP == 4) ? ((uint32_t)(addr) & 0x33ffu) : *reinterpret_cast<const uint32_t*>(tab_lane + (addr)))
-#define TW_LUTK(addr) ((TW_EXP == 1) ? ((uint32_t)(addr) & 0x33ffu) : TW_LUT(addr))
-#define TW_LUTV(addr) ((TW_EXP == 2) ? ((uint32_t)(addr) & 0x33ffu) : TW_LUT(addr))
-
 namespace twkv {
 
 namespace {
 
-constexpr int kMaxWaves = 8;          // KV heads per workgroup
+constexpr int kGroupWaves = 8;        // KV heads (waves) that walk one item together
+constexpr int kMaxWaves = 16;         // waves per workgroup: one workgroup per CU, two groups
 constexpr int kMaxGroup = 4;          // query heads per KV head handled by this kernel
 constexpr int kTableWords = 256 * 64; // 64 KB
 constexpr float kNegBig = -1e30f;
 // fp16(kAlpha4 * c) has max relative rounding error 1.05e-4 over the 4-bit table
 // (exhaustive search over the fp32 values of one octave).
 constexpr float kAlpha4 = 19.391284942626953f;
+// the same for the 2-bit table: 1.1e-7
+constexpr float kAlpha2 = 25.46918296813965f;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kInvSqrtD = 0.08838834764831845f;
+// Tiles of loads in flight per wave.  Deeper is only safe while nothing spills: a spilled
+// register is reloaded through the same in-order memory counter as the prefetched tiles,
+// so every reload waits for all of them.
+#ifndef TW_DEPTH4
+#define TW_DEPTH4 1
+#endif
+#ifndef TW_DEPTH2
+#define TW_DEPTH2 1
+#endif
 
 __device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
     if (a.pos_mode == kPosArray) return a.positions[g];
@@ -110,9 +125,13 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const char* base, in
 
 }  // namespace
 
-template <bool PAGED, int R, int DEPTH>
-__global__ void __launch_bounds__(kMaxWaves * kWave, (DEPTH <= 1 ? 4 : 2))
-attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
+template <bool PAGED, int R, int BITS, int DEPTH>
+__global__ void __launch_bounds__(kMaxWaves * kWave)
+attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves) {
+    constexpr int KW = BITS;        // dwords of K codes per lane and sub-tile (32 dims of one token)
+    constexpr int VW = BITS;        // dwords of V codes per lane and sub-tile
+    constexpr uint32_t kHeadBytes = BITS * 16;   // bytes of one head in a cache row
+    constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
     // per wave: P[row][k] as fp16, rows 0..R-1 = heads, rows 8..8+R-1 = rounding remainders
     __shared__ __attribute__((aligned(16))) half_t p_s[kMaxWaves][16][32];
@@ -121,18 +140,33 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     const int nthreads = blockDim.x;
     const int wave = uniform(tid / kWave), lane = tid % kWave;   // wave index is wave-uniform: keep it scalar
     const int ln = lane & 15, kg = lane >> 4;
-    const int waves = nthreads / kWave;
+    // The workgroup's waves form groups of group_waves (one KV head each); a group walks its
+    // own list of items and never synchronises with the others once the table is built.
+    const int grp = wave / group_waves, wv = wave % group_waves;
+    const int ngroups = (nthreads / kWave) / group_waves;
     const int Hk = a.num_kv_heads;
 
     const char* tab_lane = reinterpret_cast<const char*>(tab_s);
-    const uint32_t lane4 = (uint32_t)lane * 4u;
-    const uint32_t kvp = (uint32_t)Hk * 64u;           // bytes per cache row (all heads)
+    // byte offset of this lane's replica inside a table entry (entries are 256 bytes apart)
+    const uint32_t lane_rep = BITS == 4 ? (uint32_t)lane * 4u : (uint32_t)(lane & 31) * 8u;
+    const uint32_t kvp = (uint32_t)Hk * kHeadBytes;    // bytes per cache row (all heads)
     const uint32_t nrow = (uint32_t)Hk * 2u;           // bytes per norm row
     // per-lane byte offsets inside a 16-token sub-tile, fixed for the whole kernel
-    const uint32_t koff = (uint32_t)ln * kvp + 16u * (uint32_t)kg;
-    uint32_t voff[4];
+    // K is loaded with lane l on token l/4, quarter l%4 of the head's row, so that four adjacent
+    // lanes read one contiguous piece (a quarter of the cache accesses of loading in operand
+    // order); ds_bpermute then moves it to operand order: lane (ln, kg) takes token ln, quarter kg.
+    const uint32_t koff = (uint32_t)(lane >> 2) * kvp + (kHeadBytes / 4) * (uint32_t)(lane & 3);
+    const int ksrc = 4 * (4 * ln + kg);                // byte address of the source lane for ds_bpermute
+    uint32_t voff[VW];
 #pragma unroll
-    for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(4 * kg + i) * kvp + 4u * (uint32_t)ln;
+    for (int i = 0; i < VW; i++) {
+        if (BITS == 4) voff[i] = (uint32_t)(4 * kg + i) * kvp + 4u * (uint32_t)ln;
+        else voff[i] = (uint32_t)(4 * kg + 2 * i + (ln & 1)) * kvp + 4u * (uint32_t)(ln >> 1);
+    }
+    // 2-bit V: which halves of its two dwords a lane keeps and which it hands to lane ^ 1
+    const bool odd = (ln & 1) != 0;
+    const uint32_t sel_keep = odd ? 0x07060302u : 0x05040100u;
+    const uint32_t sel_send = odd ? 0x05040100u : 0x07060302u;
     const uint32_t sub_bytes = 16u * kvp;              // sub-tile b follows sub-tile a when contiguous
     // After the sub-tile swap a lane owns token ln of sub-tile (kg >> 1); lanes with odd kg idle.
     const int my_sub = kg >> 1;
@@ -143,113 +177,173 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     const uint4* p_r = reinterpret_cast<const uint4*>(&p_s[wave][ln][8 * kg]);
     constexpr float kRaise = 5.0f;                     // raise the running max only past 2^5
 
-    bool table_ready = false;
-    for (int item = blockIdx.x; item < total_items; item += gridDim.x) {
+    auto lut32 = [&](uint32_t addr) -> uint32_t { return *reinterpret_cast<const uint32_t*>(tab_lane + addr); };
+    auto lut64 = [&](uint32_t addr) -> uint2 { return *reinterpret_cast<const uint2*>(tab_lane + addr); };
+
+    // ---- state of the item in hand (wave-uniform)
+    int chunk = 0, g = 0, h = 0, n = 0, t0 = 0, t1 = 0;
+    const char *kseq = nullptr, *vseq = nullptr, *knseq = nullptr, *vnseq = nullptr;
+    const int* bt = nullptr;
+    long long seq_row0 = 0;
+    auto decode = [&](int item) -> bool {                    // false: the chunk holds no token
         const int hg = item % hgroups;
-        const int chunk = (item / hgroups) % a.nsplit;
-        const int g = item / (hgroups * a.nsplit);
-        const int h = hg * waves + wave;                      // KV head of this wave
-        const int n = uniform(seq_pos(a, g)) + 1;
-        int t0, t1;
+        chunk = (item / hgroups) % a.nsplit;
+        g = item / (hgroups * a.nsplit);
+        h = hg * group_waves + wv;                            // KV head of this wave
+        n = uniform(seq_pos(a, g)) + 1;
         chunk_range(n, chunk, a.nsplit, t0, t1);
-        if (t0 >= t1) continue;                               // uniform
-
+        if (t0 >= t1) return false;
         // scalar bases of this wave's head
-        const char* kseq = reinterpret_cast<const char*>(a.k) + (long long)h * 64;
-        const char* vseq = reinterpret_cast<const char*>(a.v) + (long long)h * 64;
-        const char* knseq = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
-        const char* vnseq = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
-        const int* bt = PAGED ? a.block_table + (long long)g * a.bt_stride : nullptr;
-        const long long seq_row0 = (long long)g * a.seq_stride_rows;
+        kseq = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes;
+        vseq = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes;
+        knseq = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
+        vnseq = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
+        bt = PAGED ? a.block_table + (long long)g * a.bt_stride : nullptr;
+        seq_row0 = (long long)g * a.seq_stride_rows;
+        return true;
+    };
 
-        // Buffer descriptors: base = first cache row of the tile (contiguous cache) or of the
-        // 16-token page (paged cache), extent = the rows that exist, so lanes past the end
-        // of the sequence read zeros instead of foreign memory.  All scalar.
-        auto page_row = [&](int ts) -> long long {   // paged: past the end re-read the last page (masked)
-            return (long long)uniform(bt[min(ts, t1 - 1) >> 4]) * kPageTokens;
-        };
-        auto issue_k = [&](uint4 (&kreg)[2], int tile) {
-            if (PAGED) {
+    // Buffer descriptors: base = first cache row of the tile (contiguous cache) or of the
+    // 16-token page (paged cache), extent = the rows that exist, so lanes past the end
+    // of the sequence read zeros instead of foreign memory.  All scalar.
+    auto page_row = [&](int ts) -> long long {   // paged: past the end re-read the last page (masked)
+        return (long long)uniform(bt[min(ts, t1 - 1) >> 4]) * kPageTokens;
+    };
+    auto load_k = [&](__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t (&dst)[KW]) {
+        if constexpr (BITS == 4) {
+            uint32x4_t q = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+            dst[0] = q[0]; dst[1] = q[1]; dst[2] = q[2]; dst[3] = q[3];
+        } else {
+            uint32x2_t q = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
+            dst[0] = q[0]; dst[1] = q[1];
+        }
+    };
+    auto issue_k = [&](uint32_t (&kreg)[2][KW], int tile) {
+        if (PAGED) {
 #pragma unroll
-                for (int sub = 0; sub < 2; sub++) {
-                    __amdgpu_buffer_rsrc_t r = make_rsrc(kseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp);
-                    uint32x4_t q = __builtin_amdgcn_raw_buffer_load_b128(r, (int)koff, 0, 0);
-                    kreg[sub] = uint4{q[0], q[1], q[2], q[3]};
-                }
-            } else {
-                __amdgpu_buffer_rsrc_t r = make_rsrc(kseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
-                uint32x4_t q0 = __builtin_amdgcn_raw_buffer_load_b128(r, (int)koff, 0, 0);
-                uint32x4_t q1 = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + sub_bytes), 0, 0);
-                kreg[0] = uint4{q0[0], q0[1], q0[2], q0[3]};
-                kreg[1] = uint4{q1[0], q1[1], q1[2], q1[3]};
+            for (int sub = 0; sub < 2; sub++)
+                load_k(make_rsrc(kseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp), koff, kreg[sub]);
+        } else {
+            __amdgpu_buffer_rsrc_t r = make_rsrc(kseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
+            load_k(r, koff, kreg[0]);
+            load_k(r, koff + sub_bytes, kreg[1]);
+        }
+    };
+    auto issue_v = [&](uint32_t (&vreg)[2][VW], int tile) {
+        if (PAGED) {
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp);
+#pragma unroll
+                for (int i = 0; i < VW; i++) vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff[i], 0, 0);
             }
-        };
-        auto issue_v = [&](uint32_t (&vreg)[2][4], int tile) {
-            if (PAGED) {
+        } else {
+            __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
 #pragma unroll
-                for (int sub = 0; sub < 2; sub++) {
-                    __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp);
+            for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff[i], 0, 0);
-                }
-            } else {
-                __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
-#pragma unroll
-                for (int sub = 0; sub < 2; sub++) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)(voff[i] + sub * sub_bytes), 0, 0);
-                }
+                for (int i = 0; i < VW; i++)
+                    vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)(voff[i] + sub * sub_bytes), 0, 0);
             }
-        };
-        // fp16 bits of kn (low half) and vn (high half) of this lane's token.  When a norm row
-        // (all KV heads of one token) is a multiple of 16 bytes the lane fetches the 16 bytes
-        // that hold its head with one b128 load (rows of consecutive tokens are contiguous, so
-        // the 32 useful lanes read one contiguous run) and picks its half-word; a 2-byte gather
-        // over the same rows costs ~15 % of the whole scan's bandwidth.
-        auto pick = [&](const uint32x4_t& q) -> uint32_t {
-            const int dw = (h & 7) >> 1;
-            uint32_t w = dw == 0 ? q[0] : dw == 1 ? q[1] : dw == 2 ? q[2] : q[3];
-            return (h & 1) ? (w >> 16) : (w & 0xffffu);
-        };
-        auto issue_n = [&](int tile) -> uint32_t {
-            const bool wide = (nrow & 15u) == 0;
-            const uint32_t hgrp = (uint32_t)(h >> 3) * 16u;          // 16-byte group of this head inside a row
-            if (PAGED) {
-                long long r0 = page_row(tile), r1 = page_row(tile + 16);
-                const long long rr = my_sub ? r1 : r0;
-                if (wide) {
-                    uint32x4_t kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
-                    if (useful) {
-                        const char* kp = reinterpret_cast<const char*>(a.k_norms) + (rr + ln) * nrow + hgrp;
-                        const char* vp = reinterpret_cast<const char*>(a.v_norms) + (rr + ln) * nrow + hgrp;
-                        kq = *reinterpret_cast<const uint32x4_t*>(kp);
-                        vq = *reinterpret_cast<const uint32x4_t*>(vp);
-                    }
-                    return pick(kq) | (pick(vq) << 16);
-                }
-                uint32_t kk = *reinterpret_cast<const uint16_t*>(knseq + (rr + ln) * nrow);
-                uint32_t vv = *reinterpret_cast<const uint16_t*>(vnseq + (rr + ln) * nrow);
-                return kk | (vv << 16);
-            }
-            const long long row = seq_row0 + tile;
-            const int rows = max(min(n - tile, 32), 0);
+        }
+    };
+    // fp16 bits of kn (low half) and vn (high half) of this lane's token.  When a norm row
+    // (all KV heads of one token) is a multiple of 16 bytes the lane fetches the 16 bytes
+    // that hold its head with one b128 load (rows of consecutive tokens are contiguous, so
+    // the 32 useful lanes read one contiguous run) and picks its half-word; a 2-byte gather
+    // over the same rows costs ~15 % of the whole scan's bandwidth.
+    auto pick = [&](const uint32x4_t& q) -> uint32_t {
+        const int dw = (h & 7) >> 1;
+        uint32_t w = dw == 0 ? q[0] : dw == 1 ? q[1] : dw == 2 ? q[2] : q[3];
+        return (h & 1) ? (w >> 16) : (w & 0xffffu);
+    };
+    auto issue_n = [&](int tile) -> uint32_t {
+        const bool wide = (nrow & 15u) == 0;
+        const uint32_t hgrp = (uint32_t)(h >> 3) * 16u;          // 16-byte group of this head inside a row
+        if (PAGED) {
+            long long r0 = page_row(tile), r1 = page_row(tile + 16);
+            const long long rr = my_sub ? r1 : r0;
             if (wide) {
-                __amdgpu_buffer_rsrc_t rk = make_rsrc(reinterpret_cast<const char*>(a.k_norms) + row * nrow, rows * (int)nrow);
-                __amdgpu_buffer_rsrc_t rv = make_rsrc(reinterpret_cast<const char*>(a.v_norms) + row * nrow, rows * (int)nrow);
                 uint32x4_t kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
                 if (useful) {
-                    kq = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)(noff + hgrp), 0, 0);
-                    vq = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)(noff + hgrp), 0, 0);
+                    const char* kp = reinterpret_cast<const char*>(a.k_norms) + (rr + ln) * nrow + hgrp;
+                    const char* vp = reinterpret_cast<const char*>(a.v_norms) + (rr + ln) * nrow + hgrp;
+                    kq = *reinterpret_cast<const uint32x4_t*>(kp);
+                    vq = *reinterpret_cast<const uint32x4_t*>(vp);
                 }
                 return pick(kq) | (pick(vq) << 16);
             }
-            __amdgpu_buffer_rsrc_t rk = make_rsrc(knseq + row * nrow, rows * (int)nrow);
-            __amdgpu_buffer_rsrc_t rv = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
-            uint32_t kk = __builtin_amdgcn_raw_buffer_load_b16(rk, (int)noff, 0, 0);
-            uint32_t vv = __builtin_amdgcn_raw_buffer_load_b16(rv, (int)noff, 0, 0);
+            uint32_t kk = *reinterpret_cast<const uint16_t*>(knseq + (rr + ln) * nrow);
+            uint32_t vv = *reinterpret_cast<const uint16_t*>(vnseq + (rr + ln) * nrow);
             return kk | (vv << 16);
-        };
+        }
+        const long long row = seq_row0 + tile;
+        const int rows = max(min(n - tile, 32), 0);
+        if (wide) {
+            __amdgpu_buffer_rsrc_t rk = make_rsrc(reinterpret_cast<const char*>(a.k_norms) + row * nrow, rows * (int)nrow);
+            __amdgpu_buffer_rsrc_t rv = make_rsrc(reinterpret_cast<const char*>(a.v_norms) + row * nrow, rows * (int)nrow);
+            uint32x4_t kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
+            if (useful) {
+                kq = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)(noff + hgrp), 0, 0);
+                vq = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)(noff + hgrp), 0, 0);
+            }
+            return pick(kq) | (pick(vq) << 16);
+        }
+        __amdgpu_buffer_rsrc_t rk = make_rsrc(knseq + row * nrow, rows * (int)nrow);
+        __amdgpu_buffer_rsrc_t rv = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
+        uint32_t kk = __builtin_amdgcn_raw_buffer_load_b16(rk, (int)noff, 0, 0);
+        uint32_t vv = __builtin_amdgcn_raw_buffer_load_b16(rv, (int)noff, 0, 0);
+        return kk | (vv << 16);
+    };
+
+    // DEPTH tiles of loads are in flight per wave; each register set is re-issued (for the
+    // tile DEPTH further on) as soon as its contents have been expanded.
+    uint32_t kring[DEPTH][2][KW];
+    uint32_t vring[DEPTH][2][VW];
+    uint32_t nring[DEPTH];
+    auto issue_first = [&]() {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (d == 0 || t0 + 32 * d < t1) {
+                issue_k(kring[d], t0 + 32 * d);
+                nring[d] = issue_n(t0 + 32 * d);
+                issue_v(vring[d], t0 + 32 * d);
+            }
+        }
+    };
+
+    // The first loads of the first item are in flight while the workgroup builds its table.
+    const int item_step = (int)gridDim.x * ngroups;
+    int item = (int)blockIdx.x * ngroups + grp;
+    bool ready = false;          // the item is decoded, holds tokens, and its first loads are issued
+    if (item < total_items && decode(item)) {
+        issue_first();
+        ready = true;
+    }
+    // ---- dequantization table, once per workgroup: entry e fills 256 bytes with replicas
+    for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
+        const int e = i >> 6;
+        if constexpr (BITS == 4) {
+            half2_t p = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
+            uint32_t w = *reinterpret_cast<uint32_t*>(&p);
+            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
+        } else {
+            half2_t p0 = {(half_t)(kAlpha * kCentroids2[e & 3]), (half_t)(kAlpha * kCentroids2[(e >> 4) & 3])};
+            half2_t p1 = {(half_t)(kAlpha * kCentroids2[(e >> 2) & 3]), (half_t)(kAlpha * kCentroids2[(e >> 6) & 3])};
+            uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
+            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
+        }
+    }
+    for (int i = tid; i < kMaxWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
+    __syncthreads();             // the only workgroup-wide barrier; every wave reaches it
+
+    for (; item < total_items; item += item_step) {
+        if (!ready) {
+            if (!decode(item)) continue;                      // uniform over the wave
+            issue_first();
+        }
+        ready = false;
+        const int ntiles = (t1 - t0 + 31) >> 5;
 
         float4_t o[8];
 #pragma unroll
@@ -258,37 +352,9 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
 #pragma unroll
         for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
 
-        // DEPTH tiles of loads are in flight per wave; a slot is re-issued (for the tile DEPTH
-        // further on) as soon as its contents have been expanded.
-        const int ntiles = (t1 - t0 + 31) >> 5;
-        uint4 kring[DEPTH][2];
-        uint32_t vring[DEPTH][2][4];
-        uint32_t nring[DEPTH];
-#pragma unroll
-        for (int d = 0; d < DEPTH; d++) {
-            if (d < ntiles && TW_EXP != 5) {
-                issue_k(kring[d], t0 + 32 * d);
-                nring[d] = issue_n(t0 + 32 * d);
-                issue_v(vring[d], t0 + 32 * d);
-            }
-        }
-
-        // The first loads are already in flight while the workgroup builds its table.
-        if (!table_ready) {
-        // ---- dequantization table, once per workgroup: entry e, 64 identical words
-        for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
-            int e = i >> 6;
-            half2_t p = {(half_t)(kAlpha4 * kCentroids4[e & 15]), (half_t)(kAlpha4 * kCentroids4[e >> 4])};
-            uint32_t w = *reinterpret_cast<uint32_t*>(&p);
-            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
-        }
-        for (int i = tid; i < kMaxWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
-        __syncthreads();
-            table_ready = true;
-        }
-
         // A operand of the score MFMAs: q_rot[head][32kg + 8j + i]; row m carries the
-        // fp16 value of head m, row m + 8 what the rounding left over.
+        // fp16 value of head m, row m + 8 what the rounding left over.  The 2-bit table
+        // returns the codes of a byte in the order 0,2,1,3.
         half8_t aq[4];
         {
             const int hq = ln & 7;
@@ -301,7 +367,8 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                 float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
-                    float x = (hq < R) ? v[i] : 0.0f;
+                    const int src = BITS == 4 ? i : ((i & 4) | ((i & 1) << 1) | ((i & 2) >> 1));
+                    float x = (hq < R) ? v[src] : 0.0f;
                     half_t hi = (half_t)x;
                     half_t lo = (half_t)(x - (float)hi);
                     aq[j][i] = lo_part ? lo : hi;
@@ -309,65 +376,41 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
             }
         }
 
-
         for (int it0 = 0; it0 < ntiles; it0 += DEPTH) {
 #pragma unroll
           for (int d = 0; d < DEPTH; d++) {
             const int it = it0 + d;
-            if (it >= ntiles) break;
-            uint4 (&kreg)[2] = kring[d];
-            uint32_t (&vreg)[2][4] = vring[d];
+            if (DEPTH > 1 && it >= ntiles) break;
+            uint32_t (&kreg)[2][KW] = kring[d];
+            uint32_t (&vreg)[2][VW] = vring[d];
             uint32_t& nreg = nring[d];
             const int tile = t0 + 32 * it;
             const int next_tile = tile + 32 * DEPTH;
             const bool more = it + DEPTH < ntiles;
 
-#if TW_EXP == 5
-            {   // loads only, plain global loads with per-lane 64-bit pointers
-                const char* kp = kseq + (seq_row0 + tile) * kvp + koff;
-                const char* vp = vseq + (seq_row0 + tile) * kvp;
-                uint4 ka = *reinterpret_cast<const uint4*>(kp);
-                uint4 kb2 = *reinterpret_cast<const uint4*>(kp + sub_bytes);
-                uint32_t f = ka.x ^ ka.w ^ kb2.y ^ kb2.z;
-#pragma unroll
-                for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) f ^= *reinterpret_cast<const uint32_t*>(vp + voff[i] + sub * sub_bytes);
-                if (useful) {
-                    const char* np_ = reinterpret_cast<const char*>(a.k_norms) + (seq_row0 + tile) * nrow + noff;
-                    const char* nq_ = reinterpret_cast<const char*>(a.v_norms) + (seq_row0 + tile) * nrow + noff;
-                    uint4 n1 = *reinterpret_cast<const uint4*>(np_);
-                    uint4 n2 = *reinterpret_cast<const uint4*>(nq_);
-                    f ^= n1.x ^ n2.w;
-                }
-                o[0][0] += __uint_as_float(f & 0x3fffffu);
-                continue;
-            }
-#endif
-#if TW_EXP == 4
-            {   // loads only: fold the loaded words into one accumulator and re-issue
-                uint32_t f = kreg[0].x ^ kreg[0].y ^ kreg[0].z ^ kreg[0].w ^ kreg[1].x ^ kreg[1].y ^ kreg[1].z ^ kreg[1].w ^ nreg;
-#pragma unroll
-                for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) f ^= vreg[sub][i];
-                o[0][0] += __uint_as_float(f & 0x3fffffu);
-                if (more) { issue_k(kreg, next_tile); nreg = issue_n(next_tile); issue_v(vreg, next_tile); }
-                continue;
-            }
-#endif
             // ---- scores S[head][token] for both sub-tiles
             float4_t s[2];
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
-                const uint32_t w[4] = {kreg[sub].x, kreg[sub].y, kreg[sub].z, kreg[sub].w};
+                uint32_t kw[KW];
+#pragma unroll
+                for (int i = 0; i < KW; i++) kw[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(ksrc, (int)kreg[sub][i]);
                 union { uint32_t u[4]; half8_t h; } kv[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    kv[j].u[0] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0400u));
-                    kv[j].u[1] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0500u));
-                    kv[j].u[2] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0600u));
-                    kv[j].u[3] = TW_LUTK(__builtin_amdgcn_perm(w[j], lane4, 0x0c0c0700u));
+                    if constexpr (BITS == 4) {
+                        const uint32_t w = kw[j];
+                        kv[j].u[0] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0400u));
+                        kv[j].u[1] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0500u));
+                        kv[j].u[2] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0600u));
+                        kv[j].u[3] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0700u));
+                    } else {
+                        const uint32_t w = kw[j >> 1];
+                        const uint32_t sel = (j & 1) ? 0x0c0c0600u : 0x0c0c0400u;
+                        uint2 l0 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel));
+                        uint2 l1 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel + 0x100u));
+                        kv[j].u[0] = l0.x; kv[j].u[1] = l0.y; kv[j].u[2] = l1.x; kv[j].u[3] = l1.y;
+                    }
                 }
                 s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -422,29 +465,62 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
             __builtin_amdgcn_wave_barrier();
 
             // ---- O[head][dim 8ln + j] += P[head][token] V[token][dim]
-            uint32_t xe[4], xo[4];   // [2*sub + pair]: index bytes for even / odd dims
+            if constexpr (BITS == 4) {
+                uint32_t xe[4], xo[4];   // [2*sub + pair]: index bytes for even / odd dims
 #pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
+                for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
-                for (int pr = 0; pr < 2; pr++) {
-                    uint32_t wa = vreg[sub][2 * pr], wb = vreg[sub][2 * pr + 1];
-                    xe[2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
-                    xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                    for (int pr = 0; pr < 2; pr++) {
+                        uint32_t wa = vreg[sub][2 * pr], wb = vreg[sub][2 * pr + 1];
+                        xe[2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                        xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                    }
+                }
+                if (more) issue_v(vreg, next_tile);
+#pragma unroll
+                for (int jp = 0; jp < 4; jp++) {         // two dims (even, odd) per step: 8 look-ups, 2 MFMAs
+                    const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
+                    union { uint32_t u[4]; half8_t h; } be, bo;
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        be.u[q4] = lut32(__builtin_amdgcn_perm(xe[q4], lane_rep, sel));
+                        bo.u[q4] = lut32(__builtin_amdgcn_perm(xo[q4], lane_rep, sel));
+                    }
+                    o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * jp], 0, 0, 0);
+                    o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * jp + 1], 0, 0, 0);
+                }
+            } else {
+                // Per sub-tile: wa = 16-bit codes of tokens (4kg, 4kg+2), wb = of (4kg+1, 4kg+3) for
+                // this lane's 8 dims.  ie/io: per byte, low nibble = token a dims (d, d+1), high
+                // nibble = token b dims (d, d+1); bytes = (tokens 0,1 | d=0), (0,1 | d=4),
+                // (2,3 | d=0), (2,3 | d=4) for ie and d = 2, 6 for io.
+                uint32_t ie[2], io[2];
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+                    const uint32_t keep = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_keep);
+                    const uint32_t send = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_send);
+                    const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xf, 0xf, false);  // lane ^ 1
+                    const uint32_t wa = odd ? recv : keep, wb = odd ? keep : recv;
+                    ie[sub] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                    io[sub] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                }
+                if (more) issue_v(vreg, next_tile);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {            // dims (2q, 2q+1): 4 look-ups, 2 MFMAs
+                    const uint32_t x0 = (q & 1) ? io[0] : ie[0], x1 = (q & 1) ? io[1] : ie[1];
+                    const uint32_t sel = 0x0c0c0400u + ((uint32_t)(q >> 1) << 8);
+                    uint2 l00 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel));
+                    uint2 l01 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel + 0x200u));
+                    uint2 l10 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel));
+                    uint2 l11 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel + 0x200u));
+                    union { uint32_t u[4]; half8_t h; } be, bo;
+                    be.u[0] = l00.x; be.u[1] = l01.x; be.u[2] = l10.x; be.u[3] = l11.x;
+                    bo.u[0] = l00.y; bo.u[1] = l01.y; bo.u[2] = l10.y; bo.u[3] = l11.y;
+                    o[2 * q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * q], 0, 0, 0);
+                    o[2 * q + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * q + 1], 0, 0, 0);
                 }
             }
-            if (more) issue_v(vreg, next_tile);
-#pragma unroll
-            for (int jp = 0; jp < 4; jp++) {         // two dims (even, odd) per step: 8 look-ups, 2 MFMAs
-                const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
-                union { uint32_t u[4]; half8_t h; } be, bo;
-#pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) {
-                    be.u[q4] = TW_LUTV(__builtin_amdgcn_perm(xe[q4], lane4, sel));
-                    bo.u[q4] = TW_LUTV(__builtin_amdgcn_perm(xo[q4], lane4, sel));
-                }
-                o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * jp], 0, 0, 0);
-                o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * jp + 1], 0, 0, 0);
-            }
+            if (DEPTH > 1) __builtin_amdgcn_sched_barrier(0);   // keep the unrolled tiles from interleaving (register pressure)
           }
         }
 
@@ -461,7 +537,7 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
                 float* part = a.ws + ((long long)g * a.num_heads + (long long)h * R + r) * a.ws_stride +
                               (long long)chunk * kPartialFloats;
 #pragma unroll
-                for (int j = 0; j < 8; j++) part[8 * ln + j] = o[j][r] * (1.0f / kAlpha4);
+                for (int j = 0; j < 8; j++) part[8 * ln + j] = o[j][r] * (1.0f / kAlpha);
                 if (ln == 0) {
                     part[kHeadDim] = m_run[r];
                     part[kHeadDim + 1] = l_run[r];
@@ -471,33 +547,34 @@ attention_mfma4_kernel(AttnArgs a, int total_items, int hgroups) {
     }
 }
 
-static int resident_groups() {
+static int compute_units() {
     static int cached = 0;
     if (cached == 0) {
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             cus = 256;
-        cached = (TW_DEPTH <= 1 ? 2 : 1) * cus;   // 64 KB of LDS and <= 128 VGPRs per workgroup of 8 waves: two per CU
+        cached = cus;
     }
     return cached;
 }
 
+// waves that walk one item together: the KV heads, at most kGroupWaves at a time
 static int scan_waves(const AttnArgs& a) {
-    int waves = a.num_kv_heads < kMaxWaves ? a.num_kv_heads : kMaxWaves;
+    int waves = a.num_kv_heads < kGroupWaves ? a.num_kv_heads : kGroupWaves;
     while (a.num_kv_heads % waves != 0) waves--;
     return waves;
 }
 
 float attention_mfma_q_scale(int bits) {
-    (void)bits;
-    return kLog2e * kInvSqrtD / kAlpha4;   // score scale of kernels.cu:1707 in base 2, table scale undone
+    // score scale of kernels.cu:1707 in base 2, table scale undone
+    return kLog2e * kInvSqrtD / (bits == 4 ? kAlpha4 : kAlpha2);
 }
 
 // Shape check; with rotate_query also q_rot = R q (kernels.cu:1671-1681) into the workspace.
 bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     const int R = a.num_heads / a.num_kv_heads;
-    if (a.bits != 4) return false;
+    if (a.bits != 4 && a.bits != 2) return false;
     if (R != 1 && R != 2 && R != 4) return false;
     // needs the split workspace with room for q_rot behind each block's partials
     if (!a.ws || !a.qrot) return false;
@@ -529,19 +606,26 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     const int waves = scan_waves(a);
     const int hgroups = a.num_kv_heads / waves;
     const int items = a.G * a.nsplit * hgroups;
-    int grid = resident_groups();
-    if (items < grid) grid = items;
-    const int R = a.num_heads / a.num_kv_heads;
-    const dim3 g3(grid), b3(waves * kWave);
-#ifndef TW_DEPTH
-#define TW_DEPTH 1
-#endif
-#define TW_LAUNCH(P, RR) hipLaunchKernelGGL((attention_mfma4_kernel<P, RR, TW_DEPTH>), g3, b3, 0, s, a, items, hgroups)
-    if (a.block_table) {
-        if (R == 1) TW_LAUNCH(true, 1); else if (R == 2) TW_LAUNCH(true, 2); else TW_LAUNCH(true, 4);
-    } else {
-        if (R == 1) TW_LAUNCH(false, 1); else if (R == 2) TW_LAUNCH(false, 2); else TW_LAUNCH(false, 4);
+    // One workgroup per CU (80 KB of LDS, <= 128 VGPRs), made of as many groups as fit in
+    // kMaxWaves waves; fewer groups or workgroups when there are not that many items.
+    int ngroups = kMaxWaves / waves;
+    int grid = compute_units();
+    if (items < grid * ngroups) {
+        ngroups = (items + grid - 1) / grid;
+        if (ngroups < 1) ngroups = 1;
+        grid = (items + ngroups - 1) / ngroups;
     }
+    const int R = a.num_heads / a.num_kv_heads;
+    const dim3 g3(grid), b3(ngroups * waves * kWave);
+#define TW_LAUNCH(P, RR, BB) hipLaunchKernelGGL((attention_mfma_kernel<P, RR, BB, (BB == 4 ? TW_DEPTH4 : TW_DEPTH2)>), g3, b3, 0, s, a, items, hgroups, waves)
+#define TW_LAUNCH_R(P, BB) \
+    do { if (R == 1) TW_LAUNCH(P, 1, BB); else if (R == 2) TW_LAUNCH(P, 2, BB); else TW_LAUNCH(P, 4, BB); } while (0)
+    if (a.block_table) {
+        if (a.bits == 4) TW_LAUNCH_R(true, 4); else TW_LAUNCH_R(true, 2);
+    } else {
+        if (a.bits == 4) TW_LAUNCH_R(false, 4); else TW_LAUNCH_R(false, 2);
+    }
+#undef TW_LAUNCH_R
 #undef TW_LAUNCH
 }
 

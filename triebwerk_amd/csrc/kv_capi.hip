@@ -71,7 +71,7 @@ bool check_bits(const char* fn, int bits) {
 // ws_floats_per_head: room per (sequence, head) in the caller's workspace.
 void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     if (ctx_bound < 1) ctx_bound = 1;
-    const bool mfma = a.bits == 4 && g_variant.load() != 1 && a.num_heads / a.num_kv_heads <= 4;
+    const bool mfma = a.bits != 0 && g_variant.load() != 1 && a.num_heads / a.num_kv_heads <= 4;
     // workgroups per split: the MFMA scan takes up to 8 KV heads per workgroup,
     // the vector-ALU kernel one (KV head, tile of query heads) each
     long long base_groups;
@@ -411,7 +411,7 @@ void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_ha
     // one rotation launch for the appended K and V rows and, when the MFMA scan will run,
     // for the query as well
     const int R = num_heads / num_kv_heads;
-    const bool fuse_q = mfma_wanted(a) && a.qrot && (R == 1 || R == 2 || R == 4) && bits == 4 &&
+    const bool fuse_q = mfma_wanted(a) && a.qrot && (R == 1 || R == 2 || R == 4) &&
                         (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0;
     if (g_variant.load() == 1 || !fuse_q) {
         tw_turbo_kv_append_batch(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotation, pos, msl, G,
