@@ -44,10 +44,11 @@ WORKLOADS = {
 }
 BYTES_HEAD = {0: 256, 4: 66, 2: 34}  # per (token, kv head): fp16 row | codes + fp16 norm
 
-# HBM bytes per launch of the context-scanning kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# on this file's own run (counter KiB scaled by what `--copy-calibration` reads for a copy of
-# known size); the summaries are profiles/scan_kv{4,2,16}_target_pmc.txt.  Keyed by (workload, kv_bits).
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch (read + write) of the context-scanning kernel, from rocprofv3 --pmc FETCH_SIZE
+# and WRITE_SIZE on this file's own run, each counter scaled by what `--copy-calibration` reads for a
+# copy of known size (2.0 and 1.0); summary and commands in profiles/scan_target_hbm_traffic_pmc.txt.
+# Keyed by (workload, kv_bits); a measurement of the kernels as committed with that file, not live.
+MEASURED_TRAFFIC_BYTES = {("target", 4): 560.6e6, ("target", 2): 291.9e6, ("target", 0): 2151.2e6}
 
 
 def algorithmic_bytes(n_tokens_total: int, G: int, L: int, H: int, Hk: int, kv_bits: int, with_append: bool) -> int:
