@@ -1,0 +1,232 @@
+"""GPU parity at the benchmark's full sizes (one layer of each): batch 64, context 8192,
+Qwen3-0.6B KV shape; the ragged paged case with contexts in [512, 8192]; the 2-bit case
+with 32 query heads at context 4097.
+
+The oracle is too slow to quantize 64 x 8192 tokens, so the cache is built on the GPU by
+the T-token append and checked three ways: a few whole sequences against the oracle bit
+for bit, every other sequence against the one it replicates (the same rows must give the
+same bytes wherever they are written), and a checksum of the per-sequence checksums.
+Attention is then checked for EVERY sequence against the oracle run over the cache the GPU
+wrote, for both kernel families, and the two families against each other.
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+import gen
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+D = 128
+
+
+@pytest.fixture(scope="module")
+def kv():
+    import torch
+    from triebwerk_amd import kvcache
+    assert torch.cuda.is_available()
+    yield kvcache
+    kvcache.set_attention_variant(0)
+    kvcache.set_num_splits(0)
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    import torch
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def rel_err_rows(got, want):
+    got = got.astype(np.float64).reshape(-1, D)
+    want = want.astype(np.float64).reshape(-1, D)
+    return np.max(np.abs(got - want), axis=1) / np.max(np.abs(want), axis=1)
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_target_shape_append_and_attention(kv, oracle, rotation_fixture, bits):
+    import torch
+    G, H, Hk, ctx = 64, 16, 8, 8192
+    kv_dim, q_dim = Hk * D, H * D
+    kvp = kv_dim * bits // 8
+    msl = ctx
+    n_base = 4                                   # distinct sequences; sequence g replicates g % n_base
+    r = gen.rng(900 + bits)
+    rot = dev(rotation_fixture)
+    base_k = [gen.kv_rows_with_outliers(r, (ctx, kv_dim), kv_dim)[0] for _ in range(n_base)]
+    base_v = [gen.normal_f16(r, (ctx, kv_dim)) for _ in range(n_base)]
+    d_base_k = [dev(x) for x in base_k]
+    d_base_v = [dev(x) for x in base_v]
+
+    ck = torch.zeros((G, msl, kvp), dtype=torch.uint8, device="cuda")
+    cv = torch.zeros_like(ck)
+    kn = torch.zeros((G, msl, Hk), dtype=torch.float16, device="cuda")
+    vn = torch.zeros_like(kn)
+    tok = dev(np.arange(ctx, dtype=np.int32))
+    for g in range(G):                           # T-token append (kernels.cu:1482-1560), one sequence per call
+        kv.launch_turbo_kv_quantize(ck[g], kn[g], d_base_k[g % n_base], rot, tok, msl, ctx, Hk, D, kv_dim, bits)
+        kv.launch_turbo_kv_quantize(cv[g], vn[g], d_base_v[g % n_base], rot, tok, msl, ctx, Hk, D, kv_dim, bits)
+    h_ck, h_cv, h_kn, h_vn = host(ck), host(cv), host(kn), host(vn)
+
+    # (1) base sequences against the oracle, every byte
+    for b in range(n_base):
+        for rows, codes, norms, what in ((base_k[b], h_ck[b], h_kn[b], "K"), (base_v[b], h_cv[b], h_vn[b], "V")):
+            oq = np.zeros((msl, kvp), np.uint8); on = np.zeros((msl, Hk), np.float16)
+            oracle.turbo_kv_quantize(oq, on, rows, rotation_fixture, np.arange(ctx, dtype=np.int32), msl, ctx, Hk, D,
+                                     kv_dim, bits)
+            assert np.array_equal(codes, oq), f"{what} codes of sequence {b}: {(codes != oq).sum()} bytes differ"
+            assert np.array_equal(norms.view(np.uint16), on.view(np.uint16)), f"{what} norms of sequence {b}"
+    # (2) replicas equal their base; (3) checksum of checksums over the whole cache
+    sums = []
+    for g in range(G):
+        b = g % n_base
+        assert np.array_equal(h_ck[g], h_ck[b]) and np.array_equal(h_cv[g], h_cv[b]), f"sequence {g} != its base {b}"
+        assert np.array_equal(h_kn[g].view(np.uint16), h_kn[b].view(np.uint16))
+        assert np.array_equal(h_vn[g].view(np.uint16), h_vn[b].view(np.uint16))
+        sums.append(zlib.crc32(h_ck[g].tobytes()) ^ zlib.crc32(h_cv[g].tobytes()))
+    base_sums = [sums[b] for b in range(n_base)]
+    assert zlib.crc32(np.array(sums, np.uint32).tobytes()) == \
+        zlib.crc32(np.array([base_sums[g % n_base] for g in range(G)], np.uint32).tobytes())
+
+    # attention over the whole batch, every sequence with its own query and (ragged by a few) position
+    q = gen.normal_f16(r, (G, q_dim))
+    pos = (ctx - 1 - (np.arange(G) % 5)).astype(np.int32)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, h_ck, h_cv, h_kn, h_vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim,
+                                     kv_dim, bits)
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    outs = {}
+    for variant in (0, 1):
+        kv.set_attention_variant(variant)
+        out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+        kv.launch_turbo_gqa_attention_batch(out, dev(q), ck, cv, kn, vn, rot, scratch, dev(pos), msl, G, H, Hk, D,
+                                            q_dim, kv_dim, bits)
+        outs[variant] = host(out)
+        err = rel_err_rows(outs[variant], want)
+        assert err.max() <= TOL, f"variant {variant}: max rel err {err.max():.3e} at head vector {err.argmax()}"
+    kv.set_attention_variant(0)
+    cross = rel_err_rows(outs[0], outs[1])
+    assert cross.max() <= TOL, f"MFMA vs vector-ALU kernels: {cross.max():.3e}"
+    # same cache and query in two batch slots give the same output bits (no dependence on placement)
+    q2 = q.copy(); q2[n_base:2 * n_base] = q2[:n_base]
+    pos2 = pos.copy(); pos2[n_base:2 * n_base] = pos2[:n_base]
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    kv.launch_turbo_gqa_attention_batch(out, dev(q2), ck, cv, kn, vn, rot, scratch, dev(pos2), msl, G, H, Hk, D,
+                                        q_dim, kv_dim, bits)
+    o = host(out)
+    assert np.array_equal(o[:n_base].view(np.uint16), o[n_base:2 * n_base].view(np.uint16))
+
+
+def test_target_shape_fp16_cache(kv, oracle):
+    import torch
+    G, H, Hk, ctx = 16, 16, 8, 8192              # a quarter of the batch: the oracle needs the cache in host memory
+    kv_dim, q_dim = Hk * D, H * D
+    msl = ctx
+    r = gen.rng(950)
+    g_ = torch.Generator(device="cuda"); g_.manual_seed(951)
+    ck = torch.randn((G, msl, kv_dim), generator=g_, device="cuda", dtype=torch.float16)
+    cv = torch.randn((G, msl, kv_dim), generator=g_, device="cuda", dtype=torch.float16)
+    pos = (ctx - 1 - (np.arange(G) % 3)).astype(np.int32)
+    k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim)); q = gen.normal_f16(r, (G, q_dim))
+    kv.launch_kv_cache_write_batch(ck, cv, dev(k), dev(v), dev(pos), msl, G, kv_dim)
+    h_ck, h_cv = host(ck), host(cv)
+    for g in range(G):                           # appended rows land where they should, nothing else moves
+        assert np.array_equal(h_ck[g, pos[g]].view(np.uint16), k[g].view(np.uint16))
+        assert np.array_equal(h_cv[g, pos[g]].view(np.uint16), v[g].view(np.uint16))
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, h_ck, h_cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    kv.launch_gqa_attention_batch(out, dev(q), ck, cv, scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim)
+    err = rel_err_rows(host(out), want)
+    assert err.max() <= TOL, f"max rel err {err.max():.3e}"
+
+
+def test_ragged_paged_batch64(kv, oracle, rotation_fixture):
+    """Contexts uniform in [512, 8192], 16-token pages in random order (4-bit)."""
+    import torch
+    bits, G, H, Hk = 4, 64, 16, 8
+    kv_dim, q_dim = Hk * D, H * D
+    kvp = kv_dim * bits // 8
+    r = gen.rng(960)
+    lens = gen.ragged_contexts(r, G, 512, 8192)
+    lens[0], lens[1] = 512, 8192
+    pages_per_seq = 8192 // 16
+    msl = pages_per_seq * 16
+    bt = gen.shuffled_block_table(r, G, pages_per_seq)
+    n_pages = G * pages_per_seq
+    g_ = torch.Generator(device="cuda"); g_.manual_seed(961)
+    p_ck = torch.randint(0, 256, (n_pages, 16, kvp), generator=g_, device="cuda", dtype=torch.uint8)
+    p_cv = torch.randint(0, 256, (n_pages, 16, kvp), generator=g_, device="cuda", dtype=torch.uint8)
+    p_kn = (11.3 + 0.7 * torch.randn((n_pages, 16, Hk), generator=g_, device="cuda")).to(torch.float16)
+    p_vn = (11.3 + 0.7 * torch.randn((n_pages, 16, Hk), generator=g_, device="cuda")).to(torch.float16)
+    rot = dev(rotation_fixture)
+    # one appended token per sequence through the paged append, then attention
+    pos = (lens - 1).astype(np.int32)
+    k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim)); q = gen.normal_f16(r, (G, q_dim))
+    d_bt = dev(bt)
+    kv.tw_paged_turbo_kv_append_batch(p_ck, p_kn, p_cv, p_vn, dev(k), dev(v), rot, dev(pos), d_bt, pages_per_seq, G,
+                                      Hk, D, kv_dim, bits)
+    idx = torch.from_numpy(bt.astype(np.int64)).cuda()
+
+    def gather(pool):                            # pages in block-table order = the contiguous layout
+        return host(pool[idx].reshape(G, msl, pool.shape[-1]))
+    ck, cv, kn, vn = gather(p_ck), gather(p_cv), gather(p_kn), gather(p_vn)
+    # the appended rows equal the oracle's contiguous append, bit for bit
+    ock, ocv, okn, ovn = ck.copy(), cv.copy(), kn.copy(), vn.copy()
+    for g in range(G):
+        ock[g, pos[g]] = 0; ocv[g, pos[g]] = 0; okn[g, pos[g]] = 0; ovn[g, pos[g]] = 0
+    oracle.turbo_kv_quantize_batch(ock, okn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(ocv, ovn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    assert np.array_equal(ck, ock) and np.array_equal(cv, ocv)
+    assert np.array_equal(kn.view(np.uint16), okn.view(np.uint16)) and np.array_equal(vn.view(np.uint16), ovn.view(np.uint16))
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    ws = torch.zeros(kv.attention_workspace_floats(G, H, msl), dtype=torch.float32, device="cuda")
+    for variant in (0, 1):
+        kv.set_attention_variant(variant)
+        out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+        kv.tw_paged_turbo_gqa_attention_batch(out, dev(q), p_ck, p_cv, p_kn, p_vn, rot, ws, dev(pos), d_bt,
+                                              pages_per_seq, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+        err = rel_err_rows(host(out), want)
+        assert err.max() <= TOL, f"variant {variant}: max rel err {err.max():.3e} (sequence {err.argmax() // H})"
+    kv.set_attention_variant(0)
+
+
+def test_tq2_gqa4_context4097(kv, oracle, rotation_fixture):
+    """2-bit codes, 32 query heads on 8 KV heads, batch 16, context 4096 + 1."""
+    import torch
+    bits, G, H, Hk, ctx = 2, 16, 32, 8, 4097
+    kv_dim, q_dim = Hk * D, H * D
+    kvp = kv_dim * bits // 8
+    msl = ctx
+    r = gen.rng(970)
+    g_ = torch.Generator(device="cuda"); g_.manual_seed(971)
+    ck = torch.randint(0, 256, (G, msl, kvp), generator=g_, device="cuda", dtype=torch.uint8)
+    cv = torch.randint(0, 256, (G, msl, kvp), generator=g_, device="cuda", dtype=torch.uint8)
+    kn = (11.3 + 0.7 * torch.randn((G, msl, Hk), generator=g_, device="cuda")).to(torch.float16)
+    vn = (11.3 + 0.7 * torch.randn((G, msl, Hk), generator=g_, device="cuda")).to(torch.float16)
+    rot = dev(rotation_fixture)
+    pos = np.full(G, ctx - 1, np.int32)
+    k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim)); q = gen.normal_f16(r, (G, q_dim))
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    kv.tw_turbo_append_attention_batch(out, dev(q), dev(k), dev(v), ck, cv, kn, vn, rot, scratch, dev(pos), msl, G, H,
+                                       Hk, D, q_dim, kv_dim, bits)
+    h_ck, h_cv, h_kn, h_vn = host(ck), host(cv), host(kn), host(vn)
+    ock, ocv, okn, ovn = h_ck.copy(), h_cv.copy(), h_kn.copy(), h_vn.copy()
+    ock[:, ctx - 1] = 0; ocv[:, ctx - 1] = 0; okn[:, ctx - 1] = 0; ovn[:, ctx - 1] = 0
+    oracle.turbo_kv_quantize_batch(ock, okn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(ocv, ovn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    assert np.array_equal(h_ck, ock) and np.array_equal(h_cv, ocv)
+    assert np.array_equal(h_kn.view(np.uint16), okn.view(np.uint16)) and np.array_equal(h_vn.view(np.uint16), ovn.view(np.uint16))
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ock, ocv, okn, ovn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    err = rel_err_rows(host(out), want)
+    assert err.max() <= TOL, f"max rel err {err.max():.3e}"
