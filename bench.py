@@ -183,7 +183,7 @@ def main():
     K, W = args.steps, args.warmup
     kv_dim, q_dim = Hk * D, H * D
     total_steps = W + K + K + 2          # warm-up, graph-timed, kernel-timed (eager), slack
-    msl = w["ctx"] + total_steps
+    msl = (w["ctx"] + total_steps + 255) // 256 * 256   # the engine's max_seq_len: context + room for the steps, rounded up
 
     lib = _lib.load()
     torch.cuda.set_device(0)

@@ -76,17 +76,32 @@ __device__ __forceinline__ long long cache_row(const int* __restrict__ block_tab
 // out evenly, so every chunk of one sequence has the same length to within one tile
 // whatever max_seq_len the caller allocated.  Empty (t0 >= t1) when n has fewer tiles
 // than nsplit.
+// Chunks 2j and 2j+1 do not split their tiles in halves but kPairShare : 64 - kPairShare.
+// The MFMA scan runs an even and the following odd chunk on the two wave groups of one CU,
+// and the group in the upper wave slots gets ~5 % less of the CU (measured; s_setprio does
+// not change it), so an even split leaves the lower group idle at the end.
+#ifndef TW_PAIR_SHARE
+#define TW_PAIR_SHARE 33
+#endif
+constexpr unsigned kPairShare = TW_PAIR_SHARE;
+__device__ __forceinline__ unsigned chunk_boundary(unsigned tiles, unsigned c, unsigned nsplit) {
+    if (c >= nsplit) return tiles;
+    if ((c & 1u) == 0) return (c * tiles) / nsplit;             // tiles * nsplit < 2^32 (nsplit <= 64)
+    const unsigned lo = ((c - 1) * tiles) / nsplit;
+    const unsigned hi = c + 1 >= nsplit ? tiles : ((c + 1) * tiles) / nsplit;
+    return lo + ((hi - lo) * kPairShare + 32u) / 64u;
+}
 __device__ __forceinline__ void chunk_range(int n, int c, int nsplit, int& t0, int& t1) {
-    const unsigned tiles = (unsigned)(n + 31) >> 5;             // tiles * nsplit < 2^32 (nsplit <= 64)
-    t0 = 32 * (int)(((unsigned)c * tiles) / (unsigned)nsplit);
-    int e = 32 * (int)(((unsigned)(c + 1) * tiles) / (unsigned)nsplit);
+    const unsigned tiles = (unsigned)(n + 31) >> 5;
+    t0 = 32 * (int)chunk_boundary(tiles, (unsigned)c, (unsigned)nsplit);
+    int e = 32 * (int)chunk_boundary(tiles, (unsigned)c + 1u, (unsigned)nsplit);
     t1 = e < n ? e : n;
 }
 // Does chunk c hold any token?  Always when the sequence has at least nsplit tiles.
 __device__ __forceinline__ bool chunk_nonempty(int n, int c, int nsplit) {
     const unsigned tiles = (unsigned)(n + 31) >> 5;
     if (tiles >= (unsigned)nsplit) return true;
-    return ((unsigned)(c + 1) * tiles) / (unsigned)nsplit > ((unsigned)c * tiles) / (unsigned)nsplit;
+    return chunk_boundary(tiles, (unsigned)c + 1u, (unsigned)nsplit) > chunk_boundary(tiles, (unsigned)c, (unsigned)nsplit);
 }
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -67,6 +67,12 @@ rotate_kernel(RotArgs a) {
     const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (dblk * 16 + i16) * kHeadDim);
     const uint4* xsrc = reinterpret_cast<const uint4*>(a.seg_src[seg] + (long long)row * a.seg_stride[seg] +
                                                        (long long)head * kHeadDim);
+    // cache row of this vector (its load overlaps the operand loads)
+    long long crow = 0;
+    if (!is_query) {
+        if (a.token_list) crow = a.positions[row];               // sequence 0, kernels.cu:1499, 1553
+        else crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, a.positions[row]);
+    }
     float rv[32], xv[32];
 #pragma unroll
     for (int q = 0; q < 16; q++) {
@@ -123,9 +129,6 @@ rotate_kernel(RotArgs a) {
     uint32_t p2 = (uint32_t)__shfl((int)packed, i16 + 32, 64);
     uint32_t p3 = (uint32_t)__shfl((int)packed, i16 + 48, 64);
     if (kk == 0 && v < nvec) {
-        long long crow;
-        if (a.token_list) crow = a.positions[row];               // sequence 0, kernels.cu:1499, 1553
-        else crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, a.positions[row]);
         constexpr int BPH = kHeadDim * BITS / 8;                  // bytes per head: 64 or 32
         uint8_t* dst = a.seg_codes[seg] + (crow * a.num_kv_heads + head) * BPH + dblk * (2 * BITS);
         if (BITS == 4) {
@@ -183,22 +186,39 @@ merge_rotate_kernel(AttnArgs a) {
         else if (a.pos_mode == kPosScalar) n = a.pos_scalar + 1;
         else n = g + 1;
         const float* part = a.ws + (long long)vv * a.ws_stride;
-        float mg = -1e30f;
-        for (int c = 0; c < a.nsplit; c++) {
-            if (chunk_nonempty(n, c, a.nsplit)) mg = fmaxf(mg, part[(long long)c * kPartialFloats + kHeadDim]);
-        }
-        float lsum = 0.0f;
+        // Chunks in blocks of 8 with every load of a block issued before the first use, so a
+        // block costs one memory latency rather than one per chunk; the running maximum is
+        // carried across blocks as in an online softmax.
+        float mg = -1e30f, lsum = 0.0f;
         float4 av = {0.f, 0.f, 0.f, 0.f};
-        for (int c = 0; c < a.nsplit; c++) {
-            if (!chunk_nonempty(n, c, a.nsplit)) continue;
-            const float* pc = part + (long long)c * kPartialFloats;
-            float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
-            lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);
-            float4 p4 = *reinterpret_cast<const float4*>(pc + k4);
-            av.x = __builtin_fmaf(p4.x, f, av.x);
-            av.y = __builtin_fmaf(p4.y, f, av.y);
-            av.z = __builtin_fmaf(p4.z, f, av.z);
-            av.w = __builtin_fmaf(p4.w, f, av.w);
+        for (int c0 = 0; c0 < a.nsplit; c0 += 8) {
+            float mc[8], lc[8];
+            float4 pc4[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int c = c0 + j;
+                const bool live = c < a.nsplit && chunk_nonempty(n, c, a.nsplit);   // else: no workgroup wrote this slot
+                const float* pc = part + (long long)(live ? c : 0) * kPartialFloats;
+                mc[j] = pc[kHeadDim];
+                lc[j] = pc[kHeadDim + 1];
+                pc4[j] = *reinterpret_cast<const float4*>(pc + k4);
+                if (!live) { mc[j] = -1e30f; lc[j] = 0.0f; pc4[j] = float4{0.f, 0.f, 0.f, 0.f}; }
+            }
+            float mb = mg;
+#pragma unroll
+            for (int j = 0; j < 8; j++) mb = fmaxf(mb, mc[j]);
+            const float fo = a.m_log2 ? __builtin_amdgcn_exp2f(mg - mb) : __expf(mg - mb);
+            lsum *= fo; av.x *= fo; av.y *= fo; av.z *= fo; av.w *= fo;
+            mg = mb;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                float f = a.m_log2 ? __builtin_amdgcn_exp2f(mc[j] - mg) : __expf(mc[j] - mg);
+                lsum = __builtin_fmaf(lc[j], f, lsum);
+                av.x = __builtin_fmaf(pc4[j].x, f, av.x);
+                av.y = __builtin_fmaf(pc4[j].y, f, av.y);
+                av.z = __builtin_fmaf(pc4[j].z, f, av.z);
+                av.w = __builtin_fmaf(pc4[j].w, f, av.w);
+            }
         }
         const float inv = 1.0f / (lsum + 1e-8f);
         float4 o4 = {av.x * inv, av.y * inv, av.z * inv, av.w * inv};
