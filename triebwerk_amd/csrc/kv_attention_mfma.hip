@@ -76,6 +76,7 @@ namespace {
 constexpr int kGroupWaves = 8;        // KV heads (waves) that walk one item together
 constexpr int kMaxWaves = 16;         // waves per workgroup: one workgroup per CU, two groups
 constexpr int kMaxGroup = 4;          // query heads per KV head handled by this kernel
+constexpr int kMaxBalanceSeqs = 4096; // sequences the balanced walk can index (16 KB of LDS)
 constexpr int kTableWords = 256 * 64; // 64 KB
 constexpr float kNegBig = -1e30f;
 // fp16(kAlpha4 * c) has max relative rounding error 1.05e-4 over the 4-bit table
@@ -135,6 +136,9 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
     // per wave: P[row][k] as fp16, rows 0..R-1 = heads, rows 8..8+R-1 = rounding remainders
     __shared__ __attribute__((aligned(16))) half_t p_s[kMaxWaves][16][32];
+    // balanced walk: tiles of the sequences before g, and {tiles per group, total tiles}
+    __shared__ int pre_s[kMaxBalanceSeqs + 1];
+    __shared__ int bal_s[2];
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
@@ -185,6 +189,15 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     const char *kseq = nullptr, *vseq = nullptr, *knseq = nullptr, *vnseq = nullptr;
     const int* bt = nullptr;
     long long seq_row0 = 0;
+    int nseg = 0;                                             // balanced walk: partials sequence g gets; 0 = even chunks
+    auto set_bases = [&]() {                                  // scalar bases of this wave's head
+        kseq = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes;
+        vseq = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes;
+        knseq = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
+        vnseq = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
+        bt = PAGED ? a.block_table + (long long)g * a.bt_stride : nullptr;
+        seq_row0 = (long long)g * a.seq_stride_rows;
+    };
     auto decode = [&](int item) -> bool {                    // false: the chunk holds no token
         const int hg = item % hgroups;
         chunk = (item / hgroups) % a.nsplit;
@@ -193,13 +206,27 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
         n = uniform(seq_pos(a, g)) + 1;
         chunk_range(n, chunk, a.nsplit, t0, t1);
         if (t0 >= t1) return false;
-        // scalar bases of this wave's head
-        kseq = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes;
-        vseq = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes;
-        knseq = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
-        vnseq = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
-        bt = PAGED ? a.block_table + (long long)g * a.bt_stride : nullptr;
-        seq_row0 = (long long)g * a.seq_stride_rows;
+        set_bases();
+        return true;
+    };
+    // Balanced walk (ragged batches).  All 32-token tiles of all sequences form one list; every
+    // group of waves takes `quota` consecutive tiles of it, cut where a sequence ends.  The piece
+    // of sequence g that group number gb takes is partial gb - (tiles before g) / quota of g.
+    int bal_cur = 0, bal_end = 0, bal_g = 0, bal_quota = 1, bal_gb = 0;
+    auto next_piece = [&]() -> bool {
+        if (bal_cur >= bal_end) return false;
+        while (pre_s[bal_g + 1] <= bal_cur) bal_g++;
+        g = bal_g;
+        const int first = pre_s[g], last = pre_s[g + 1];
+        const int stop = min(bal_end, last);
+        n = uniform(seq_pos(a, g)) + 1;
+        t0 = 32 * (bal_cur - first);
+        t1 = min(32 * (stop - first), n);
+        chunk = bal_gb - first / bal_quota;
+        nseg = (last - 1) / bal_quota - first / bal_quota + 1;
+        bal_cur = stop;
+        h = wv;
+        set_bases();
         return true;
     };
 
@@ -312,11 +339,48 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
         }
     };
 
-    // The first loads of the first item are in flight while the workgroup builds its table.
+    // Even chunks or balanced walk?  Every wave looks at the spread of the sequence lengths
+    // itself (cheap), so that in the even case its first loads are in flight while the
+    // workgroup builds its table; wave 0 also leaves the prefix of tiles in LDS.
+    bool balanced = false;
+    if (a.balance) {
+        int carry = 0, tmin = 0x7fffffff, tmax = 0;
+        for (int base = 0; base < a.G; base += kWave) {
+            const int gg = base + lane;
+            const int t = gg < a.G ? (seq_pos(a, gg) + 1 + 31) >> 5 : 0;
+            if (gg < a.G) { tmin = min(tmin, t); tmax = max(tmax, t); }
+            if (wave == 0) {
+                int inc = t;
+#pragma unroll
+                for (int off = 1; off < kWave; off <<= 1) {
+                    int up = __shfl_up(inc, off, 64);
+                    if (lane >= off) inc += up;
+                }
+                if (gg < a.G) pre_s[gg + 1] = carry + inc;
+                carry += __shfl(inc, kWave - 1, 64);
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            tmin = min(tmin, __shfl_xor(tmin, off, 64));
+            tmax = max(tmax, __shfl_xor(tmax, off, 64));
+        }
+        balanced = uniform((tmax - tmin) * 8 > tmax ? 1 : 0) != 0;   // even chunks serve (nearly) equal lengths better
+        if (wave == 0 && lane == 0) {
+            pre_s[0] = 0;
+            const int groups = (int)gridDim.x * ngroups;
+            const int quota = (carry + groups - 1) / groups;
+            const int by_slots = (tmax + a.max_slots - 2) / (a.max_slots - 1);   // a sequence gets <= max_slots pieces
+            bal_s[0] = max(max(quota, by_slots), 1);
+            bal_s[1] = carry;
+        }
+    }
+    // The first loads of the first item are in flight while the workgroup builds its table
+    // (not in the balanced walk, whose first piece is only known after the barrier).
     const int item_step = (int)gridDim.x * ngroups;
     int item = (int)blockIdx.x * ngroups + grp;
     bool ready = false;          // the item is decoded, holds tokens, and its first loads are issued
-    if (item < total_items && decode(item)) {
+    if (!balanced && item < total_items && decode(item)) {
         issue_first();
         ready = true;
     }
@@ -337,12 +401,33 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     for (int i = tid; i < kMaxWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
     __syncthreads();             // the only workgroup-wide barrier; every wave reaches it
 
-    for (; item < total_items; item += item_step) {
-        if (!ready) {
-            if (!decode(item)) continue;                      // uniform over the wave
-            issue_first();
+    if (balanced) {
+        bal_quota = bal_s[0];
+        bal_gb = (int)blockIdx.x * ngroups + grp;
+        const long long start = (long long)bal_gb * bal_quota;
+        bal_cur = (int)min(start, (long long)bal_s[1]);
+        bal_end = (int)min(start + bal_quota, (long long)bal_s[1]);
+        int lo = 0, hi = a.G;                                 // last sequence that starts at or before bal_cur
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (pre_s[mid] <= bal_cur) lo = mid; else hi = mid;
         }
-        ready = false;
+        bal_g = lo;
+    }
+
+    for (;;) {
+        if (balanced) {
+            if (!next_piece()) break;
+            issue_first();
+        } else {
+            if (item >= total_items) break;
+            if (!ready) {
+                if (!decode(item)) { item += item_step; continue; }   // uniform over the wave
+                issue_first();
+            }
+            ready = false;
+            item += item_step;
+        }
         const int ntiles = (t1 - t0 + 31) >> 5;
 
         float4_t o[8];
@@ -541,6 +626,9 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
                 if (ln == 0) {
                     part[kHeadDim] = m_run[r];
                     part[kHeadDim + 1] = l_run[r];
+                    // whoever holds the sequence's first token tells the merge, in the spare word of
+                    // partial 0, how many partials there are (0: even chunks)
+                    if (t0 == 0) reinterpret_cast<int*>(part - (long long)chunk * kPartialFloats)[kHeadDim + 2] = balanced ? nseg : 0;
                 }
             }
         }
@@ -583,6 +671,9 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     if (items <= 0 || items > 0x7fffffff) return false;
     a.force_merge = 1;
     a.m_log2 = 1;
+    a.slots_from_ws = 1;
+    // ragged batches: cut the work by tiles, not by sequence (decided on the device from the positions)
+    a.balance = (a.num_kv_heads == scan_waves(a) && a.G <= kMaxBalanceSeqs && a.max_slots >= 3 && a.G > 1) ? 1 : 0;
     if (rotate_query) {
         RotArgs r;
         memset(&r, 0, sizeof(r));

@@ -267,13 +267,17 @@ attention_merge_kernel(AttnArgs a) {
     const int head = blockIdx.x, g = blockIdx.y, d = threadIdx.x;
     const int n = seq_pos(a, g) + 1;
     const float* part = a.ws + ((long long)g * a.num_heads + head) * a.ws_stride;
+    // which slots were written: the first nseg (balanced MFMA scan) or the non-empty even chunks
+    const int nseg = a.slots_from_ws ? reinterpret_cast<const int*>(part)[kHeadDim + 2] : 0;
+    auto live = [&](int c) -> bool { return nseg > 0 ? c < nseg : chunk_nonempty(n, c, a.nsplit); };
+    const int nslots = nseg > 0 ? nseg : a.nsplit;
     float mg = kNegBig;
-    for (int cidx = 0; cidx < a.nsplit; cidx++) {
-        if (chunk_nonempty(n, cidx, a.nsplit)) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
+    for (int cidx = 0; cidx < nslots; cidx++) {
+        if (live(cidx)) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
     }
     float lsum = 0.0f, av = 0.0f;
-    for (int cidx = 0; cidx < a.nsplit; cidx++) {
-        if (!chunk_nonempty(n, cidx, a.nsplit)) continue;   // no workgroup wrote this slot
+    for (int cidx = 0; cidx < nslots; cidx++) {
+        if (!live(cidx)) continue;                          // no workgroup wrote this slot
         const float* pc = part + (long long)cidx * kPartialFloats;
         float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
         lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);

@@ -96,8 +96,18 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     if (!have_ws) nsplit = 1;
     a.nsplit = nsplit;
     a.chunk_len = 0;   // chunks are cut per sequence on the device (chunk_range)
+    // The MFMA scan may cut a ragged batch into up to max_slots pieces per sequence instead
+    // (a long sequence among short ones takes several groups' worth of tiles).
+    int slots = nsplit;
+    if (have_ws && mfma && a.pos_mode != kPosScalar) {
+        slots = 4 * nsplit + 2;
+        if (slots > max_by_ws) slots = max_by_ws;
+        if (slots > kMaxSplits) slots = kMaxSplits;
+        if (slots < nsplit) slots = nsplit;
+    }
+    a.max_slots = slots;
     if (have_ws) {
-        long long qoff = ((long long)nsplit * kPartialFloats + 3) & ~3LL;
+        long long qoff = ((long long)slots * kPartialFloats + 3) & ~3LL;
         a.ws_stride = qoff + kHeadDim;
         a.qrot = a.ws + qoff;
     } else {

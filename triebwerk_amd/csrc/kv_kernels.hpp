@@ -85,6 +85,9 @@ struct AttnArgs {
     int chunk_len;          // tokens per split, multiple of 64
     int force_merge;        // the scan kernel wrote partials even though nsplit == 1
     int m_log2;             // partial maxima are in base-2 units
+    int balance;            // MFMA scan: may cut the batch by tiles instead of by sequence (ragged lengths)
+    int max_slots;          // partials the workspace holds per (sequence, head): >= nsplit
+    int slots_from_ws;      // merge: the spare word of partial 0 holds the number of partials (0: even chunks)
 };
 
 constexpr int kPartialFloats = kHeadDim + 4;  // acc[128], running max, running sum, 2 pad (16-byte rows)

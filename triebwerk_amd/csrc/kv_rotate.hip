@@ -186,18 +186,21 @@ merge_rotate_kernel(AttnArgs a) {
         else if (a.pos_mode == kPosScalar) n = a.pos_scalar + 1;
         else n = g + 1;
         const float* part = a.ws + (long long)vv * a.ws_stride;
+        const int nseg = a.slots_from_ws ? reinterpret_cast<const int*>(part)[kHeadDim + 2] : 0;
         // Chunks in blocks of 8 with every load of a block issued before the first use, so a
         // block costs one memory latency rather than one per chunk; the running maximum is
         // carried across blocks as in an online softmax.
         float mg = -1e30f, lsum = 0.0f;
         float4 av = {0.f, 0.f, 0.f, 0.f};
-        for (int c0 = 0; c0 < a.nsplit; c0 += 8) {
+        const int nslots = nseg > 0 ? nseg : a.nsplit;
+        for (int c0 = 0; c0 < nslots; c0 += 8) {
             float mc[8], lc[8];
             float4 pc4[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const int c = c0 + j;
-                const bool live = c < a.nsplit && chunk_nonempty(n, c, a.nsplit);   // else: no workgroup wrote this slot
+                // else: no workgroup wrote this slot
+                const bool live = c < nslots && (nseg > 0 || chunk_nonempty(n, c, a.nsplit));
                 const float* pc = part + (long long)(live ? c : 0) * kPartialFloats;
                 mc[j] = pc[kHeadDim];
                 lc[j] = pc[kHeadDim + 1];
