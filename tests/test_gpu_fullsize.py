@@ -230,3 +230,38 @@ def test_tq2_gqa4_context4097(kv, oracle, rotation_fixture):
     oracle.turbo_gqa_attention_batch(want, q, ock, ocv, okn, ovn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
     err = rel_err_rows(host(out), want)
     assert err.max() <= TOL, f"max rel err {err.max():.3e}"
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_extremely_ragged_batch(kv, oracle, rotation_fixture, bits):
+    """Lengths from 1 token to 8192 in one batch of 100: the scan cuts such a batch by tiles, not
+    by sequence, and a sequence's partials come from a varying number of wave groups."""
+    import torch
+    G, H, Hk = 100, 16, 8
+    kv_dim, q_dim = Hk * D, H * D
+    kvp = kv_dim * bits // 8
+    msl = 8192
+    r = gen.rng(980 + bits)
+    lens = np.concatenate([np.array([1, 2, 31, 32, 33, 63, 64, 65, 8192, 8191, 4097, 1000]),
+                           r.integers(1, 300, size=G - 12)]).astype(np.int32)
+    r.shuffle(lens)
+    g_ = torch.Generator(device="cuda"); g_.manual_seed(981 + bits)
+    ck = torch.randint(0, 256, (G, msl, kvp), generator=g_, device="cuda", dtype=torch.uint8)
+    cv = torch.randint(0, 256, (G, msl, kvp), generator=g_, device="cuda", dtype=torch.uint8)
+    kn = (11.3 + 0.7 * torch.randn((G, msl, Hk), generator=g_, device="cuda")).to(torch.float16)
+    vn = (11.3 + 0.7 * torch.randn((G, msl, Hk), generator=g_, device="cuda")).to(torch.float16)
+    rot = dev(rotation_fixture)
+    pos = (lens - 1).astype(np.int32)
+    q = gen.normal_f16(r, (G, q_dim))
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, host(ck), host(cv), host(kn), host(vn), rotation_fixture, pos, msl, G, H, Hk,
+                                     D, q_dim, kv_dim, bits)
+    scratch = torch.full((G * H * msl,), float("nan"), dtype=torch.float32, device="cuda")   # nothing may rely on its content
+    for variant in (0, 1):
+        kv.set_attention_variant(variant)
+        out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+        kv.launch_turbo_gqa_attention_batch(out, dev(q), ck, cv, kn, vn, rot, scratch, dev(pos), msl, G, H, Hk, D,
+                                            q_dim, kv_dim, bits)
+        err = rel_err_rows(host(out), want)
+        assert err.max() <= TOL, f"variant {variant}: max rel err {err.max():.3e} (sequence {err.argmax() // H}, length {lens[err.argmax() // H]})"
+    kv.set_attention_variant(0)
