@@ -281,6 +281,25 @@ def main():
     launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=False) / (Kp * L)
     achieved = launch_bytes / (kern_ms * 1e-3) * 1e-9
 
+    # ---- what a plain contiguous read kernel reaches on this GPU: over 4 GiB, and over exactly the
+    # scan's bytes per launch on memory not touched since (launch overheads included, as for the scan)
+    probe = torch.empty(int(4 << 30), dtype=torch.uint8, device="cuda")
+    probe.fill_(1)
+    torch.cuda.synchronize()
+    lib.tw_kv_measure_read_bandwidth.restype = C.c_double
+    read_big = lib.tw_kv_measure_read_bandwidth(C.c_void_p(probe.data_ptr()), C.c_size_t(probe.numel()), 3,
+                                                C.c_void_p(stream.cuda_stream))
+    nb = int(launch_bytes) // 16 * 16
+    same, reps = 0.0, 0
+    for off in range(0, probe.numel() - nb + 1, max(nb, 1) + (1 << 20)):
+        same += lib.tw_kv_measure_read_bandwidth(C.c_void_p(probe.data_ptr() + off // 16 * 16), C.c_size_t(nb), 1,
+                                                 C.c_void_p(stream.cuda_stream))
+        reps += 1
+        if reps == 6:
+            break
+    read_same = same / max(reps, 1)
+    del probe
+
     result = {
         "metric": "decode-attn tokens/s",
         "value": tokens_per_s,
@@ -316,6 +335,8 @@ def main():
             "frac": achieved / HBM_PEAK_GBS,
             "launch_ms": kern_ms,
             "launch_algorithmic_MB": launch_bytes * 1e-6,
+            "plain_read_GBps_4GiB": read_big,
+            "plain_read_GBps_same_bytes_per_launch": read_same,
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, kv_bits)) if not overridden else None,
         },
     }

@@ -139,6 +139,12 @@ void tw_kv_set_num_splits(int nsplit);
 void tw_kv_profile_attention(int enable);
 int tw_kv_profile_read(double* total_ms, int* launches);
 
+/* No counterpart in the reference.  Rate (GB/s) at which this GPU streams `bytes` of device
+ * memory through a plain contiguous 16-byte-per-lane read kernel, averaged over `iters`
+ * launches and timed with HIP events on `s`; blocks until done.  The benchmark quotes it as
+ * the practical ceiling beside the published HBM peak.  Returns 0 on error. */
+double tw_kv_measure_read_bandwidth(const void* dev_buf, size_t bytes, int iters, hipStream_t s);
+
 /* Floats of workspace the *_ws / paged attention entry points need for a
  * (G, num_heads, max_context) problem at the automatic split count.  The
  * reference-signature launchers instead fit their split count to the

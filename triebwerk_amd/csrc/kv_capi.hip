@@ -151,6 +151,13 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done =
     }
     check_launch(fn);
 }
+int compute_units_host() {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    return cus;
+}
 }  // namespace
 
 extern "C" {
@@ -180,6 +187,50 @@ int tw_kv_profile_read(double* total_ms, int* launches) {
     if (launches) *launches = g_prof.used;
     g_prof.used = 0;
     return 0;
+}
+
+// A plain streaming read of [buf, buf + bytes): 16 bytes per lane, eight loads in flight,
+// grid-stride.  What this GPU delivers for the friendliest possible access pattern; the
+// benchmark quotes it next to the scan's rate.
+__device__ unsigned g_stream_read_sink;
+__global__ void __launch_bounds__(512) stream_read_kernel(const uint4* __restrict__ src, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    unsigned acc = 0;
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = src[i + j * stride];
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+    }
+    for (; i < n16; i += stride) { uint4 v = src[i]; acc ^= v.x ^ v.y ^ v.z ^ v.w; }
+    if (acc == 0x9e3779b9u) g_stream_read_sink = acc;   // keeps the loads alive; practically never taken
+}
+
+double tw_kv_measure_read_bandwidth(const void* dev_buf, size_t bytes, int iters, hipStream_t s) {
+    if (!dev_buf || bytes < 16 || iters < 1 || (reinterpret_cast<uintptr_t>(dev_buf) & 15u) != 0) {
+        set_error(1, "tw_kv_measure_read_bandwidth: needs a 16-byte aligned device buffer and iters >= 1");
+        return 0.0;
+    }
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return 0.0;
+    const size_t n16 = bytes / 16;
+    const int bpc = 4, thr = 512;                 // the best of several shapes tried on MI355X
+    const int grid = compute_units_host() * bpc;
+    hipLaunchKernelGGL(stream_read_kernel, dim3(grid), dim3(thr), 0, s, reinterpret_cast<const uint4*>(dev_buf), n16);
+    hipEventRecord(e0, s);
+    for (int i = 0; i < iters; i++)
+        hipLaunchKernelGGL(stream_read_kernel, dim3(grid), dim3(thr), 0, s, reinterpret_cast<const uint4*>(dev_buf), n16);
+    hipEventRecord(e1, s);
+    float ms = 0.0f;
+    double gbps = 0.0;
+    if (hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess && ms > 0.0f)
+        gbps = (double)n16 * 16.0 * iters / (ms * 1e-3) * 1e-9;
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    check_launch("tw_kv_measure_read_bandwidth");
+    return gbps;
 }
 
 size_t tw_attention_workspace_floats(int G, int num_heads, int max_context) {
