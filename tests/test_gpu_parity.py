@@ -388,6 +388,29 @@ def test_turbo_prefill_attention(kv, oracle, rotation_fixture, bits):
     assert rel_err(host(out), want) <= TOL
 
 
+@pytest.mark.parametrize("bits,H,Hk,T", [(4, 16, 8, 700), (2, 16, 8, 645), (4, 8, 2, 601), (2, 4, 4, 530), (4, 4, 1, 1111)])
+def test_turbo_prefill_attention_long(kv, oracle, rotation_fixture, bits, H, Hk, T):
+    """Prompts long enough for the scratch (T floats per query token and head) to hold split
+    partials: the prefill runs on the matrix cores, several query tokens per wave, for
+    GQA groups of 2, 4 and 1 and prompt lengths that are not multiples of the token block."""
+    import torch
+    r = gen.rng(340 + bits + H + T)
+    msl = T + 3
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, 1, Hk, msl, [T], bits)
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    oracle.turbo_gqa_prefill_attention(want, q, ck[0], cv[0], kn[0], vn[0], rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+    scratch = torch.full((T * H * T,), float("nan"), dtype=torch.float32, device="cuda")
+    for variant in (0, 1):
+        kv.set_attention_variant(variant)
+        out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+        kv.launch_turbo_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), dev(kn[0]), dev(vn[0]),
+                                              dev(rotation_fixture), scratch, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+        assert rel_err(host(out), want) <= TOL, f"variant {variant}"
+    kv.set_attention_variant(0)
+
+
 @pytest.mark.parametrize("bits", [4, 2])
 def test_golden_case_on_gpu(kv, rotation_fixture, bits):
     """Committed vectors: append 37 tokens on the GPU, compare every byte, then attention."""

@@ -694,6 +694,10 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
 }
 
 void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
+    if (prefill_mfma_usable(a)) {
+        launch_prefill_mfma_scan(a, s);
+        return;
+    }
     const int waves = scan_waves(a);
     const int hgroups = a.num_kv_heads / waves;
     const int items = a.G * a.nsplit * hgroups;

@@ -100,5 +100,8 @@ bool launch_merge_rotate(const AttnArgs& a, hipStream_t s);   // MFMA merge + ro
 bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query);
 float attention_mfma_q_scale(int bits);
 void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);
+// causal prefill with blocks of query tokens per wave (kv_prefill_mfma.hip); same workspace and merge
+bool prefill_mfma_usable(const AttnArgs& a);
+void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s);
 
 }  // namespace twkv
