@@ -66,6 +66,7 @@
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
+#include "kv_mfma_util.hpp"
 
 #include <cstring>
 
@@ -73,19 +74,7 @@ namespace twkv {
 
 namespace {
 
-constexpr int kGroupWaves = 8;        // KV heads (waves) that walk one item together
-constexpr int kMaxWaves = 16;         // waves per workgroup: one workgroup per CU, two groups
 constexpr int kMaxGroup = 4;          // query heads per KV head handled by this kernel
-constexpr int kMaxBalanceSeqs = 4096; // sequences the balanced walk can index (16 KB of LDS)
-constexpr int kTableWords = 256 * 64; // 64 KB
-constexpr float kNegBig = -1e30f;
-// fp16(kAlpha4 * c) has max relative rounding error 1.05e-4 over the 4-bit table
-// (exhaustive search over the fp32 values of one octave).
-constexpr float kAlpha4 = 19.391284942626953f;
-// the same for the 2-bit table: 1.1e-7
-constexpr float kAlpha2 = 25.46918296813965f;
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kInvSqrtD = 0.08838834764831845f;
 // Tiles of loads in flight per wave.  Deeper is only safe while nothing spills: a spilled
 // register is reloaded through the same in-order memory counter as the prefetched tiles,
 // so every reload waits for all of them.
@@ -95,34 +84,6 @@ constexpr float kInvSqrtD = 0.08838834764831845f;
 #ifndef TW_DEPTH2
 #define TW_DEPTH2 1
 #endif
-
-__device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
-    if (a.pos_mode == kPosArray) return a.positions[g];
-    if (a.pos_mode == kPosScalar) return a.pos_scalar;
-    return g;
-}
-
-
-__device__ __forceinline__ float h2f_bits(uint32_t bits16) {
-    union { uint16_t u; half_t h; } cv;
-    cv.u = (uint16_t)bits16;
-    return (float)cv.h;
-}
-
-__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
-
-typedef uint32_t uint32x4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t uint32x2_t __attribute__((ext_vector_type(2)));
-
-// Buffer descriptor over [base, base + bytes).  Every input is forced into scalar
-// registers: a descriptor held in vector registers makes each load a serialising loop.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const char* base, int bytes) {
-    uint64_t p = reinterpret_cast<uint64_t>(base);
-    uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)p);
-    uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32));
-    char* q = reinterpret_cast<char*>(((uint64_t)hi << 32) | lo);
-    return __builtin_amdgcn_make_buffer_rsrc(q, 0, __builtin_amdgcn_readfirstlane(bytes), 0x00020000);
-}
 
 }  // namespace
 
@@ -635,7 +596,7 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     }
 }
 
-static int compute_units() {
+int compute_units() {
     static int cached = 0;
     if (cached == 0) {
         int dev = 0, cus = 0;
