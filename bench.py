@@ -50,7 +50,7 @@ BYTES_HEAD = {0: 256, 4: 66, 2: 34}  # per (token, kv head): fp16 row | codes + 
 # and WRITE_SIZE on this file's own run, each counter scaled by what `--copy-calibration` reads for a
 # copy of known size (2.0 and 1.0); summary and commands in profiles/scan_target_hbm_traffic_pmc.txt.
 # Keyed by (workload, kv_bits); a measurement of the kernels as committed with that file, not live.
-MEASURED_TRAFFIC_BYTES = {("target", 4): 560.6e6, ("target", 2): 291.9e6, ("target", 0): 2151.2e6}
+MEASURED_TRAFFIC_BYTES = {("target", 4): 560.8e6, ("target", 2): 292.3e6, ("target", 0): 2151.2e6}
 
 
 def algorithmic_bytes(n_tokens_total: int, G: int, L: int, H: int, Hk: int, kv_bits: int, with_append: bool) -> int:
