@@ -41,11 +41,16 @@
 //      offset fixed for the whole kernel); pages of the paged layout only change
 //      the scalar base.
 //   scheduling: one persistent workgroup of 16 waves per CU.  Its waves form two groups of
-//      8 (one KV head per wave); each group walks its own list of (sequence, chunk, head
-//      group) items, so the 64 KB table is built once per CU and waves never synchronise
-//      after that.  Measured: the waves in the upper wave slots of a CU (the second group,
-//      or a second workgroup) run ~5 % slower than the lower ones whatever their s_setprio,
-//      so the kernel ends with half of each CU idle for the last ~5 % of its time.
+//      8 (one KV head per wave); each group walks its own list of items, so the 64 KB table
+//      is built once per CU and waves never synchronise after that.  Items are cut one of
+//      two ways, chosen on the device from the positions: even chunks (every sequence into
+//      nsplit chunks of 32-token tiles; item = sequence, chunk, head group) when the lengths
+//      are within 1/8 of each other, else the balanced walk (all tiles of all sequences in
+//      one list, an equal run per group, cut where a sequence ends), whose pieces number
+//      the partials of a sequence 0, 1, 2, ...  Measured: the waves in the upper wave slots
+//      of a CU (the second group, or a second workgroup) run ~5 % slower than the lower ones
+//      whatever their s_setprio; chunk_range therefore gives even chunks 33/64 and odd
+//      chunks 31/64 of a pair's tiles.
 //   precision: fp16 operands would cost ~5e-4 relative error each for q_rot and for
 //      the probabilities.  Both are split into hi + lo fp16 parts that ride in MFMA
 //      rows the GQA group leaves empty (head n -> row n and n+8), so the split costs
@@ -61,8 +66,10 @@
 //      n^1 share dwords, so each loads the dword of two of the four tokens and they trade
 //      halves with one DPP move.  Index bytes hold (token a dims d,d+1 | token b dims d,d+1),
 //      so one look-up returns the B-operand dwords (a,b) of dim d and of dim d+1.
-// The partial (acc[128], max, sum) per (sequence, head, chunk) goes to the split
-// workspace; merge_rotate_kernel combines, normalises and rotates back.
+// The partial (acc[128], max, sum) per (sequence, head, chunk or piece) goes to the split
+// workspace; merge_rotate_kernel combines, normalises and rotates back.  The wave that holds
+// a sequence's first token also leaves, in a spare word of partial 0, how many partials the
+// sequence has (0 = even chunks, where chunk_nonempty tells).
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"

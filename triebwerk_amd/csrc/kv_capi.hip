@@ -95,7 +95,6 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     if (have_ws && nsplit > max_by_ws) nsplit = max_by_ws;
     if (!have_ws) nsplit = 1;
     a.nsplit = nsplit;
-    a.chunk_len = 0;   // chunks are cut per sequence on the device (chunk_range)
     // The MFMA scan may cut a ragged batch into up to max_slots pieces per sequence instead
     // (a long sequence among short ones takes several groups' worth of tiles).
     int slots = nsplit;

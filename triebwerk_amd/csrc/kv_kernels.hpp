@@ -82,7 +82,6 @@ struct AttnArgs {
     long long ws_stride;    // floats per (g, head) block
     float* qrot;            // ws + offset of q_rot inside a block (128 floats), or NULL
     int nsplit;             // >= 1; 1 = no workspace, one workgroup walks the sequence
-    int chunk_len;          // tokens per split, multiple of 64
     int force_merge;        // the scan kernel wrote partials even though nsplit == 1
     int m_log2;             // partial maxima are in base-2 units
     int balance;            // MFMA scan: may cut the batch by tiles instead of by sequence (ragged lengths)
