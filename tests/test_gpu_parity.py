@@ -602,3 +602,20 @@ def test_engine_prefix_broadcast(oracle):
     for g in range(1, G):
         assert np.array_equal(k[g, :T], k[0, :T]) and np.array_equal(n[g, :T], n[0, :T])
         assert not k[g, T:].any()
+
+
+def test_plain_read_bandwidth_probe(kv):
+    """The calibration kernel the benchmark quotes: plausible on a large buffer, an error on a bad one."""
+    import ctypes as C
+    import torch
+    from triebwerk_amd import _lib
+    lib = _lib.load()
+    buf = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    gbps = lib.tw_kv_measure_read_bandwidth(C.c_void_p(buf.data_ptr()), C.c_size_t(buf.numel()), 2, C.c_void_p(s))
+    assert 1000.0 < gbps < 8000.0, gbps          # above any PCIe or cache-less rate, below the HBM peak
+    assert torch.all(buf == 1)                   # it only reads
+    lib.tw_kv_clear_error()
+    assert lib.tw_kv_measure_read_bandwidth(C.c_void_p(buf.data_ptr() + 1), C.c_size_t(1 << 20), 1, C.c_void_p(s)) == 0.0
+    assert lib.tw_kv_last_error() != 0
+    lib.tw_kv_clear_error()
