@@ -58,8 +58,9 @@ def test_engine_kv_bits_switch(capfd):
 
 
 def test_cache_sizes_match_the_reference_readme():
-    """README.md:163-168: G=4, 28 layers: 1,024 tokens fp16 448 MiB -> TQ4 ~116 MiB;
-    8,192 tokens TQ4 ~1,005 MiB (1056 bytes per token per layer)."""
+    """README.md:163-165: G=4, 28 layers, 1,024 tokens: fp16 448 MB, TQ4 116 MB.  The table's longer
+    rows are not 8x those (8,192 tokens: 3,893 / 1,005 MB), so beyond the first row the test checks the
+    arithmetic the layout fixes: 4096 | 1056 | 544 bytes per token and layer."""
     from triebwerk_amd import _lib
     lib = _lib.load()
 
