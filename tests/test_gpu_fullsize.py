@@ -148,13 +148,14 @@ def test_target_shape_fp16_cache(kv, oracle):
     assert err.max() <= TOL, f"max rel err {err.max():.3e}"
 
 
-def test_ragged_paged_batch64(kv, oracle, rotation_fixture):
-    """Contexts uniform in [512, 8192], 16-token pages in random order (4-bit)."""
+@pytest.mark.parametrize("bits", [4, 2])
+def test_ragged_paged_batch64(kv, oracle, rotation_fixture, bits):
+    """Contexts uniform in [512, 8192], 16-token pages in random order."""
     import torch
-    bits, G, H, Hk = 4, 64, 16, 8
+    G, H, Hk = 64, 16, 8
     kv_dim, q_dim = Hk * D, H * D
     kvp = kv_dim * bits // 8
-    r = gen.rng(960)
+    r = gen.rng(960 + bits)
     lens = gen.ragged_contexts(r, G, 512, 8192)
     lens[0], lens[1] = 512, 8192
     pages_per_seq = 8192 // 16

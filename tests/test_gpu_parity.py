@@ -515,6 +515,58 @@ def test_paged_cache_equals_contiguous(kv, oracle, rotation_fixture, bits):
     assert rel_err(host(out), want) <= TOL
 
 
+@pytest.mark.parametrize("ragged", [False, True])
+@pytest.mark.parametrize("H", [8, 16, 32])
+def test_tq2_eight_kv_heads_paged_and_contiguous(kv, oracle, rotation_fixture, H, ragged):
+    """2-bit cache with 8 KV heads (256-byte rows: the scan whose waves load whole rows together), GQA
+    groups of 1, 2 and 4, over shuffled 16-token pages and over the contiguous layout, with nearly equal
+    lengths (even chunks) and with very unequal ones (balanced walk), for several split counts."""
+    import torch
+    bits, Hk = 2, 8
+    r = gen.rng(430 + H + int(ragged))
+    lens = np.array([1, 15, 16, 17, 31, 32, 33, 64, 65, 700, 1023, 1024] if ragged else [1000, 1001, 1023, 1024, 990, 1024])
+    G = len(lens)
+    kv_dim, q_dim = Hk * D, H * D
+    pages_per_seq = 64
+    msl = pages_per_seq * 16
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits, outliers=False)
+    bt = gen.shuffled_block_table(r, G, pages_per_seq)
+    n_pages = G * pages_per_seq
+
+    def scatter(contig, width, dtype):
+        pool = np.full((n_pages, 16, width), 0, dtype)
+        for g in range(G):
+            for i in range(pages_per_seq):
+                pool[bt[g, i]] = contig[g, 16 * i:16 * (i + 1)]
+        return pool
+
+    p_ck, p_cv = dev(scatter(ck, kv_dim // 4, np.uint8)), dev(scatter(cv, kv_dim // 4, np.uint8))
+    p_kn, p_vn = dev(scatter(kn, Hk, np.float16)), dev(scatter(vn, Hk, np.float16))
+    q = gen.normal_f16(r, (G, q_dim))
+    pos = (lens - 1).astype(np.int32)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    rot, d_q, d_pos, d_bt = dev(rotation_fixture), dev(q), dev(pos), dev(bt)
+    d_c = [dev(x) for x in (ck, cv, kn, vn)]
+    ws = torch.full((kv.attention_workspace_floats(G, H, msl),), float("nan"), dtype=torch.float32, device="cuda")
+    try:
+        for nsplit in (0, 1, 3, 8):
+            kv.set_num_splits(nsplit)
+            out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+            kv.tw_paged_turbo_gqa_attention_batch(out, d_q, p_ck, p_cv, p_kn, p_vn, rot, ws, d_pos, d_bt,
+                                                  pages_per_seq, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+            err = rel_err(host(out), want)
+            assert err <= TOL, f"paged, nsplit={nsplit}: {err}"
+            out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+            scratch = torch.full((G * H * msl,), float("nan"), dtype=torch.float32, device="cuda")
+            kv.launch_turbo_gqa_attention_batch(out, d_q, d_c[0], d_c[1], d_c[2], d_c[3], rot, scratch, d_pos, msl, G, H, Hk,
+                                                D, q_dim, kv_dim, bits)
+            err = rel_err(host(out), want)
+            assert err <= TOL, f"contiguous, nsplit={nsplit}: {err}"
+    finally:
+        kv.set_num_splits(0)
+
+
 # ------------------------------------------------------------------ engine: append -> attention -> positions, eager and graph
 @pytest.mark.parametrize("kv_bits", [0, 4, 2])
 @pytest.mark.parametrize("use_graph", [False, True])

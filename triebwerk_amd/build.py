@@ -24,6 +24,7 @@ SOURCES = [
     "kv_append.hip",
     "kv_attention_valu.hip",
     "kv_attention_mfma.hip",
+    "kv_attention_mfma2c.hip",
     "kv_prefill_mfma.hip",
     "kv_rotate.hip",
     "kv_capi.hip",

@@ -666,6 +666,10 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
         launch_prefill_mfma_scan(a, s);
         return;
     }
+    if (attention_mfma2c_usable(a)) {
+        launch_attention_mfma2c_scan(a, s);
+        return;
+    }
     const int waves = scan_waves(a);
     const int hgroups = a.num_kv_heads / waves;
     const int items = a.G * a.nsplit * hgroups;

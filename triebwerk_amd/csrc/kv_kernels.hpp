@@ -102,5 +102,8 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);
 // causal prefill with blocks of query tokens per wave (kv_prefill_mfma.hip); same workspace and merge
 bool prefill_mfma_usable(const AttnArgs& a);
 void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s);
+// 2-bit decode scan for 8 KV heads whose waves load whole cache rows together (kv_attention_mfma2c.hip)
+bool attention_mfma2c_usable(const AttnArgs& a);
+void launch_attention_mfma2c_scan(const AttnArgs& a, hipStream_t s);
 
 }  // namespace twkv
