@@ -147,6 +147,9 @@ def main():
     ap.add_argument("--nsplit", type=int, default=0)
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--producers", default="none", choices=["none", "fused", "separate"],
+                    help="also run QK RMSNorm + RoPE each layer: fused into the append, or as the reference's two "
+                         "launches (not part of the metric's definition; off by default)")
     ap.add_argument("--ctx", type=int, default=None, help="override the workload's context length")
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--layers", type=int, default=None, help="override the workload's layer count")
@@ -239,6 +242,14 @@ def main():
     out = torch.zeros((L, G, q_dim), device="cuda", dtype=torch.float16)
     stream = torch.cuda.Stream()
     use_graph = not args.no_graph
+    if args.producers != "none":
+        gw = torch.Generator(device="cuda"); gw.manual_seed(7)
+        q_norm = (1.0 + 0.1 * torch.randn((L, D), generator=gw, device="cuda")).to(torch.float16)
+        k_norm = (1.0 + 0.1 * torch.randn((L, D), generator=gw, device="cuda")).to(torch.float16)
+        inv = 1e6 ** (-torch.arange(0, D, 2, device="cuda", dtype=torch.float64) / D)
+        ang = torch.arange(msl, device="cuda", dtype=torch.float64)[:, None] * inv[None, :]
+        rope_cos, rope_sin = torch.cos(ang).to(torch.float16).contiguous(), torch.sin(ang).to(torch.float16).contiguous()
+        eng.set_producers(1 if args.producers == "fused" else 2, q_norm, k_norm, 1e-6, False, rope_cos, rope_sin, D)
 
     def step():
         eng.decode_step(q, k, v, out, use_graph=use_graph, stream=stream)
@@ -320,7 +331,8 @@ def main():
             "context_first_timed_step": [int(ctx0.min()), int(ctx0.max())],
             "tokens_attended_per_step": n_tokens_timed / K,
             "hipgraph": use_graph,
-            "step": "append K,V + decode attention for every layer, positions += 1",
+            "step": ("append K,V + decode attention for every layer, positions += 1" if args.producers == "none" else
+                     f"QK RMSNorm + RoPE ({args.producers}) + append K,V + decode attention for every layer, positions += 1"),
             **({"shared_prefix_tokens": w["prefix"][0], "prefix_append_and_broadcast_ms": prefix_ms} if w.get("prefix") else {}),
         },
         "step_algorithmic_GB": step_bytes * 1e-9,

@@ -26,6 +26,7 @@
 #ifndef TRIEBWERK_KV_H
 #define TRIEBWERK_KV_H
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -111,6 +112,34 @@ void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const ui
 /* engine.cpp:133, kernels.cu:1376 -- positions[g] += 1 on the device. */
 void launch_increment_positions(int* positions, int G, hipStream_t s);
 
+/* The producers of q and k, the step in front of the append (forward_layer_batch step 3,
+ * engine.cpp:1972-1977; single sequence engine.cpp:1060-1066).  In place, fp16 in and out.
+ *
+ * engine.cpp:126, kernels.cu:1345 -- per-head RMSNorm of the num_q heads of every q row and the
+ * num_kv heads of every k row; q_dim and kv_dim are row strides (a gated q projection passes
+ * 2*num_q*head_dim and the gate half stays untouched); `biased` adds 1 to the weights. */
+void launch_qk_norm_batch(tw_half* q, tw_half* k, const tw_half* q_weight, const tw_half* k_weight,
+                          int num_q, int num_kv, int head_dim, int G, float eps, int q_dim,
+                          int kv_dim, hipStream_t s, bool biased);
+
+/* engine.cpp:127, kernels.cu:1348 -- rotary embedding of the first rope_dim coordinates of every
+ * head of q and k with the table row positions[g] (rope_dim/2 entries per position).  rope_dim:
+ * 128, or a multiple of 16 up to 64. */
+void launch_rope_batch(tw_half* q, tw_half* k, const tw_half* cos_table, const tw_half* sin_table,
+                       const int* positions, int max_seq_len, int G, int num_heads,
+                       int num_kv_heads, int head_dim, int q_dim, int kv_dim, int rope_dim,
+                       hipStream_t s);
+
+/* engine.cpp:162, kernels.cu:706 -- per-head RMSNorm, one sequence. */
+void launch_qk_norm(tw_half* q, tw_half* k, const tw_half* q_weight, const tw_half* k_weight,
+                    int num_q_heads, int num_kv_heads, int head_dim, float eps, hipStream_t stream);
+
+/* engine.cpp:163, kernels.cu:719 -- rotary embedding, one sequence, `pos` by value, full width
+ * (table rows of head_dim/2 entries). */
+void launch_rope(tw_half* q, tw_half* k, const tw_half* cos_table, const tw_half* sin_table,
+                 int pos, int max_seq_len, int num_heads, int num_kv_heads, int head_dim,
+                 hipStream_t stream);
+
 /* ------------------------------------------------------------------ Part 2
  * Error state, tuning and the entry points the reference has no twin for.   */
 
@@ -169,6 +198,32 @@ void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_ha
                                      float* as, const int* pos, int msl, int G, int num_heads,
                                      int num_kv_heads, int head_dim, int q_dim, int kv_dim,
                                      int bits, hipStream_t s);
+
+/* Producers fused into the path (steps 3-5 of forward_layer_batch, engine.cpp:1972-2006, in one
+ * call): per-head RMSNorm (q_weight / k_weight, `biased`) and rotary embedding (tables as for
+ * launch_rope_batch) of q and k, append of K and V at positions[g], attention over
+ * 0..positions[g].  Same cache bytes and, within the attention tolerance, the same output as
+ * launch_qk_norm_batch + launch_rope_batch + the append + the attention.  q_weight == NULL skips
+ * the normalisation, cos_table == NULL the rotation.
+ *
+ * Compressed cache: normalisation and rotation happen in the launch that rotates and quantizes the
+ * rows, so q and k are only read (when that launch is not available for the shape, they are
+ * transformed in place first: treat their contents after the call as unspecified). */
+void tw_qk_norm_rope_turbo_append_attention_batch(
+    tw_half* out, tw_half* q, tw_half* k_buf, const tw_half* v_buf, const tw_half* q_weight,
+    const tw_half* k_weight, float eps, int biased, const tw_half* cos_table,
+    const tw_half* sin_table, int rope_dim, uint8_t* ck_q, uint8_t* cv_q, tw_half* k_norms,
+    tw_half* v_norms, const tw_half* rotation, float* as, const int* pos, int msl, int G,
+    int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim, int bits, hipStream_t s);
+
+/* fp16 cache: one launch transforms q in place and writes the transformed K rows and the V rows
+ * to the cache (instead of qk_norm + rope + kv_cache_write), then the attention.  k_buf is only read. */
+void tw_qk_norm_rope_append_attention_batch(
+    tw_half* out, tw_half* q, const tw_half* k_buf, const tw_half* v_buf, const tw_half* q_weight,
+    const tw_half* k_weight, float eps, int biased, const tw_half* cos_table,
+    const tw_half* sin_table, int rope_dim, tw_half* ck, tw_half* cv, float* as, const int* pos,
+    int msl, int G, int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+    hipStream_t s);
 
 /* Paged cache.  A page holds TW_PAGE_TOKENS consecutive positions of one
  * sequence in the same row layout the contiguous cache uses, so
@@ -247,6 +302,17 @@ void* tw_engine_cache_ptr(tw_engine* e, int layer, int which);
 int* tw_engine_positions(tw_engine* e);          /* device int32[G] */
 const tw_half* tw_engine_rotation(tw_engine* e); /* device, NULL when kv_bits==0 */
 int tw_engine_set_positions(tw_engine* e, const int* host_positions, int G);
+
+/* Make the producers of q and k part of every step (forward_layer_batch step 3,
+ * engine.cpp:1972-1977): per-head RMSNorm with the weights of the step's layer (q_norm, k_norm:
+ * device, (num_layers, head_dim); NULL = none) and rotary embedding from the tables (device,
+ * (positions, rope_dim/2); NULL = none).  mode 1 fuses them into the append (see
+ * tw_qk_norm_rope_turbo_append_attention_batch), mode 2 runs the reference's two launches first,
+ * mode 0 switches them off.  The pointers are kept, not copied.  With producers the q and k rows
+ * handed to a step are scratch: they may come back transformed. */
+int tw_engine_set_producers(tw_engine* e, int mode, const tw_half* q_norm, const tw_half* k_norm,
+                            float eps, int biased, const tw_half* rope_cos, const tw_half* rope_sin,
+                            int rope_dim);
 
 /* One decode step of the path for `layer`: append K,V at positions[g], then
  * attention over 0..positions[g] (forward_layer_batch steps 4-5,

@@ -327,6 +327,32 @@ void turbo_attention_head(uint16_t* out_head, const uint16_t* q_head,
     }
 }
 
+
+// ---------------------------------------------------------------- producers of q and k: per-head RMSNorm and RoPE
+// One block of qk_norm_kernel (kernels.cu:137-186, 128 threads) or qk_norm_batch_kernel
+// (kernels.cu:880-923, head_dim threads): thread t sums v*v over i = t, t + nthreads, ...
+// (fused multiply-adds), block sum, rms = rsqrtf(sum / head_dim + eps), then
+// data[i] = half((float(data[i]) * rms) * w[i]), w[i] + 1 first when `biased`.
+void norm_head(uint16_t* data, const uint16_t* w, int head_dim, int nthreads, float eps, bool biased) {
+    float per_thread[1024];
+    if (nthreads > 1024) abort();
+    for (int t = 0; t < nthreads; t++) {
+        float sum_sq = 0.0f;
+        for (int i = t; i < head_dim; i += nthreads) {
+            float v = h2f(data[i]);
+            sum_sq = fmaf(v, v, sum_sq);
+        }
+        per_thread[t] = sum_sq;
+    }
+    float total = block_sum(per_thread, nthreads);
+    float rms = 1.0f / sqrtf(total / (float)head_dim + eps);   // rsqrtf (kernels.cu:179, 916)
+    for (int i = 0; i < head_dim; i++) {
+        float wv = h2f(w[i]);
+        if (biased) wv += 1.0f;
+        data[i] = f2h((h2f(data[i]) * rms) * wv);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -562,6 +588,88 @@ void tw_oracle_turbo_gqa_prefill_attention(uint16_t* out, const uint16_t* q,
 
 void tw_oracle_increment_positions(int* positions, int G) {
     for (int g = 0; g < G; g++) positions[g]++;
+}
+
+void tw_oracle_qk_norm(uint16_t* q, uint16_t* k, const uint16_t* q_weight, const uint16_t* k_weight,
+                       int num_q_heads, int num_kv_heads, int head_dim, float eps) {
+    // launch_qk_norm (kernels.cu:706-717): one block of 128 threads per head, Q heads first
+    for (int h = 0; h < num_q_heads; h++) norm_head(q + (size_t)h * head_dim, q_weight, head_dim, 128, eps, false);
+    for (int h = 0; h < num_kv_heads; h++) norm_head(k + (size_t)h * head_dim, k_weight, head_dim, 128, eps, false);
+}
+
+void tw_oracle_qk_norm_batch(uint16_t* q, uint16_t* k, const uint16_t* q_weight, const uint16_t* k_weight,
+                             int num_q, int num_kv, int head_dim, int G, float eps,
+                             int q_dim, int kv_dim, int biased) {
+    // launch_qk_norm_batch (kernels.cu:1345-1347): G * (num_q + num_kv) blocks of head_dim threads
+    for (int g = 0; g < G; g++) {
+        for (int h = 0; h < num_q; h++)
+            norm_head(q + (size_t)g * q_dim + (size_t)h * head_dim, q_weight, head_dim, head_dim, eps, biased != 0);
+        for (int h = 0; h < num_kv; h++)
+            norm_head(k + (size_t)g * kv_dim + (size_t)h * head_dim, k_weight, head_dim, head_dim, eps, biased != 0);
+    }
+}
+
+void tw_oracle_rope(uint16_t* q, uint16_t* k, const uint16_t* cos_table, const uint16_t* sin_table,
+                    int pos, int max_seq_len, int num_heads, int num_kv_heads, int head_dim) {
+    // launch_rope + rope_kernel (kernels.cu:719-735, 193-235): table row `pos` of head_dim/2 entries;
+    // out0 = q0*c - q1*s, out1 = q1*c + q0*s, each one multiply and one fused multiply-add
+    (void)max_seq_len;
+    const int half = head_dim / 2;
+    const uint16_t* ct = cos_table + (size_t)pos * half;
+    const uint16_t* st = sin_table + (size_t)pos * half;
+    for (int pass = 0; pass < 2; pass++) {
+        uint16_t* x = pass ? k : q;
+        const int heads = pass ? num_kv_heads : num_heads;
+        for (int h = 0; h < heads; h++) {
+            uint16_t* xh = x + (size_t)h * head_dim;
+            for (int d = 0; d < half; d++) {
+                float c = h2f(ct[d]), sn = h2f(st[d]);
+                float x0 = h2f(xh[d]), x1 = h2f(xh[d + half]);
+                xh[d] = f2h(fmaf(x0, c, -(x1 * sn)));
+                xh[d + half] = f2h(fmaf(x1, c, x0 * sn));
+            }
+        }
+    }
+}
+
+void tw_oracle_rope_batch(uint16_t* q, uint16_t* k, const uint16_t* cos_table, const uint16_t* sin_table,
+                          const int* positions, int max_seq_len, int G, int num_heads, int num_kv_heads,
+                          int head_dim, int q_dim, int kv_dim, int rope_dim) {
+    // rope_batch_kernel (kernels.cu:927-961): table row positions[g] of rope_dim/2 entries; only the first
+    // rope_dim coordinates of a head turn; out0 = q0*c - q1*s, out1 = q0*s + q1*c
+    (void)max_seq_len;
+    const int half = rope_dim / 2;
+    for (int g = 0; g < G; g++) {
+        const int pos = positions[g];
+        const uint16_t* ct = cos_table + (size_t)pos * half;
+        const uint16_t* st = sin_table + (size_t)pos * half;
+        for (int pass = 0; pass < 2; pass++) {
+            uint16_t* x = pass ? k + (size_t)g * kv_dim : q + (size_t)g * q_dim;
+            const int heads = pass ? num_kv_heads : num_heads;
+            for (int h = 0; h < heads; h++) {
+                uint16_t* xh = x + (size_t)h * head_dim;
+                for (int d = 0; d < half; d++) {
+                    float c = h2f(ct[d]), sn = h2f(st[d]);
+                    float x0 = h2f(xh[d]), x1 = h2f(xh[d + half]);
+                    xh[d] = f2h(fmaf(x0, c, -(x1 * sn)));
+                    xh[d + half] = f2h(fmaf(x0, sn, x1 * c));
+                }
+            }
+        }
+    }
+}
+
+void tw_oracle_rope_tables(uint16_t* cos_table, uint16_t* sin_table, int max_seq_len, int rope_dim, float theta) {
+    // precompute_rope (engine.cpp:554-574); powf, cosf and sinf are this machine's libm
+    const int half = rope_dim / 2;
+    for (int pos = 0; pos < max_seq_len; pos++) {
+        for (int d = 0; d < half; d++) {
+            float freq = 1.0f / powf(theta, (float)(2 * d) / rope_dim);
+            float angle = pos * freq;
+            cos_table[(size_t)pos * half + d] = f2h(cosf(angle));
+            sin_table[(size_t)pos * half + d] = f2h(sinf(angle));
+        }
+    }
 }
 
 }  // extern "C"

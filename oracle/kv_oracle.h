@@ -26,6 +26,8 @@
  *   fp16 attention: float64 softmax(QK^T/sqrt(D))V
  *   turbo attn    : float64 attention on the dequantized cache (identity)
  *   bookkeeping   : brute-force position model on tiny shapes
+ *   qk norm, rope : float64 RMSNorm and complex rotation; position 0 and unit weights are
+ *                   identities bit for bit; pair norms are kept; strides leave gaps untouched
  * The reference ships no golden vector, test or fixture for this path, so the
  * kernel source text is the only authority the restatement can be read against.
  * What stays unpinned: the fast-math last-ulp behaviour of the CUDA build.
@@ -125,6 +127,28 @@ void tw_oracle_turbo_gqa_prefill_attention(uint16_t* out, const uint16_t* q,
 
 /* increment_positions_kernel, kernels.cu:1371-1374. */
 void tw_oracle_increment_positions(int* positions, int G);
+
+/* Producers of q and k, the step before the append (engine.cpp:1972-1977).
+ * qk_norm_kernel (kernels.cu:137-186) / qk_norm_batch_kernel (880-923): per-head RMSNorm in place;
+ * q_dim / kv_dim are row strides; biased adds 1 to the weights.
+ * rope_kernel (193-235) / rope_batch_kernel (927-961): rotary embedding in place from fp16 tables
+ * of rope_dim/2 entries per position (single sequence: rope_dim = head_dim).  The two differ in the
+ * operand order of the second output (q1*c + q0*s against q0*s + q1*c).
+ * `a*b - c*d` and `a*b + c*d` are restated as fma(a, b, -(c*d)) and fma(a, b, c*d): the first product
+ * fused, the second rounded -- which product nvcc fuses is a last-ulp question only a run of the
+ * CUDA build could settle (parity unpinned at that level, like the fast-math ulps). */
+void tw_oracle_qk_norm(uint16_t* q, uint16_t* k, const uint16_t* q_weight, const uint16_t* k_weight,
+                       int num_q_heads, int num_kv_heads, int head_dim, float eps);
+void tw_oracle_qk_norm_batch(uint16_t* q, uint16_t* k, const uint16_t* q_weight, const uint16_t* k_weight,
+                             int num_q, int num_kv, int head_dim, int G, float eps,
+                             int q_dim, int kv_dim, int biased);
+void tw_oracle_rope(uint16_t* q, uint16_t* k, const uint16_t* cos_table, const uint16_t* sin_table,
+                    int pos, int max_seq_len, int num_heads, int num_kv_heads, int head_dim);
+void tw_oracle_rope_batch(uint16_t* q, uint16_t* k, const uint16_t* cos_table, const uint16_t* sin_table,
+                          const int* positions, int max_seq_len, int G, int num_heads, int num_kv_heads,
+                          int head_dim, int q_dim, int kv_dim, int rope_dim);
+/* precompute_rope, engine.cpp:554-574. */
+void tw_oracle_rope_tables(uint16_t* cos_table, uint16_t* sin_table, int max_seq_len, int rope_dim, float theta);
 
 /* Threads the OpenMP loops over (sequence, head) will use. */
 int  tw_oracle_num_threads(void);

@@ -49,6 +49,11 @@ class Oracle:
         lib.tw_oracle_turbo_gqa_attention_batch.argtypes = [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I]
         lib.tw_oracle_turbo_gqa_prefill_attention.argtypes = [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I]
         lib.tw_oracle_increment_positions.argtypes = [P, I]
+        lib.tw_oracle_qk_norm.argtypes = [P, P, P, P, I, I, I, C.c_float]
+        lib.tw_oracle_qk_norm_batch.argtypes = [P, P, P, P, I, I, I, I, C.c_float, I, I, I]
+        lib.tw_oracle_rope.argtypes = [P, P, P, P, I, I, I, I, I]
+        lib.tw_oracle_rope_batch.argtypes = [P, P, P, P, P, I, I, I, I, I, I, I, I]
+        lib.tw_oracle_rope_tables.argtypes = [P, P, I, I, C.c_float]
         lib.tw_oracle_num_threads.restype = I
         lib.tw_oracle_set_num_threads.argtypes = [I]
 
@@ -125,6 +130,28 @@ class Oracle:
 
     def increment_positions(self, pos, G):
         self.lib.tw_oracle_increment_positions(_p(pos, np.int32), G)
+
+    def qk_norm(self, q, k, qw, kw, H, Hk, D, eps):
+        self.lib.tw_oracle_qk_norm(_p(q, np.float16), _p(k, np.float16), _p(qw, np.float16), _p(kw, np.float16),
+                                   H, Hk, D, eps)
+
+    def qk_norm_batch(self, q, k, qw, kw, H, Hk, D, G, eps, q_dim, kv_dim, biased=False):
+        self.lib.tw_oracle_qk_norm_batch(_p(q, np.float16), _p(k, np.float16), _p(qw, np.float16),
+                                         _p(kw, np.float16), H, Hk, D, G, eps, q_dim, kv_dim, int(biased))
+
+    def rope(self, q, k, ct, st, pos, msl, H, Hk, D):
+        self.lib.tw_oracle_rope(_p(q, np.float16), _p(k, np.float16), _p(ct, np.float16), _p(st, np.float16),
+                                pos, msl, H, Hk, D)
+
+    def rope_batch(self, q, k, ct, st, positions, msl, G, H, Hk, D, q_dim, kv_dim, rope_dim):
+        self.lib.tw_oracle_rope_batch(_p(q, np.float16), _p(k, np.float16), _p(ct, np.float16), _p(st, np.float16),
+                                      _p(positions, np.int32), msl, G, H, Hk, D, q_dim, kv_dim, rope_dim)
+
+    def rope_tables(self, msl, rope_dim, theta):
+        ct = np.empty((msl, rope_dim // 2), np.float16)
+        st = np.empty((msl, rope_dim // 2), np.float16)
+        self.lib.tw_oracle_rope_tables(ct.ctypes.data, st.ctypes.data, msl, rope_dim, theta)
+        return ct, st
 
     def num_threads(self):
         return self.lib.tw_oracle_num_threads()

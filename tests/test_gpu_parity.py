@@ -567,6 +567,148 @@ def test_tq2_eight_kv_heads_paged_and_contiguous(kv, oracle, rotation_fixture, H
         kv.set_num_splits(0)
 
 
+# ------------------------------------------------------------------ producers of q and k: RMSNorm and RoPE
+def rope_tables(msl, rope_dim, theta=1e6):
+    d = np.arange(rope_dim // 2, dtype=np.float64)
+    ang = np.arange(msl, dtype=np.float64)[:, None] * theta ** (-2.0 * d / rope_dim)[None, :]
+    return np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
+
+
+def producer_inputs(r, G, H, Hk, q_dim, kv_dim):
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim))
+    q[0] = (q[0].astype(np.float32) * 30).astype(np.float16)
+    k[G - 1] = (k[G - 1].astype(np.float32) * 1e-3).astype(np.float16)
+    k[0, :D] = 0                                         # a zero head: rms = 1/sqrt(eps)
+    qw = (1.0 + 0.3 * r.standard_normal(D)).astype(np.float16)
+    kw = (1.0 + 0.3 * r.standard_normal(D)).astype(np.float16)
+    return q, k, qw, kw
+
+
+@pytest.mark.parametrize("biased", [False, True])
+def test_qk_norm_batch_bit_exact(kv, oracle, biased):
+    r = gen.rng(700 + biased)
+    G, H, Hk = 37, 16, 8
+    q_dim, kv_dim = 2 * H * D, Hk * D            # gated projection: the second half of a q row is the gate
+    q, k, qw, kw = producer_inputs(r, G, H, Hk, q_dim, kv_dim)
+    d_q, d_k = dev(q), dev(k)
+    kv.launch_qk_norm_batch(d_q, d_k, dev(qw), dev(kw), H, Hk, D, G, 1e-6, q_dim, kv_dim, biased=biased)
+    oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, 1e-6, q_dim, kv_dim, biased)
+    assert_bytes_equal(host(d_q), q, "normalised q")
+    assert_bytes_equal(host(d_k), k, "normalised k")
+
+
+@pytest.mark.parametrize("rope_dim", [128, 64, 32, 48])
+def test_rope_batch_bit_exact(kv, oracle, rope_dim):
+    r = gen.rng(710 + rope_dim)
+    G, H, Hk, msl = 29, 8, 2, 4096
+    q_dim, kv_dim = H * D + 64, Hk * D
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim))
+    ct, st = rope_tables(msl, rope_dim)
+    pos = r.integers(0, msl, G).astype(np.int32); pos[0] = 0; pos[1] = msl - 1
+    d_q, d_k = dev(q), dev(k)
+    kv.launch_rope_batch(d_q, d_k, dev(ct), dev(st), dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, rope_dim)
+    oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, rope_dim)
+    assert_bytes_equal(host(d_q), q, "rotated q")
+    assert_bytes_equal(host(d_k), k, "rotated k")
+
+
+def test_qk_norm_and_rope_single_sequence_bit_exact(kv, oracle):
+    r = gen.rng(720)
+    H, Hk, msl = 16, 8, 777
+    q = gen.normal_f16(r, (H * D,)); k = gen.normal_f16(r, (Hk * D,))
+    qw = (1.0 + 0.3 * r.standard_normal(D)).astype(np.float16); kw = (0.7 * r.standard_normal(D)).astype(np.float16)
+    ct, st = rope_tables(msl, D, theta=10000.0)
+    d_q, d_k = dev(q), dev(k)
+    kv.launch_qk_norm(d_q, d_k, dev(qw), dev(kw), H, Hk, D, 1e-6)
+    oracle.qk_norm(q, k, qw, kw, H, Hk, D, 1e-6)
+    assert_bytes_equal(host(d_q), q, "normalised q"); assert_bytes_equal(host(d_k), k, "normalised k")
+    kv.launch_rope(d_q, d_k, dev(ct), dev(st), 613, msl, H, Hk, D)
+    oracle.rope(q, k, ct, st, 613, msl, H, Hk, D)
+    assert_bytes_equal(host(d_q), q, "rotated q"); assert_bytes_equal(host(d_k), k, "rotated k")
+
+
+def test_producer_rejects_unsupported_shapes(kv):
+    import torch
+    q = torch.zeros(2, 256, dtype=torch.float16, device="cuda"); k = torch.zeros(2, 256, dtype=torch.float16, device="cuda")
+    w = torch.ones(128, dtype=torch.float16, device="cuda")
+    pos = torch.zeros(2, dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="head_dim"):
+        kv.launch_qk_norm_batch(q, k, w, w, 4, 4, 64, 2, 1e-6, 256, 256)
+    with pytest.raises(RuntimeError, match="rope_dim"):
+        kv.launch_rope_batch(q, k, w, w, pos, 16, 2, 2, 2, 128, 256, 256, 96)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("bits,H,Hk,norm,rope_dim", [(4, 16, 8, True, 128), (2, 16, 8, True, 128), (4, 32, 8, True, 64),
+                                                     (2, 8, 8, False, 128), (4, 16, 8, True, 0)])
+def test_fused_norm_rope_turbo_step(kv, oracle, rotation_fixture, bits, H, Hk, norm, rope_dim, variant):
+    """RMSNorm + RoPE + append + attention in one call == the oracle's four steps: cache bytes bit for
+    bit, output within the attention tolerance.  variant 1 takes the kernels of their own."""
+    import torch
+    r = gen.rng(730 + bits + H + rope_dim)
+    G, msl = 9, 384
+    kv_dim, q_dim = Hk * D, H * D
+    lens = [1, 33, 64, 100, 257, 300, 319, 200, 383]
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits, outliers=False)
+    pos = np.array(lens, np.int32)
+    pos[8] = 383
+    q, k, qw, kw = producer_inputs(r, G, H, Hk, q_dim, kv_dim)
+    v = gen.normal_f16(r, (G, kv_dim))
+    ct, st = rope_tables(msl, rope_dim) if rope_dim else (None, None)
+    d_ck, d_cv, d_kn, d_vn = dev(ck), dev(cv), dev(kn), dev(vn)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.set_attention_variant(variant)
+    try:
+        kv.tw_qk_norm_rope_turbo_append_attention_batch(
+            out, dev(q), dev(k), dev(v), dev(qw) if norm else None, dev(kw) if norm else None, 1e-6, False,
+            dev(ct) if rope_dim else None, dev(st) if rope_dim else None, rope_dim, d_ck, d_cv, d_kn, d_vn,
+            dev(rotation_fixture), scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    finally:
+        kv.set_attention_variant(0)
+    if norm:
+        oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, 1e-6, q_dim, kv_dim, False)
+    if rope_dim:
+        oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, rope_dim)
+    oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(cv, vn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    assert_bytes_equal(host(d_ck), ck, "K codes"); assert_bytes_equal(host(d_cv), cv, "V codes")
+    assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+    assert rel_err(host(out), want) <= TOL
+
+
+@pytest.mark.parametrize("rope_dim", [128, 64])
+def test_fused_norm_rope_fp16_step(kv, oracle, rope_dim):
+    """fp16 cache: one launch normalises and rotates q in place and writes the transformed K rows and the
+    V rows to the cache; q and the cache are the oracle's bit for bit."""
+    import torch
+    r = gen.rng(740 + rope_dim)
+    G, H, Hk, msl = 6, 16, 8, 160
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+    pos = np.array([0, 1, 17, 64, 100, 159], np.int32)
+    for g in range(G):
+        ck[g, pos[g]:] = 0; cv[g, pos[g]:] = 0
+    q, k, qw, kw = producer_inputs(r, G, H, Hk, q_dim, kv_dim)
+    v = gen.normal_f16(r, (G, kv_dim))
+    ct, st = rope_tables(msl, rope_dim)
+    d_q, d_ck, d_cv = dev(q), dev(ck), dev(cv)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.tw_qk_norm_rope_append_attention_batch(out, d_q, dev(k), dev(v), dev(qw), dev(kw), 1e-6, True, dev(ct), dev(st),
+                                              rope_dim, d_ck, d_cv, scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim)
+    oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, 1e-6, q_dim, kv_dim, True)
+    oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, rope_dim)
+    oracle.kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    assert_bytes_equal(host(d_q), q, "q after the call")
+    assert_bytes_equal(host(d_ck), ck, "K cache"); assert_bytes_equal(host(d_cv), cv, "V cache")
+    assert rel_err(host(out), want) <= TOL
+
+
 # ------------------------------------------------------------------ engine: append -> attention -> positions, eager and graph
 @pytest.mark.parametrize("kv_bits", [0, 4, 2])
 @pytest.mark.parametrize("use_graph", [False, True])
@@ -632,6 +774,73 @@ def test_engine_decode_steps(oracle, kv_bits, use_graph):
             assert_bytes_equal(host(c[3]), o_vn[l], f"layer {l} V norms")
     eng.reset()
     assert not host(eng.cache(0)[0]).any() and not host(eng.positions()).any()
+
+
+@pytest.mark.parametrize("kv_bits", [0, 4, 2])
+@pytest.mark.parametrize("mode", [1, 2])
+def test_engine_decode_steps_with_producers(oracle, kv_bits, mode):
+    """The engine's step with per-layer QK RMSNorm and RoPE, fused (mode 1) or as launches of their own
+    (mode 2), captured in a graph: caches bit for bit and outputs within tolerance of the oracle's
+    norm -> rope -> append -> attention, over several steps (positions advance, so the table row does)."""
+    import torch
+    from triebwerk_amd import Engine
+    r = gen.rng(560 + kv_bits + mode)
+    L, H, Hk, G, msl, steps = 3, 16, 8, 5, 48, 4
+    kv_dim, q_dim = Hk * D, H * D
+    eng = Engine(max_seq_len=1024, kv_bits=kv_bits)
+    eng.set_shape(L, H, Hk, D)
+    eng.alloc_batch(G, msl)
+    start = np.array([0, 3, 10, 31, 41], np.int32)
+    eng.set_positions(start)
+    rot = host(eng.rotation()) if kv_bits else None
+    qn = (1.0 + 0.2 * r.standard_normal((L, D))).astype(np.float16); kn_w = (1.0 + 0.2 * r.standard_normal((L, D))).astype(np.float16)
+    ct, st = rope_tables(msl, D)
+    eng.set_producers(mode, dev(qn), dev(kn_w), 1e-6, False, dev(ct), dev(st), D)
+    if kv_bits == 0:
+        o_k = [np.zeros((G, msl, kv_dim), np.float16) for _ in range(L)]
+        o_v = [np.zeros((G, msl, kv_dim), np.float16) for _ in range(L)]
+    else:
+        kvp = kv_dim * kv_bits // 8
+        o_k = [np.zeros((G, msl, kvp), np.uint8) for _ in range(L)]; o_v = [np.zeros((G, msl, kvp), np.uint8) for _ in range(L)]
+        o_kn = [np.zeros((G, msl, Hk), np.float16) for _ in range(L)]; o_vn = [np.zeros((G, msl, Hk), np.float16) for _ in range(L)]
+    pos = start.copy()
+    d_q = torch.zeros((L, G, q_dim), dtype=torch.float16, device="cuda")
+    d_k = torch.zeros((L, G, kv_dim), dtype=torch.float16, device="cuda")
+    d_v = torch.zeros((L, G, kv_dim), dtype=torch.float16, device="cuda")
+    d_out = torch.zeros((L, G, q_dim), dtype=torch.float16, device="cuda")
+    stream = torch.cuda.Stream()
+    for step in range(steps):
+        q = gen.normal_f16(r, (L, G, q_dim)); k = gen.normal_f16(r, (L, G, kv_dim)); v = gen.normal_f16(r, (L, G, kv_dim))
+        d_q.copy_(dev(q)); d_k.copy_(dev(k)); d_v.copy_(dev(v))
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            eng.decode_step(d_q, d_k, d_v, d_out, use_graph=True, stream=stream)
+        stream.synchronize()
+        got = host(d_out)
+        for l in range(L):
+            want = np.zeros((G, q_dim), np.float16)
+            ql, kl = q[l].copy(), k[l].copy()
+            oracle.qk_norm_batch(ql, kl, qn[l], kn_w[l], H, Hk, D, G, 1e-6, q_dim, kv_dim, False)
+            oracle.rope_batch(ql, kl, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, D)
+            if kv_bits == 0:
+                oracle.kv_cache_write_batch(o_k[l], o_v[l], kl, v[l], pos, msl, G, kv_dim)
+                oracle.gqa_attention_batch(want, ql, o_k[l], o_v[l], pos, msl, G, H, Hk, D, q_dim, kv_dim)
+            else:
+                oracle.turbo_kv_quantize_batch(o_k[l], o_kn[l], kl, rot, pos, msl, G, Hk, D, kv_dim, kv_bits)
+                oracle.turbo_kv_quantize_batch(o_v[l], o_vn[l], v[l], rot, pos, msl, G, Hk, D, kv_dim, kv_bits)
+                oracle.turbo_gqa_attention_batch(want, ql, o_k[l], o_v[l], o_kn[l], o_vn[l], rot, pos, msl, G, H, Hk, D,
+                                                 q_dim, kv_dim, kv_bits)
+            err = rel_err(got[l], want)
+            assert err <= TOL, f"step {step} layer {l}: {err}"
+        oracle.increment_positions(pos, G)
+    for l in range(L):
+        c = eng.cache(l)
+        assert_bytes_equal(host(c[0]), o_k[l], f"layer {l} K cache")
+        assert_bytes_equal(host(c[1]), o_v[l], f"layer {l} V cache")
+        if kv_bits:
+            assert_bytes_equal(host(c[2]), o_kn[l], f"layer {l} K norms")
+            assert_bytes_equal(host(c[3]), o_vn[l], f"layer {l} V norms")
+    eng.set_producers(0)
 
 
 def test_engine_prefix_broadcast(oracle):

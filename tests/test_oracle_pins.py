@@ -496,3 +496,159 @@ def test_golden_case_reproduces(oracle, rotation_fixture, bits):
     out = np.zeros((G, q_dim), np.float16)
     oracle.turbo_gqa_attention_batch(out, np.ascontiguousarray(z["q"]), ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
     assert np.array_equal(out, z["out"])
+
+
+# ------------------------------------------------------------------ producers: QK RMSNorm and RoPE
+def _f64(a):
+    return a.astype(np.float64)
+
+
+@pytest.mark.parametrize("biased", [False, True])
+def test_qk_norm_is_rmsnorm(oracle, biased):
+    """x / sqrt(mean(x^2) + eps) * w in float64, per head; the gap between the heads and the row
+    stride (gate half of a gated q projection) is not touched."""
+    r = gen.rng(610 + biased)
+    G, H, Hk, D = 3, 4, 2, 128
+    q_dim, kv_dim = 2 * H * D, Hk * D + 64
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim))
+    q[1] = (q[1].astype(np.float32) * 40).astype(np.float16)        # large row
+    k[2] = (k[2].astype(np.float32) * 1e-3).astype(np.float16)      # tiny row: eps matters
+    qw = (1.0 + 0.3 * r.standard_normal(D)).astype(np.float16)
+    kw = (0.5 * r.standard_normal(D)).astype(np.float16)
+    eps = 1e-6
+    q0, k0 = q.copy(), k.copy()
+    oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, eps, q_dim, kv_dim, biased)
+    for x, x0, w, heads in ((q, q0, qw, H), (k, k0, kw, Hk)):
+        ww = _f64(w) + (1.0 if biased else 0.0)
+        for g in range(G):
+            for h in range(heads):
+                v = _f64(x0[g, h * D:(h + 1) * D])
+                want = v / np.sqrt(np.mean(v * v) + eps) * ww
+                got = _f64(x[g, h * D:(h + 1) * D])
+                assert np.max(np.abs(got - want)) <= 1e-3 * np.max(np.abs(want)) + 1e-7
+            assert np.array_equal(x[g, heads * D:].view(np.uint16), x0[g, heads * D:].view(np.uint16))
+
+
+def test_qk_norm_single_equals_batch_of_one_and_scaling(oracle):
+    """The single-sequence kernel (128 threads striding the head) and the batch kernel (one thread
+    per element) agree on 128-wide heads; scaling the input by a power of two does not change the
+    result when eps is negligible (RMSNorm is scale-free), which a dropped 1/head_dim would break
+    together with the float64 check above."""
+    r = gen.rng(612)
+    H, Hk, D = 6, 2, 128
+    q = gen.normal_f16(r, (H * D,)); k = gen.normal_f16(r, (Hk * D,))
+    qw = (1.0 + 0.1 * r.standard_normal(D)).astype(np.float16); kw = (1.0 + 0.1 * r.standard_normal(D)).astype(np.float16)
+    q1, k1, q2, k2 = q.copy(), k.copy(), q.copy().reshape(1, -1), k.copy().reshape(1, -1)
+    oracle.qk_norm(q1, k1, qw, kw, H, Hk, D, 1e-6)
+    oracle.qk_norm_batch(q2, k2, qw, kw, H, Hk, D, 1, 1e-6, H * D, Hk * D, False)
+    assert np.array_equal(q1.view(np.uint16), q2[0].view(np.uint16))
+    assert np.array_equal(k1.view(np.uint16), k2[0].view(np.uint16))
+    q3 = (q.astype(np.float32) * 4).astype(np.float16); k3 = (k.astype(np.float32) * 4).astype(np.float16)
+    oracle.qk_norm(q3, k3, qw, kw, H, Hk, D, 0.0)
+    q4, k4 = q.copy(), k.copy()
+    oracle.qk_norm(q4, k4, qw, kw, H, Hk, D, 0.0)
+    assert np.array_equal(q3.view(np.uint16), q4.view(np.uint16))
+    assert np.array_equal(k3.view(np.uint16), k4.view(np.uint16))
+
+
+def test_qk_norm_unit_weight_gives_unit_rms(oracle):
+    r = gen.rng(613)
+    H, Hk, D, G = 2, 2, 128, 4
+    q = gen.normal_f16(r, (G, H * D)); k = gen.normal_f16(r, (G, Hk * D))
+    one = np.ones(D, np.float16)
+    oracle.qk_norm_batch(q, k, one, one, H, Hk, D, G, 1e-6, H * D, Hk * D, False)
+    rms = np.sqrt(np.mean(_f64(q.reshape(G, H, D)) ** 2, axis=-1))
+    assert np.all(np.abs(rms - 1.0) < 2e-3)
+    zero = np.zeros(D, np.float16)                       # biased: weight 0 means scale 1
+    q2 = gen.normal_f16(r, (G, H * D)); k2 = gen.normal_f16(r, (G, Hk * D))
+    q3, k3 = q2.copy(), k2.copy()
+    oracle.qk_norm_batch(q2, k2, one, one, H, Hk, D, G, 1e-6, H * D, Hk * D, False)
+    oracle.qk_norm_batch(q3, k3, zero, zero, H, Hk, D, G, 1e-6, H * D, Hk * D, True)
+    assert np.array_equal(q2.view(np.uint16), q3.view(np.uint16)) and np.array_equal(k2.view(np.uint16), k3.view(np.uint16))
+
+
+def _tables(r, msl, rope_dim, theta=1e6):
+    """cos/sin of pos * theta^(-2d/rope_dim) in float64, rounded to fp16 (engine.cpp:554-574)."""
+    d = np.arange(rope_dim // 2, dtype=np.float64)
+    ang = np.arange(msl, dtype=np.float64)[:, None] * theta ** (-2.0 * d / rope_dim)[None, :]
+    return np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
+
+
+@pytest.mark.parametrize("rope_dim", [128, 64])
+def test_rope_batch_is_a_complex_rotation(oracle, rope_dim):
+    """(x_d + i x_{d+half}) * (c + i s) in float64 with the fp16 table values; coordinates past
+    rope_dim, the gap behind the heads and other sequences' rows are left alone."""
+    r = gen.rng(620 + rope_dim)
+    G, H, Hk, D, msl = 4, 4, 2, 128, 300
+    q_dim, kv_dim = H * D + 32, Hk * D
+    ct, st = _tables(r, msl, rope_dim)
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim))
+    pos = np.array([0, 1, 137, 299], np.int32)
+    q0, k0 = q.copy(), k.copy()
+    oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, rope_dim)
+    half = rope_dim // 2
+    for x, x0, heads in ((q, q0, H), (k, k0, Hk)):
+        for g in range(G):
+            c, s = _f64(ct[pos[g]]), _f64(st[pos[g]])
+            for h in range(heads):
+                v = _f64(x0[g, h * D:(h + 1) * D]); got = _f64(x[g, h * D:(h + 1) * D])
+                z = (v[:half] + 1j * v[half:rope_dim]) * (c + 1j * s)
+                assert np.max(np.abs(got[:half] - z.real)) <= 2e-3 * np.max(np.abs(v)) + 1e-6
+                assert np.max(np.abs(got[half:rope_dim] - z.imag)) <= 2e-3 * np.max(np.abs(v)) + 1e-6
+                assert np.array_equal(x[g, h * D + rope_dim:(h + 1) * D].view(np.uint16),
+                                      x0[g, h * D + rope_dim:(h + 1) * D].view(np.uint16))
+            assert np.array_equal(x[g, heads * D:].view(np.uint16), x0[g, heads * D:].view(np.uint16))
+    # position 0: cos = 1 and sin = 0 exactly, so the row comes back bit for bit
+    assert np.array_equal(q[0].view(np.uint16), q0[0].view(np.uint16))
+    assert np.array_equal(k[0].view(np.uint16), k0[0].view(np.uint16))
+
+
+def test_rope_single_rotates_like_batch_and_differs_only_in_operand_order(oracle):
+    """Same rotation from both kernels; exactly representable inputs (small integers, table entries
+    that are powers of two) make every product exact, so the two operand orders give equal bits."""
+    r = gen.rng(630)
+    H, Hk, D, msl = 3, 2, 128, 8
+    ct = np.full((msl, D // 2), 0.5, np.float16); st = np.full((msl, D // 2), -0.25, np.float16)
+    q = r.integers(-8, 9, H * D).astype(np.float16); k = r.integers(-8, 9, Hk * D).astype(np.float16)
+    q1, k1 = q.copy(), k.copy()
+    q2, k2 = q.copy().reshape(1, -1), k.copy().reshape(1, -1)
+    oracle.rope(q1, k1, ct, st, 5, msl, H, Hk, D)
+    oracle.rope_batch(q2, k2, ct, st, np.array([5], np.int32), msl, 1, H, Hk, D, H * D, Hk * D, D)
+    assert np.array_equal(q1.view(np.uint16), q2[0].view(np.uint16)) and np.array_equal(k1.view(np.uint16), k2[0].view(np.uint16))
+    v = _f64(q.reshape(H, D))
+    want0 = v[:, :64] * 0.5 - v[:, 64:] * -0.25
+    want1 = v[:, 64:] * 0.5 + v[:, :64] * -0.25
+    got = _f64(q1.reshape(H, D))
+    assert np.array_equal(got[:, :64], want0) and np.array_equal(got[:, 64:], want1)
+    # general inputs: within one fp16 step of each other and of the float64 rotation
+    ct, st = _tables(r, msl, D)
+    q = gen.normal_f16(r, (H * D,)); k = gen.normal_f16(r, (Hk * D,))
+    q1, k1, q2, k2 = q.copy(), k.copy(), q.copy().reshape(1, -1), k.copy().reshape(1, -1)
+    oracle.rope(q1, k1, ct, st, 7, msl, H, Hk, D)
+    oracle.rope_batch(q2, k2, ct, st, np.array([7], np.int32), msl, 1, H, Hk, D, H * D, Hk * D, D)
+    assert np.max(np.abs(_f64(q1) - _f64(q2[0]))) <= 2 ** -8 * np.max(np.abs(_f64(q)))
+
+
+def test_rope_keeps_pair_norms_and_inverts(oracle):
+    """A rotation keeps |x_d|^2 + |x_{d+half}|^2 (to the tables' fp16 rounding), and the table with
+    the sine negated undoes it."""
+    r = gen.rng(640)
+    G, H, Hk, D, msl = 2, 2, 2, 128, 64
+    ct, st = _tables(r, msl, D, theta=10000.0)
+    q = gen.normal_f16(r, (G, H * D)); k = gen.normal_f16(r, (G, Hk * D))
+    q0 = q.copy()
+    pos = np.array([17, 63], np.int32)
+    oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, H * D, Hk * D, D)
+    a = _f64(q0.reshape(G, H, 2, 64)); b = _f64(q.reshape(G, H, 2, 64))
+    n0 = (a ** 2).sum(axis=2); n1 = (b ** 2).sum(axis=2)
+    assert np.max(np.abs(n1 - n0) / (n0 + 1e-3)) < 5e-3
+    oracle.rope_batch(q, k, ct, (-st.astype(np.float32)).astype(np.float16), pos, msl, G, H, Hk, D, H * D, Hk * D, D)
+    assert np.max(np.abs(_f64(q) - _f64(q0))) <= 4e-3 * np.max(np.abs(_f64(q0)))
+
+
+def test_rope_tables_follow_the_recipe(oracle):
+    ct, st = oracle.rope_tables(200, 64, 1e6)
+    want_c, want_s = _tables(None, 200, 64, 1e6)
+    # float32 powf/cosf against float64: a few fp16 steps at large angles
+    assert np.max(np.abs(_f64(ct) - _f64(want_c))) < 4e-3 and np.max(np.abs(_f64(st) - _f64(want_s))) < 4e-3
+    assert np.all(ct[0] == 1.0) and np.all(st[0] == 0.0)

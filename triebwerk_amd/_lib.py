@@ -36,6 +36,10 @@ SIGNATURES = {
     "launch_gqa_prefill_attention": (None, [P, P, P, P, P, I, I, I, I, I, I, I, P]),
     "launch_turbo_gqa_prefill_attention": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
     "launch_increment_positions": (None, [P, I, P]),
+    "launch_qk_norm_batch": (None, [P, P, P, P, I, I, I, I, C.c_float, I, I, P, C.c_bool]),
+    "launch_rope_batch": (None, [P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
+    "launch_qk_norm": (None, [P, P, P, P, I, I, I, C.c_float, P]),
+    "launch_rope": (None, [P, P, P, P, I, I, I, I, I, P]),
     # Part 2
     "tw_kv_last_error": (I, []),
     "tw_kv_last_error_string": (C.c_char_p, []),
@@ -50,6 +54,10 @@ SIGNATURES = {
     "tw_attention_workspace_floats": (SZ, [I, I, I]),
     "tw_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_turbo_append_attention_batch": (None, [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
+    "tw_qk_norm_rope_turbo_append_attention_batch": (None, [P, P, P, P, P, P, C.c_float, I, P, P, I, P, P, P, P, P, P, P,
+                                                            I, I, I, I, I, I, I, I, P]),
+    "tw_qk_norm_rope_append_attention_batch": (None, [P, P, P, P, P, P, C.c_float, I, P, P, I, P, P, P, P,
+                                                      I, I, I, I, I, I, I, P]),
     "tw_paged_kv_cache_write_batch": (None, [P, P, P, P, P, P, I, I, I, P]),
     "tw_paged_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_paged_gqa_attention_batch": (None, [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
@@ -69,6 +77,7 @@ SIGNATURES = {
     "tw_engine_positions": (P, [P]),
     "tw_engine_rotation": (P, [P]),
     "tw_engine_set_positions": (I, [P, P, I]),
+    "tw_engine_set_producers": (I, [P, I, P, P, C.c_float, I, P, P, I]),
     "tw_engine_layer_step": (I, [P, I, P, P, P, P, P]),
     "tw_engine_decode_step": (I, [P, P, P, P, P, I, P]),
     "tw_engine_broadcast_prefix": (I, [P, I, I, I, I, P]),

@@ -500,6 +500,175 @@ void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_ha
     run_attention(a, s, fn, /*query_done=*/true);
 }
 
+// ---------------------------------------------------------------- producers of q and k
+static bool check_rope_dim(const char* fn, int rope_dim) {
+    if (rope_dim == kHeadDim || (rope_dim >= 16 && rope_dim <= 64 && rope_dim % 16 == 0)) return true;
+    set_error(1, "%s: rope_dim=%d, expected 128 or a multiple of 16 up to 64", fn, rope_dim);
+    return false;
+}
+
+static void fill_producer(ProducerArgs& p, tw_half* q, tw_half* k, int rows, int num_heads,
+                          int num_kv_heads, long long q_stride, long long kv_stride) {
+    memset(&p, 0, sizeof(p));
+    p.q = reinterpret_cast<half_t*>(q);
+    p.k = reinterpret_cast<half_t*>(k);
+    p.rows = rows;
+    p.num_heads = num_heads;
+    p.num_kv_heads = num_kv_heads;
+    p.q_stride = q_stride;
+    p.kv_stride = kv_stride;
+}
+
+void launch_qk_norm_batch(tw_half* q, tw_half* k, const tw_half* q_weight, const tw_half* k_weight,
+                          int num_q, int num_kv, int head_dim, int G, float eps, int q_dim,
+                          int kv_dim, hipStream_t s, bool biased) {
+    const char* fn = "launch_qk_norm_batch";
+    if (head_dim != kHeadDim) { set_error(1, "%s: head_dim=%d, only 128 is supported", fn, head_dim); return; }
+    ProducerArgs p;
+    fill_producer(p, q, k, G, num_q, num_kv, q_dim, kv_dim);
+    p.norm = 1; p.q_weight = H(q_weight); p.k_weight = H(k_weight); p.eps = eps; p.biased = biased ? 1 : 0;
+    launch_producer(p, s);
+    check_launch(fn);
+}
+
+void launch_rope_batch(tw_half* q, tw_half* k, const tw_half* cos_table, const tw_half* sin_table,
+                       const int* positions, int max_seq_len, int G, int num_heads,
+                       int num_kv_heads, int head_dim, int q_dim, int kv_dim, int rope_dim,
+                       hipStream_t s) {
+    (void)max_seq_len;
+    const char* fn = "launch_rope_batch";
+    if (head_dim != kHeadDim) { set_error(1, "%s: head_dim=%d, only 128 is supported", fn, head_dim); return; }
+    if (!check_rope_dim(fn, rope_dim)) return;
+    ProducerArgs p;
+    fill_producer(p, q, k, G, num_heads, num_kv_heads, q_dim, kv_dim);
+    p.cos_table = H(cos_table); p.sin_table = H(sin_table); p.rope_dim = rope_dim; p.positions = positions;
+    launch_producer(p, s);
+    check_launch(fn);
+}
+
+void launch_qk_norm(tw_half* q, tw_half* k, const tw_half* q_weight, const tw_half* k_weight,
+                    int num_q_heads, int num_kv_heads, int head_dim, float eps, hipStream_t stream) {
+    const char* fn = "launch_qk_norm";
+    if (head_dim != kHeadDim) { set_error(1, "%s: head_dim=%d, only 128 is supported", fn, head_dim); return; }
+    ProducerArgs p;
+    fill_producer(p, q, k, 1, num_q_heads, num_kv_heads, 0, 0);
+    p.norm = 1; p.q_weight = H(q_weight); p.k_weight = H(k_weight); p.eps = eps;
+    launch_producer(p, stream);
+    check_launch(fn);
+}
+
+void launch_rope(tw_half* q, tw_half* k, const tw_half* cos_table, const tw_half* sin_table,
+                 int pos, int max_seq_len, int num_heads, int num_kv_heads, int head_dim,
+                 hipStream_t stream) {
+    (void)max_seq_len;
+    const char* fn = "launch_rope";
+    if (head_dim != kHeadDim) { set_error(1, "%s: head_dim=%d, only 128 is supported", fn, head_dim); return; }
+    ProducerArgs p;
+    fill_producer(p, q, k, 1, num_heads, num_kv_heads, 0, 0);
+    p.cos_table = H(cos_table); p.sin_table = H(sin_table); p.rope_dim = head_dim;
+    p.pos_scalar = pos; p.single_order = 1;
+    launch_producer(p, stream);
+    check_launch(fn);
+}
+
+void tw_qk_norm_rope_turbo_append_attention_batch(
+    tw_half* out, tw_half* q, tw_half* k_buf, const tw_half* v_buf, const tw_half* q_weight,
+    const tw_half* k_weight, float eps, int biased, const tw_half* cos_table,
+    const tw_half* sin_table, int rope_dim, uint8_t* ck_q, uint8_t* cv_q, tw_half* k_norms,
+    tw_half* v_norms, const tw_half* rotation, float* as, const int* pos, int msl, int G,
+    int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim, int bits, hipStream_t s) {
+    const char* fn = "tw_qk_norm_rope_turbo_append_attention_batch";
+    if (!check_shape(fn, num_heads, num_kv_heads, head_dim) || !check_bits(fn, bits)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, kv_dim);
+        return;
+    }
+    if (cos_table && !check_rope_dim(fn, rope_dim)) return;
+    if ((q_weight == nullptr) != (k_weight == nullptr) || (cos_table == nullptr) != (sin_table == nullptr)) {
+        set_error(1, "%s: q_weight/k_weight and cos_table/sin_table come in pairs", fn);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads,
+                num_kv_heads, bits, as);
+    a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    plan_splits(a, msl, msl);
+    const int R = num_heads / num_kv_heads;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(q_weight) | reinterpret_cast<uintptr_t>(k_weight) |
+                           reinterpret_cast<uintptr_t>(cos_table) | reinterpret_cast<uintptr_t>(sin_table)) & 15u) == 0;
+    const bool fuse = g_variant.load() != 1 && mfma_wanted(a) && a.qrot && (R == 1 || R == 2 || R == 4) &&
+                      (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0 && aligned;
+    if (!fuse) {   // the kernels of their own, in place, then the plain fused step
+        if (q_weight) launch_qk_norm_batch(q, k_buf, q_weight, k_weight, num_heads, num_kv_heads, head_dim, G, eps,
+                                           q_dim, kv_dim, s, biased != 0);
+        if (cos_table) launch_rope_batch(q, k_buf, cos_table, sin_table, pos, msl, G, num_heads, num_kv_heads,
+                                         head_dim, q_dim, kv_dim, rope_dim, s);
+        tw_turbo_append_attention_batch(out, q, k_buf, v_buf, ck_q, cv_q, k_norms, v_norms, rotation, as, pos, msl,
+                                        G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits, s);
+        return;
+    }
+    RotArgs r;
+    memset(&r, 0, sizeof(r));
+    fill_quant_segments(r, ck_q, k_norms, k_buf, cv_q, v_norms, v_buf, 2, G, num_kv_heads, kv_dim);
+    int k = r.nseg++;
+    r.seg_src[k] = H(q);
+    r.seg_stride[k] = q_dim;
+    r.seg_heads[k] = num_heads;
+    r.seg_nvec[k] = G * num_heads;
+    r.seg_units[k] = (r.seg_nvec[k] + 15) / 16 * 8;
+    r.seg_kind[k] = 1;
+    r.rotation = H(rotation);
+    r.positions = pos;
+    r.seq_stride_rows = msl;
+    r.num_kv_heads = num_kv_heads;
+    r.qrot = a.qrot;
+    r.qrot_stride = a.ws_stride;
+    r.q_scale = attention_mfma_q_scale(bits);
+    // segment 0 = K rows, 1 = V rows (left as they are), 2 = Q rows
+    r.seg_weight[0] = H(k_weight);
+    r.seg_weight[2] = H(q_weight);
+    r.seg_rope[0] = r.seg_rope[2] = cos_table ? 1 : 0;
+    r.eps = eps;
+    r.biased = biased ? 1 : 0;
+    r.cos_table = H(cos_table);
+    r.sin_table = H(sin_table);
+    r.rope_dim = rope_dim;
+    launch_rotate(r, bits, s);
+    run_attention(a, s, fn, /*query_done=*/true);
+}
+
+void tw_qk_norm_rope_append_attention_batch(
+    tw_half* out, tw_half* q, const tw_half* k_buf, const tw_half* v_buf, const tw_half* q_weight,
+    const tw_half* k_weight, float eps, int biased, const tw_half* cos_table,
+    const tw_half* sin_table, int rope_dim, tw_half* ck, tw_half* cv, float* as, const int* pos,
+    int msl, int G, int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+    hipStream_t s) {
+    const char* fn = "tw_qk_norm_rope_append_attention_batch";
+    if (!check_shape(fn, num_heads, num_kv_heads, head_dim)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, kv_dim);
+        return;
+    }
+    if (cos_table && !check_rope_dim(fn, rope_dim)) return;
+    if ((q_weight == nullptr) != (k_weight == nullptr) || (cos_table == nullptr) != (sin_table == nullptr)) {
+        set_error(1, "%s: q_weight/k_weight and cos_table/sin_table come in pairs", fn);
+        return;
+    }
+    ProducerArgs p;
+    fill_producer(p, q, const_cast<tw_half*>(k_buf), G, num_heads, num_kv_heads, q_dim, kv_dim);
+    p.v = reinterpret_cast<half_t*>(const_cast<tw_half*>(v_buf));
+    p.norm = q_weight ? 1 : 0; p.q_weight = H(q_weight); p.k_weight = H(k_weight); p.eps = eps; p.biased = biased ? 1 : 0;
+    p.cos_table = H(cos_table); p.sin_table = H(sin_table); p.rope_dim = rope_dim; p.positions = pos;
+    p.write_cache = 1;
+    p.cache_k = reinterpret_cast<half_t*>(ck);
+    p.cache_v = reinterpret_cast<half_t*>(cv);
+    p.kv_dim = kv_dim;
+    p.seq_stride_rows = msl;
+    launch_producer(p, s);
+    check_launch(fn);
+    launch_gqa_attention_batch(out, q, ck, cv, as, pos, msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, s);
+}
+
 void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const uint8_t* ck_q,
                                         const uint8_t* cv_q, const tw_half* k_norms,
                                         const tw_half* v_norms, const tw_half* rotation, float* as,

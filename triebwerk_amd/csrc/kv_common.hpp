@@ -104,6 +104,14 @@ __device__ __forceinline__ bool chunk_nonempty(int n, int c, int nsplit) {
     return chunk_boundary(tiles, (unsigned)c + 1u, (unsigned)nsplit) > chunk_boundary(tiles, (unsigned)c, (unsigned)nsplit);
 }
 
+// fp32 -> fp16 of a value that must first exist as a rounded fp32 number.  Without the barrier the
+// compiler folds a preceding multiply or fused multiply-add into the conversion (v_fma_mixlo_f16: one
+// rounding instead of two), which changes a result in a few hundred thousand.
+__device__ __forceinline__ float as_half_value(float x) {
+    asm volatile("" : "+v"(x));
+    return (float)(half_t)x;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));

@@ -46,6 +46,17 @@ struct tw_engine {
 
     hipStream_t stream = nullptr;     // engine_stream_, engine.cpp:309
 
+    // producers of q and k run with the step (forward_layer_batch step 3, engine.cpp:1972-1977);
+    // caller-owned device memory: weights (num_layers, head_dim), tables (positions, rope_dim / 2)
+    int producers = 0;                // 0 none, 1 fused into the append, 2 as launches of their own
+    const tw_half* q_norm = nullptr;
+    const tw_half* k_norm = nullptr;
+    float norm_eps = 1e-6f;
+    int norm_biased = 0;
+    const tw_half* rope_cos = nullptr;
+    const tw_half* rope_sin = nullptr;
+    int rope_dim = 0;
+
     // captured decode step
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
@@ -125,17 +136,43 @@ int carve(tw_engine* e, int G, int msl) {
 
 hipStream_t pick(tw_engine* e, hipStream_t s) { return s ? s : e->stream; }
 
-// forward_layer_batch steps 4-5, engine.cpp:1979-2006.
+// forward_layer_batch steps 4-5 (with producers: 3-5), engine.cpp:1972-2006.
 void layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, const tw_half* v,
                 tw_half* out, hipStream_t s) {
     const tw_model_shape& m = e->shape;
+    tw_half* qm = const_cast<tw_half*>(q);      // with producers q and k are the caller's scratch rows
+    tw_half* km = const_cast<tw_half*>(k);
+    const tw_half* qw = e->q_norm ? e->q_norm + (size_t)layer * m.head_dim : nullptr;
+    const tw_half* kw = e->k_norm ? e->k_norm + (size_t)layer * m.head_dim : nullptr;
+    if (e->producers == 2) {                    // the reference's sequence of launches
+        if (qw) launch_qk_norm_batch(qm, km, qw, kw, m.num_heads, m.num_kv_heads, m.head_dim, e->G, e->norm_eps,
+                                     e->q_dim(), e->kv_dim(), s, e->norm_biased != 0);
+        if (e->rope_cos) launch_rope_batch(qm, km, e->rope_cos, e->rope_sin, e->d_positions, e->batch_msl, e->G,
+                                           m.num_heads, m.num_kv_heads, m.head_dim, e->q_dim(), e->kv_dim(),
+                                           e->rope_dim, s);
+    }
+    const bool fused = e->producers == 1;
     if (e->kv_bits == 0) {
+        if (fused) {
+            tw_qk_norm_rope_append_attention_batch(out, qm, k, v, qw, kw, e->norm_eps, e->norm_biased, e->rope_cos,
+                                                   e->rope_sin, e->rope_dim, (tw_half*)e->cache[layer][0],
+                                                   (tw_half*)e->cache[layer][1], e->attn_scores, e->d_positions,
+                                                   e->batch_msl, e->G, m.num_heads, m.num_kv_heads, m.head_dim,
+                                                   e->q_dim(), e->kv_dim(), s);
+            return;
+        }
         launch_kv_cache_write_batch((tw_half*)e->cache[layer][0], (tw_half*)e->cache[layer][1], k, v,
                                     e->d_positions, e->batch_msl, e->G, e->kv_dim(), s);
         launch_gqa_attention_batch(out, q, (const tw_half*)e->cache[layer][0],
                                    (const tw_half*)e->cache[layer][1], e->attn_scores, e->d_positions,
                                    e->batch_msl, e->G, m.num_heads, m.num_kv_heads, m.head_dim,
                                    e->q_dim(), e->kv_dim(), s);
+    } else if (fused) {
+        tw_qk_norm_rope_turbo_append_attention_batch(
+            out, qm, km, v, qw, kw, e->norm_eps, e->norm_biased, e->rope_cos, e->rope_sin, e->rope_dim,
+            (uint8_t*)e->cache[layer][0], (uint8_t*)e->cache[layer][1], (tw_half*)e->cache[layer][2],
+            (tw_half*)e->cache[layer][3], e->d_rotation, e->attn_scores, e->d_positions, e->batch_msl, e->G,
+            m.num_heads, m.num_kv_heads, m.head_dim, e->q_dim(), e->kv_dim(), e->kv_bits, s);
     } else {
         tw_turbo_append_attention_batch(out, q, k, v, (uint8_t*)e->cache[layer][0],
                                         (uint8_t*)e->cache[layer][1], (tw_half*)e->cache[layer][2],
@@ -255,6 +292,18 @@ int tw_engine_set_positions(tw_engine* e, const int* host_positions, int G) {
         if (host_positions[g] < 0 || host_positions[g] >= e->batch_msl) return -2;
     // engine.cpp:2364
     return hipMemcpy(e->d_positions, host_positions, (size_t)G * sizeof(int), hipMemcpyHostToDevice) == hipSuccess ? 0 : -3;
+}
+
+int tw_engine_set_producers(tw_engine* e, int mode, const tw_half* q_norm, const tw_half* k_norm, float eps,
+                            int biased, const tw_half* rope_cos, const tw_half* rope_sin, int rope_dim) {
+    if (mode < 0 || mode > 2) return -1;
+    if ((q_norm == nullptr) != (k_norm == nullptr) || (rope_cos == nullptr) != (rope_sin == nullptr)) return -1;
+    if (rope_cos && !(rope_dim == 128 || (rope_dim >= 16 && rope_dim <= 64 && rope_dim % 16 == 0))) return -1;
+    e->drop_graph();                  // a captured step holds the old sequence of launches
+    e->producers = (q_norm || rope_cos) ? mode : 0;
+    e->q_norm = q_norm; e->k_norm = k_norm; e->norm_eps = eps; e->norm_biased = biased ? 1 : 0;
+    e->rope_cos = rope_cos; e->rope_sin = rope_sin; e->rope_dim = rope_dim;
+    return 0;
 }
 
 int tw_engine_layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k,

@@ -33,6 +33,34 @@ void launch_kv_write(half_t* ck, half_t* cv, const half_t* k, const half_t* v,
 void launch_turbo_quantize(const QuantArgs& a, int bits, hipStream_t s);
 void launch_increment(int* positions, int G, hipStream_t s);
 
+// ---------------------------------------------------------------- producers of q and k (kv_producer.hip)
+struct ProducerArgs {
+    half_t* q;               // (rows, q_stride), transformed in place
+    half_t* k;               // (rows, kv_stride)
+    half_t* v;               // write_cache only
+    long long q_stride, kv_stride;
+    int rows, num_heads, num_kv_heads;
+    int norm;                // per-head RMSNorm with q_weight / k_weight
+    const half_t* q_weight;  // (128)
+    const half_t* k_weight;
+    float eps;
+    int biased;              // weight + 1
+    const half_t* cos_table; // NULL: no rotation; (positions, rope_dim / 2)
+    const half_t* sin_table;
+    int rope_dim;
+    int single_order;        // operand order of the single-sequence rope kernel
+    const int* positions;    // device int32[rows], or NULL: pos_scalar
+    int pos_scalar;
+    int write_cache;         // K (transformed) and V rows go to their fp16 cache rows instead of back
+    half_t* cache_k;
+    half_t* cache_v;
+    int kv_dim;              // halves per cache row
+    const int* block_table;
+    int bt_stride;
+    long long seq_stride_rows;
+};
+void launch_producer(const ProducerArgs& a, hipStream_t s);
+
 // ---------------------------------------------------------------- rotation on the matrix cores
 struct RotArgs {
     int nseg;                    // up to 3 segments: K rows, V rows (quantize), Q rows (rotate only)
@@ -54,6 +82,14 @@ struct RotArgs {
     float* qrot;                 // query output: vector v at qrot + v * qrot_stride (fp32)
     long long qrot_stride;
     float q_scale;
+    // optional producers applied to a segment's vectors before anything else (kv_producer.hip has the rules)
+    const half_t* seg_weight[3]; // per-head RMSNorm weight (128), NULL = none
+    int seg_rope[3];             // rotate with the tables below at positions[row]
+    float eps;
+    int biased;
+    const half_t* cos_table;     // (positions, rope_dim / 2)
+    const half_t* sin_table;
+    int rope_dim;                // multiple of 16
 };
 
 void launch_rotate(const RotArgs& a, int bits, hipStream_t s);

@@ -1,0 +1,151 @@
+// kv_producer.hip -- the producers of q and k in front of the KV append, for gfx950:
+// per-head RMSNorm (qk_norm_kernel, kernels.cu:137-186; qk_norm_batch_kernel, 880-923) and rotary
+// position embedding (rope_kernel, 193-235; rope_batch_kernel, 927-961), as kernels of their own
+// with the reference's in-place semantics, and fused with the fp16 append (one launch instead of
+// qk_norm + rope + kv_cache_write).  The fusion into the compressed append lives in
+// kv_rotate.hip and uses norm_rope_values() below on its own register layout.
+//
+// Bits.  Both steps round to fp16 in between, as the reference's in-place kernels do:
+//   normed = half((float(x) * rms) * w),  rms = 1 / sqrt(sum / 128 + eps), w + 1 when `biased`;
+//   out0 = half(fma(x0, c, -(x1 * s)));   out1 = half(fma(x0, s, x1 * c))   (batch kernel), or
+//   out1 = half(fma(x1, c, x0 * s))   (single-sequence kernel, whose source has the other order).
+// The sum of squares keeps the reference's reduction tree: a 32-lane shuffle-down tree per group of
+// 32 coordinates, then (s0 + s2) + (s1 + s3).
+//
+// Mapping: one 64-lane wave owns a head vector, lane l holds coordinates l and l + 64, so the
+// rotary pair (d, d + 64) of a full-width rotation sits in one lane; a partial rotation (rope_dim <
+// 128) fetches the partner with a wave shuffle.  4 waves per workgroup.
+
+#include "kv_common.hpp"
+#include "kv_kernels.hpp"
+
+// Every product below is rounded to fp32 before anything else happens to it, as in the reference's
+// separate kernels: no fused multiply-add where the source has none, and no multiply fused into the
+// conversion to fp16 (one rounding instead of two changes a result in a few hundred thousand).
+#pragma clang fp contract(off)
+
+namespace twkv {
+
+namespace {
+
+constexpr int kProdWaves = 4;
+
+// sum over the 128 coordinates of a head in the reference's order; lane l passes (x[l], x[l + 64])
+__device__ __forceinline__ float head_tree_sum(float a, float b) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {     // lanes 0 and 32 end up with the sums of their 32 coordinates
+        a += __shfl_down(a, off, 32);
+        b += __shfl_down(b, off, 32);
+    }
+    const float t = a + b;                        // lane 0: s0 + s2, lane 32: s1 + s3
+    return __shfl(t, 0, 64) + __shfl(t, 32, 64);
+}
+
+struct HeadXform {
+    const half_t* weight;   // NULL: no RMSNorm
+    float eps;
+    int biased;
+    const half_t* cos_row;  // NULL: no rotation; row of rope_dim / 2 entries for this position
+    const half_t* sin_row;
+    int rope_dim;
+    int single_order;       // second output as fma(x1, c, x0 * s)
+};
+
+// RMSNorm and rotation of one head held as (x0 = coordinate lane, x1 = coordinate lane + 64), with the
+// fp16 rounding after each step
+__device__ __forceinline__ void xform_head(float& x0, float& x1, int lane, const HeadXform& t) {
+    if (t.weight) {
+        const float sum = head_tree_sum(x0 * x0, x1 * x1);
+        const float rms = 1.0f / sqrtf(sum / (float)kHeadDim + t.eps);
+        float w0 = (float)t.weight[lane], w1 = (float)t.weight[lane + 64];
+        if (t.biased) { w0 += 1.0f; w1 += 1.0f; }
+        x0 = as_half_value((x0 * rms) * w0);
+        x1 = as_half_value((x1 * rms) * w1);
+    }
+    if (t.cos_row) {
+        const int half = t.rope_dim >> 1;
+        if (half == 64) {
+            const float c = (float)t.cos_row[lane], s = (float)t.sin_row[lane];
+            const float o0 = __builtin_fmaf(x0, c, -(x1 * s));
+            const float o1 = t.single_order ? __builtin_fmaf(x1, c, x0 * s) : __builtin_fmaf(x0, s, x1 * c);
+            x0 = as_half_value(o0);
+            x1 = as_half_value(o1);
+        } else {
+            // coordinate d < rope_dim pairs with d + half (d < half) or d - half; only x0's coordinates
+            // (d = lane < 64) can be inside a partial rotation
+            const bool first = lane < half, inside = lane < t.rope_dim;
+            const int partner = first ? lane + half : lane - half;
+            const float other = __shfl(x0, inside ? partner : lane, 64);
+            if (inside) {
+                const int j = first ? lane : partner;
+                const float c = (float)t.cos_row[j], s = (float)t.sin_row[j];
+                const float a = first ? x0 : other, b = first ? other : x0;      // (x_d, x_{d + half})
+                const float o = first ? __builtin_fmaf(a, c, -(b * s))
+                                      : (t.single_order ? __builtin_fmaf(b, c, a * s) : __builtin_fmaf(a, s, b * c));
+                x0 = as_half_value(o);
+            }
+        }
+    }
+}
+
+}  // namespace
+
+// One head vector per wave.  Vector v = (row, head) with Q heads first, then K heads, then (write mode)
+// V heads.  mode 0: transform Q and K in place.  mode 1: Q in place, K into its cache row, V copied
+// into its cache row.
+__global__ void __launch_bounds__(kProdWaves* kWave)
+producer_kernel(ProducerArgs a) {
+    const int lane = threadIdx.x % kWave;
+    const long long v = (long long)blockIdx.x * kProdWaves + threadIdx.x / kWave;
+    const int per_row = a.num_heads + a.num_kv_heads * (a.write_cache ? 2 : 1);
+    if (v >= (long long)a.rows * per_row) return;
+    const int row = (int)(v / per_row);
+    int head = (int)(v - (long long)row * per_row);
+    const int pos = a.positions ? a.positions[row] : a.pos_scalar;
+
+    half_t* src;
+    half_t* dst;
+    const half_t* w;
+    bool xform = true;
+    if (head < a.num_heads) {
+        src = a.q + (long long)row * a.q_stride + (long long)head * kHeadDim;
+        dst = src;
+        w = a.q_weight;
+    } else {
+        head -= a.num_heads;
+        const bool is_v = head >= a.num_kv_heads;
+        if (is_v) head -= a.num_kv_heads;
+        half_t* base = is_v ? a.v : a.k;
+        src = base + (long long)row * a.kv_stride + (long long)head * kHeadDim;
+        dst = src;
+        w = a.k_weight;
+        xform = !is_v;
+        if (a.write_cache) {
+            const long long crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, pos);
+            dst = (is_v ? a.cache_v : a.cache_k) + crow * a.kv_dim + (long long)head * kHeadDim;
+        }
+    }
+    float x0 = (float)src[lane], x1 = (float)src[lane + 64];
+    if (xform) {
+        HeadXform t;
+        t.weight = a.norm ? w : nullptr;
+        t.eps = a.eps;
+        t.biased = a.biased;
+        t.cos_row = a.cos_table ? a.cos_table + (long long)pos * (a.rope_dim >> 1) : nullptr;
+        t.sin_row = a.cos_table ? a.sin_table + (long long)pos * (a.rope_dim >> 1) : nullptr;
+        t.rope_dim = a.rope_dim;
+        t.single_order = a.single_order;
+        xform_head(x0, x1, lane, t);
+    }
+    dst[lane] = (half_t)x0;
+    dst[lane + 64] = (half_t)x1;
+}
+
+void launch_producer(const ProducerArgs& a, hipStream_t s) {
+    const long long vecs = (long long)a.rows * (a.num_heads + a.num_kv_heads * (a.write_cache ? 2 : 1));
+    if (vecs <= 0) return;
+    const int blocks = (int)((vecs + kProdWaves - 1) / kProdWaves);
+    hipLaunchKernelGGL(producer_kernel, dim3(blocks), dim3(kProdWaves * kWave), 0, s, a);
+}
+
+}  // namespace twkv

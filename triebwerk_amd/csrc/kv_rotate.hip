@@ -2,7 +2,9 @@
 //   - the TurboQuant compressed append: y = R (x / |x|), bin search, pack, norm
 //     (turbo_kv_quantize{,_batch}_kernel, kernels.cu:1482-1636), K and V rows, and
 //   - the query rotation q_rot = R q of the compressed attention (kernels.cu:1671-1681),
-// all in one launch (any subset).
+// all in one launch (any subset); optionally with the producers of q and k applied on the way in
+// (per-head RMSNorm and rotary embedding, kernels.cu:880-961), which saves their two launches and
+// the round trip of the rows through memory.
 //
 // Bit-exactness of the append.  The reference accumulates each output coordinate as
 // one fp32 fused-multiply-add chain over k = 0..127.  v_mfma_f32_16x16x4_f32 chained
@@ -42,6 +44,21 @@ __device__ __forceinline__ float pick_half(const uint4& piece, int e, int kk) {
     return (float)cv.h;
 }
 
+// Rotary embedding of a vector held as xv[s] = coordinate 4s + kk: coordinate d < HALF pairs with d + HALF
+// (same lane, HALF4 = HALF / 4 registers further on); fp16 rounding as in rope_batch_kernel
+// (kernels.cu:927-961).  The table rows hold HALF entries and arrive as 16-byte pieces.
+template <int HALF4>
+__device__ __forceinline__ void rope_registers(float (&xv)[32], const uint4 (&cp)[8], const uint4 (&sp)[8], int kk) {
+#pragma clang fp contract(off)      // products rounded to fp32 first, as rope_batch_kernel's are
+#pragma unroll
+    for (int s = 0; s < HALF4; s++) {
+        const float c = pick_half(cp[s >> 1], s & 1, kk), sn = pick_half(sp[s >> 1], s & 1, kk);
+        const float x0 = xv[s], x1 = xv[s + HALF4];
+        xv[s] = as_half_value(__builtin_fmaf(x0, c, -(x1 * sn)));
+        xv[s + HALF4] = as_half_value(__builtin_fmaf(x0, sn, x1 * c));
+    }
+}
+
 }  // namespace
 
 template <int BITS>
@@ -67,11 +84,14 @@ rotate_kernel(RotArgs a) {
     const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (dblk * 16 + i16) * kHeadDim);
     const uint4* xsrc = reinterpret_cast<const uint4*>(a.seg_src[seg] + (long long)row * a.seg_stride[seg] +
                                                        (long long)head * kHeadDim);
-    // cache row of this vector (its load overlaps the operand loads)
+    // position of this vector's row: needed for the cache row and for the rotary table row, so it is the
+    // first thing asked for; everything that depends on it is requested before the operands are used
+    const bool roped = a.seg_rope[seg] != 0;
+    const int pos_row = (!is_query || roped) ? a.positions[row] : 0;
     long long crow = 0;
     if (!is_query) {
-        if (a.token_list) crow = a.positions[row];               // sequence 0, kernels.cu:1499, 1553
-        else crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, a.positions[row]);
+        if (a.token_list) crow = pos_row;                                // sequence 0, kernels.cu:1499, 1553
+        else crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, pos_row);
     }
     float rv[32], xv[32];
 #pragma unroll
@@ -83,9 +103,20 @@ rotate_kernel(RotArgs a) {
         xv[2 * q + 1] = pick_half(xp, 1, kk);
     }
 
-    float n2 = 0.0f;
-    if (!is_query) {
-        // sum of squares in the reference's order: xv[s] is coordinate 4s + kk; group w holds s = 8w..8w+7
+    // rotary table row of this position: rope_dim / 2 halves = rope_dim / 16 pieces
+    uint4 cpiece[8], spiece[8];
+    if (roped) {
+        const int pieces = a.rope_dim >> 4;
+        const uint4* cr = reinterpret_cast<const uint4*>(a.cos_table + (long long)pos_row * (a.rope_dim >> 1));
+        const uint4* sr = reinterpret_cast<const uint4*>(a.sin_table + (long long)pos_row * (a.rope_dim >> 1));
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            if (q < pieces) { cpiece[q] = cr[q]; spiece[q] = sr[q]; }
+        }
+    }
+
+    // sum of squares in the reference's order: xv[s] is coordinate 4s + kk; group w holds s = 8w..8w+7
+    auto tree_sum_sq = [&]() -> float {
         float sgrp[4];
 #pragma unroll
         for (int w = 0; w < 4; w++) {
@@ -99,7 +130,37 @@ rotate_kernel(RotArgs a) {
             float d = c + __shfl_xor(c, 32, 64);                 // offset 2: c0+c2 | c1+c3
             sgrp[w] = d + __shfl_xor(d, 16, 64);                 // offset 1: d0+d1
         }
-        n2 = (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
+        return (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
+    };
+
+    // ---- optional producers: per-head RMSNorm (kernels.cu:880-923), then rotary embedding (927-961),
+    // each rounded to fp16 as the in-place kernels of the reference leave it
+    if (a.seg_weight[seg]) {
+#pragma clang fp contract(off)      // (x * rms) * w: two fp32 roundings, then the one to fp16
+        const float rms = 1.0f / sqrtf(tree_sum_sq() / (float)kHeadDim + a.eps);
+        const uint4* wsrc = reinterpret_cast<const uint4*>(a.seg_weight[seg]);
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            const uint4 wp = wsrc[q];
+            float w0 = pick_half(wp, 0, kk), w1 = pick_half(wp, 1, kk);
+            if (a.biased) { w0 += 1.0f; w1 += 1.0f; }
+            xv[2 * q] = as_half_value((xv[2 * q] * rms) * w0);
+            xv[2 * q + 1] = as_half_value((xv[2 * q + 1] * rms) * w1);
+        }
+    }
+    if (roped) {
+        switch (a.rope_dim >> 1) {                               // rope_dim: 128, or a multiple of 16 up to 64
+            case 64: rope_registers<16>(xv, cpiece, spiece, kk); break;
+            case 32: rope_registers<8>(xv, cpiece, spiece, kk); break;
+            case 24: rope_registers<6>(xv, cpiece, spiece, kk); break;
+            case 16: rope_registers<4>(xv, cpiece, spiece, kk); break;
+            default: rope_registers<2>(xv, cpiece, spiece, kk); break;
+        }
+    }
+
+    float n2 = 0.0f;
+    if (!is_query) {
+        n2 = tree_sum_sq();
         const float inv = 1.0f / sqrtf(n2 + 1e-12f);
 #pragma unroll
         for (int s = 0; s < 32; s++) xv[s] *= inv;

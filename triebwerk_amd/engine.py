@@ -104,6 +104,19 @@ class Engine:
         if rc != 0:
             raise ValueError(f"set_positions failed ({rc})")
 
+    def set_producers(self, mode, q_norm=None, k_norm=None, eps=1e-6, biased=False, rope_cos=None, rope_sin=None,
+                      rope_dim=0) -> None:
+        """Run the per-head RMSNorm (weights (L, D) per layer) and the rotary embedding (tables
+        (positions, rope_dim/2)) of q and k with every step: mode 1 fused into the append, mode 2 as the
+        reference's two launches, 0 off.  The tensors must stay alive while they are set."""
+        rc = self._lib.tw_engine_set_producers(self._h, int(mode), _ptr(q_norm, "f16", "q_norm"),
+                                               _ptr(k_norm, "f16", "k_norm"), float(eps), int(biased),
+                                               _ptr(rope_cos, "f16", "rope_cos"), _ptr(rope_sin, "f16", "rope_sin"),
+                                               int(rope_dim))
+        if rc != 0:
+            raise ValueError(f"set_producers failed ({rc})")
+        self._producers = (q_norm, k_norm, rope_cos, rope_sin)
+
     def layer_step(self, layer, q, k, v, out, stream=None) -> None:
         rc = self._lib.tw_engine_layer_step(self._h, layer, _ptr(q, "f16", "q"), _ptr(k, "f16", "k"),
                                             _ptr(v, "f16", "v"), _ptr(out, "f16", "out"), _stream(stream))

@@ -230,3 +230,66 @@ def set_attention_variant(variant: int) -> None:
 
 def set_num_splits(nsplit: int) -> None:
     _lib.load().tw_kv_set_num_splits(int(nsplit))
+
+
+# ---- producers of q and k (engine.cpp:126-127, 162-163), in place
+def launch_qk_norm_batch(q, k, q_weight, k_weight, num_q, num_kv, head_dim, G, eps, q_dim, kv_dim,
+                         stream=None, biased=False):
+    lib = _lib.load()
+    lib.launch_qk_norm_batch(_ptr(q, "f16", "q"), _ptr(k, "f16", "k"), _ptr(q_weight, "f16", "q_weight"),
+                             _ptr(k_weight, "f16", "k_weight"), num_q, num_kv, head_dim, G, eps, q_dim, kv_dim,
+                             _stream(stream), bool(biased))
+    _done(lib)
+
+
+def launch_rope_batch(q, k, cos_table, sin_table, positions, max_seq_len, G, num_heads, num_kv_heads,
+                      head_dim, q_dim, kv_dim, rope_dim, stream=None):
+    lib = _lib.load()
+    lib.launch_rope_batch(_ptr(q, "f16", "q"), _ptr(k, "f16", "k"), _ptr(cos_table, "f16", "cos_table"),
+                          _ptr(sin_table, "f16", "sin_table"), _ptr(positions, "i32", "positions"), max_seq_len,
+                          G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, rope_dim, _stream(stream))
+    _done(lib)
+
+
+def launch_qk_norm(q, k, q_weight, k_weight, num_q_heads, num_kv_heads, head_dim, eps, stream=None):
+    lib = _lib.load()
+    lib.launch_qk_norm(_ptr(q, "f16", "q"), _ptr(k, "f16", "k"), _ptr(q_weight, "f16", "q_weight"),
+                       _ptr(k_weight, "f16", "k_weight"), num_q_heads, num_kv_heads, head_dim, eps,
+                       _stream(stream))
+    _done(lib)
+
+
+def launch_rope(q, k, cos_table, sin_table, pos, max_seq_len, num_heads, num_kv_heads, head_dim, stream=None):
+    lib = _lib.load()
+    lib.launch_rope(_ptr(q, "f16", "q"), _ptr(k, "f16", "k"), _ptr(cos_table, "f16", "cos_table"),
+                    _ptr(sin_table, "f16", "sin_table"), pos, max_seq_len, num_heads, num_kv_heads, head_dim,
+                    _stream(stream))
+    _done(lib)
+
+
+def tw_qk_norm_rope_turbo_append_attention_batch(out, q, k_buf, v_buf, q_weight, k_weight, eps, biased, cos_table,
+                                                 sin_table, rope_dim, ck_q, cv_q, k_norms, v_norms, rotation,
+                                                 scratch, pos, msl, G, num_heads, num_kv_heads, head_dim, q_dim,
+                                                 kv_dim, bits, stream=None):
+    lib = _lib.load()
+    lib.tw_qk_norm_rope_turbo_append_attention_batch(
+        _ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(k_buf, "f16", "k_buf"), _ptr(v_buf, "f16", "v_buf"),
+        _ptr(q_weight, "f16", "q_weight"), _ptr(k_weight, "f16", "k_weight"), eps, int(biased),
+        _ptr(cos_table, "f16", "cos_table"), _ptr(sin_table, "f16", "sin_table"), rope_dim,
+        _ptr(ck_q, "u8", "ck_q"), _ptr(cv_q, "u8", "cv_q"), _ptr(k_norms, "f16", "k_norms"),
+        _ptr(v_norms, "f16", "v_norms"), _ptr(rotation, "f16", "rotation"), _ptr(scratch, "f32", "scratch"),
+        _ptr(pos, "i32", "pos"), msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
+def tw_qk_norm_rope_append_attention_batch(out, q, k_buf, v_buf, q_weight, k_weight, eps, biased, cos_table,
+                                           sin_table, rope_dim, ck, cv, scratch, pos, msl, G, num_heads,
+                                           num_kv_heads, head_dim, q_dim, kv_dim, stream=None):
+    lib = _lib.load()
+    lib.tw_qk_norm_rope_append_attention_batch(
+        _ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(k_buf, "f16", "k_buf"), _ptr(v_buf, "f16", "v_buf"),
+        _ptr(q_weight, "f16", "q_weight"), _ptr(k_weight, "f16", "k_weight"), eps, int(biased),
+        _ptr(cos_table, "f16", "cos_table"), _ptr(sin_table, "f16", "sin_table"), rope_dim,
+        _ptr(ck, "f16", "ck"), _ptr(cv, "f16", "cv"), _ptr(scratch, "f32", "scratch"), _ptr(pos, "i32", "pos"),
+        msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, _stream(stream))
+    _done(lib)
