@@ -140,6 +140,10 @@ void launch_rope(tw_half* q, tw_half* k, const tw_half* cos_table, const tw_half
                  int pos, int max_seq_len, int num_heads, int num_kv_heads, int head_dim,
                  hipStream_t stream);
 
+/* engine.cpp:158, kernels.cu:2997 -- gated attention: data[i] = data[i] * sigmoid(gate[i]) over
+ * dim*G halves (forward_layer_batch step 6, engine.cpp:2009-2012). */
+void launch_sigmoid_gate_batch(tw_half* data, const tw_half* gate, int dim, int G, hipStream_t s);
+
 /* ------------------------------------------------------------------ Part 2
  * Error state, tuning and the entry points the reference has no twin for.   */
 
@@ -224,6 +228,38 @@ void tw_qk_norm_rope_append_attention_batch(
     const tw_half* sin_table, int rope_dim, tw_half* ck, tw_half* cv, float* as, const int* pos,
     int msl, int G, int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim,
     hipStream_t s);
+
+/* Steps 3-6 of forward_layer_batch (engine.cpp:1972-2012) for one layer in one call, every optional
+ * part switched by a NULL pointer: producers of q and k (as tw_qk_norm_rope_*), append, attention, and
+ * the sigmoid gate of gated attention applied by the kernel that writes `out`
+ * (out = half(float(half(attention)) / (1 + exp(-gate))), the arithmetic of launch_sigmoid_gate_batch).
+ * Forwards to the entry points above; their rules for q and k apply. */
+typedef struct tw_layer_step_args {
+    tw_half* out;              /* (G, q_dim) */
+    tw_half* q;                /* (G, q_dim) */
+    tw_half* k;                /* (G, kv_dim) */
+    const tw_half* v;          /* (G, kv_dim) */
+    int G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim;
+    const int* positions;      /* device int32[G] */
+    int max_seq_len;
+    const tw_half* q_weight;   /* per-head RMSNorm weights (head_dim), NULL = none */
+    const tw_half* k_weight;
+    float eps;
+    int biased;
+    const tw_half* cos_table;  /* rotary tables (positions, rope_dim/2), NULL = none */
+    const tw_half* sin_table;
+    int rope_dim;
+    int kv_bits;               /* 0 = fp16 cache, 2 or 4 = compressed */
+    void* cache_k;             /* fp16 rows or packed codes, layout of the launchers above */
+    void* cache_v;
+    tw_half* k_norms;          /* compressed only */
+    tw_half* v_norms;
+    const tw_half* rotation;   /* compressed only */
+    float* scratch;            /* G*num_heads*max_seq_len floats */
+    const tw_half* gate;       /* row g at gate + g*gate_stride, laid out like a row of out; NULL = none */
+    long long gate_stride;
+} tw_layer_step_args;
+void tw_layer_attention_step(const tw_layer_step_args* args, hipStream_t s);
 
 /* Paged cache.  A page holds TW_PAGE_TOKENS consecutive positions of one
  * sequence in the same row layout the contiguous cache uses, so

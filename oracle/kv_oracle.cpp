@@ -672,4 +672,14 @@ void tw_oracle_rope_tables(uint16_t* cos_table, uint16_t* sin_table, int max_seq
     }
 }
 
+void tw_oracle_sigmoid_gate_batch(uint16_t* data, const uint16_t* gate, int dim, int G) {
+    // sigmoid_gate_batch_kernel (kernels.cu:2987-2995): data[i] = half(d / (1 + expf(-g))) over dim * G elements
+    const long long total = (long long)dim * G;
+    for (long long i = 0; i < total; i++) {
+        float d = h2f(data[i]);
+        float g = h2f(gate[i]);
+        data[i] = f2h(d / (1.0f + expf(-g)));
+    }
+}
+
 }  // extern "C"

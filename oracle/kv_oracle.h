@@ -150,6 +150,11 @@ void tw_oracle_rope_batch(uint16_t* q, uint16_t* k, const uint16_t* cos_table, c
 /* precompute_rope, engine.cpp:554-574. */
 void tw_oracle_rope_tables(uint16_t* cos_table, uint16_t* sin_table, int max_seq_len, int rope_dim, float theta);
 
+/* sigmoid_gate_batch_kernel, kernels.cu:2987-3000: data *= sigmoid(gate), elementwise over dim*G
+ * halves (gated attention, engine.cpp:2009-2012).  expf and the division are this machine's IEEE
+ * ones; the reference's fast-math versions differ in the last bits (floating-point tolerance). */
+void tw_oracle_sigmoid_gate_batch(uint16_t* data, const uint16_t* gate, int dim, int G);
+
 /* Threads the OpenMP loops over (sequence, head) will use. */
 int  tw_oracle_num_threads(void);
 void tw_oracle_set_num_threads(int n);

@@ -54,6 +54,7 @@ class Oracle:
         lib.tw_oracle_rope.argtypes = [P, P, P, P, I, I, I, I, I]
         lib.tw_oracle_rope_batch.argtypes = [P, P, P, P, P, I, I, I, I, I, I, I, I]
         lib.tw_oracle_rope_tables.argtypes = [P, P, I, I, C.c_float]
+        lib.tw_oracle_sigmoid_gate_batch.argtypes = [P, P, I, I]
         lib.tw_oracle_num_threads.restype = I
         lib.tw_oracle_set_num_threads.argtypes = [I]
 
@@ -152,6 +153,9 @@ class Oracle:
         st = np.empty((msl, rope_dim // 2), np.float16)
         self.lib.tw_oracle_rope_tables(ct.ctypes.data, st.ctypes.data, msl, rope_dim, theta)
         return ct, st
+
+    def sigmoid_gate_batch(self, data, gate, dim, G):
+        self.lib.tw_oracle_sigmoid_gate_batch(_p(data, np.float16), _p(gate, np.float16), dim, G)
 
     def num_threads(self):
         return self.lib.tw_oracle_num_threads()

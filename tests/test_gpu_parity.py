@@ -709,6 +709,75 @@ def test_fused_norm_rope_fp16_step(kv, oracle, rope_dim):
     assert rel_err(host(out), want) <= TOL
 
 
+# ------------------------------------------------------------------ gated attention and the whole layer step
+def test_sigmoid_gate_batch(kv, oracle):
+    """Elementwise floating point (expf, division): within one fp16 step of the oracle."""
+    r = gen.rng(750)
+    dim, G = 2048, 37
+    data = gen.normal_f16(r, (G, dim)); gate = (3 * r.standard_normal((G, dim))).astype(np.float16)
+    d_data = dev(data)
+    kv.launch_sigmoid_gate_batch(d_data, dev(gate), dim, G)
+    oracle.sigmoid_gate_batch(data, gate, dim, G)
+    got = host(d_data).astype(np.float64); want = data.astype(np.float64)
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1e-4)) <= 2 ** -10
+    assert np.mean(host(d_data).view(np.uint16) == data.view(np.uint16)) > 0.999
+
+
+@pytest.mark.parametrize("kv_bits,nsplit", [(4, 0), (2, 0), (0, 0), (0, 1), (4, 1)])
+def test_layer_attention_step_with_gate(kv, oracle, rotation_fixture, kv_bits, nsplit):
+    """Producers + append + attention + sigmoid gate through one call, with the gate in the second half of
+    the q rows (gated q projection: row stride 2*H*D) == the oracle's six steps."""
+    import torch
+    r = gen.rng(760 + kv_bits + nsplit)
+    G, H, Hk, msl = 6, 16, 8, 160
+    kv_dim, q_dim = Hk * D, 2 * H * D
+    lens = np.array([1, 2, 17, 64, 100, 159])
+    pos = lens.astype(np.int32)
+    pos[5] = 159
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    qw = (1.0 + 0.2 * r.standard_normal(D)).astype(np.float16); kw = (1.0 + 0.2 * r.standard_normal(D)).astype(np.float16)
+    ct, st = rope_tables(msl, D)
+    if kv_bits:
+        ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, kv_bits, outliers=False)
+        d_kn, d_vn, d_rot = dev(kn), dev(vn), dev(rotation_fixture)
+    else:
+        ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+        for g in range(G):
+            ck[g, pos[g]:] = 0; cv[g, pos[g]:] = 0
+        d_kn = d_vn = d_rot = None
+    d_q, d_ck, d_cv = dev(q), dev(ck), dev(cv)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.set_num_splits(nsplit)
+    try:
+        kv.tw_layer_attention_step(out, d_q, dev(k), dev(v), dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, d_ck, d_cv, scratch,
+                                   kv_bits=kv_bits, k_norms=d_kn, v_norms=d_vn, rotation=d_rot, q_weight=dev(qw),
+                                   k_weight=dev(kw), eps=1e-6, cos_table=dev(ct), sin_table=dev(st), rope_dim=D,
+                                   gate=d_q, gate_stride=q_dim, gate_offset=H * D)
+    finally:
+        kv.set_num_splits(0)
+    gate_rows = q[:, H * D:].copy()
+    oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, 1e-6, q_dim, kv_dim, False)
+    oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, D)
+    want = np.zeros((G, q_dim), np.float16)
+    if kv_bits:
+        oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, kv_bits)
+        oracle.turbo_kv_quantize_batch(cv, vn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, kv_bits)
+        oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, kv_bits)
+        assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+    else:
+        oracle.kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim)
+        oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    assert_bytes_equal(host(d_ck), ck, "K cache"); assert_bytes_equal(host(d_cv), cv, "V cache")
+    attn = np.ascontiguousarray(want[:, :H * D])
+    oracle.sigmoid_gate_batch(attn, np.ascontiguousarray(gate_rows), H * D, G)
+    got = host(out)
+    assert rel_err(got[:, :H * D], attn) <= TOL
+    assert not got[:, H * D:].any(), "the gate half of the output rows is not written"
+    # the gate half of q is an input only
+    assert_bytes_equal(host(d_q)[:, H * D:], gate_rows, "gate rows")
+
+
 # ------------------------------------------------------------------ engine: append -> attention -> positions, eager and graph
 @pytest.mark.parametrize("kv_bits", [0, 4, 2])
 @pytest.mark.parametrize("use_graph", [False, True])

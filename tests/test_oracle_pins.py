@@ -652,3 +652,23 @@ def test_rope_tables_follow_the_recipe(oracle):
     # float32 powf/cosf against float64: a few fp16 steps at large angles
     assert np.max(np.abs(_f64(ct) - _f64(want_c))) < 4e-3 and np.max(np.abs(_f64(st) - _f64(want_s))) < 4e-3
     assert np.all(ct[0] == 1.0) and np.all(st[0] == 0.0)
+
+
+# ------------------------------------------------------------------ gated attention output
+def test_sigmoid_gate_is_x_times_sigmoid(oracle):
+    """data * 1/(1 + exp(-gate)) in float64; gate 0 halves exactly, a large gate leaves the bits alone,
+    a very negative one gives zero; only dim*G elements are touched."""
+    r = gen.rng(650)
+    dim, G = 256, 5
+    data = gen.normal_f16(r, (G * dim + 16,)); gate = (4 * r.standard_normal(G * dim + 16)).astype(np.float16)
+    gate[:4] = [0.0, 30.0, -30.0, -0.0]
+    data[:4] = [3.0, -1.2345, 7.0, 5.0]
+    d0 = data.copy()
+    oracle.sigmoid_gate_batch(data, gate, dim, G)
+    n = dim * G
+    want = _f64(d0[:n]) / (1.0 + np.exp(-_f64(gate[:n])))
+    assert np.max(np.abs(_f64(data[:n]) - want)) <= 2 ** -10 * np.max(np.abs(want))
+    assert data[0] == np.float16(1.5) and data[3] == np.float16(2.5)
+    assert data[1].view(np.uint16) == d0[1].view(np.uint16)
+    assert data[2] == 0
+    assert np.array_equal(data[n:].view(np.uint16), d0[n:].view(np.uint16))

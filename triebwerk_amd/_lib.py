@@ -19,6 +19,17 @@ LL = C.c_longlong
 SZ = C.c_size_t
 
 
+class LayerStepArgs(C.Structure):
+    """tw_layer_step_args of include/triebwerk_kv.h."""
+    _fields_ = [("out", P), ("q", P), ("k", P), ("v", P),
+                ("G", I), ("num_heads", I), ("num_kv_heads", I), ("head_dim", I), ("q_dim", I), ("kv_dim", I),
+                ("positions", P), ("max_seq_len", I),
+                ("q_weight", P), ("k_weight", P), ("eps", C.c_float), ("biased", I),
+                ("cos_table", P), ("sin_table", P), ("rope_dim", I),
+                ("kv_bits", I), ("cache_k", P), ("cache_v", P), ("k_norms", P), ("v_norms", P), ("rotation", P),
+                ("scratch", P), ("gate", P), ("gate_stride", LL)]
+
+
 class ModelShape(C.Structure):
     _fields_ = [("num_layers", I), ("num_heads", I), ("num_kv_heads", I), ("head_dim", I)]
 
@@ -40,6 +51,7 @@ SIGNATURES = {
     "launch_rope_batch": (None, [P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
     "launch_qk_norm": (None, [P, P, P, P, I, I, I, C.c_float, P]),
     "launch_rope": (None, [P, P, P, P, I, I, I, I, I, P]),
+    "launch_sigmoid_gate_batch": (None, [P, P, I, I, P]),
     # Part 2
     "tw_kv_last_error": (I, []),
     "tw_kv_last_error_string": (C.c_char_p, []),
@@ -58,6 +70,7 @@ SIGNATURES = {
                                                             I, I, I, I, I, I, I, I, P]),
     "tw_qk_norm_rope_append_attention_batch": (None, [P, P, P, P, P, P, C.c_float, I, P, P, I, P, P, P, P,
                                                       I, I, I, I, I, I, I, P]),
+    "tw_layer_attention_step": (None, [C.POINTER(LayerStepArgs), P]),
     "tw_paged_kv_cache_write_batch": (None, [P, P, P, P, P, P, I, I, I, P]),
     "tw_paged_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_paged_gqa_attention_batch": (None, [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),

@@ -88,7 +88,9 @@ __device__ __forceinline__ void store_head(const AttnArgs& a, int g, int head, i
 #pragma unroll 8
         for (int k = 0; k < kHeadDim; k++) o = __builtin_fmaf((float)rot[k * kHeadDim + d], o_s[k], o);
     }
-    a.out[(long long)g * a.q_stride + (long long)head * kHeadDim + d] = (half_t)o;
+    half_t h = (half_t)o;
+    if (a.gate) h = gated(h, a.gate[(long long)g * a.gate_stride + (long long)head * kHeadDim + d]);
+    a.out[(long long)g * a.q_stride + (long long)head * kHeadDim + d] = h;
 }
 
 template <int MODE, int RT>

@@ -359,6 +359,11 @@ void launch_increment_positions(int* positions, int G, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------- attention
+// Output gate of the attention call being set up on this thread (tw_layer_attention_step sets it around
+// the entry point it forwards to).
+static thread_local const tw_half* t_gate = nullptr;
+static thread_local long long t_gate_stride = 0;
+
 static void fill_common(AttnArgs& a, tw_half* out, const tw_half* q, int q_stride, const void* k,
                         const void* v, const tw_half* kn, const tw_half* vn, const tw_half* rot,
                         int G, int num_heads, int num_kv_heads, int bits, float* ws) {
@@ -367,6 +372,7 @@ static void fill_common(AttnArgs& a, tw_half* out, const tw_half* q, int q_strid
     a.k = k; a.v = v; a.k_norms = H(kn); a.v_norms = H(vn); a.rotation = H(rot);
     a.G = G; a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.bits = bits;
     a.ws = ws;
+    a.gate = H(t_gate); a.gate_stride = t_gate_stride;
 }
 
 void launch_gqa_attention(const tw_half* q, const tw_half* k_cache, const tw_half* v_cache,
@@ -667,6 +673,46 @@ void tw_qk_norm_rope_append_attention_batch(
     launch_producer(p, s);
     check_launch(fn);
     launch_gqa_attention_batch(out, q, ck, cv, as, pos, msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, s);
+}
+
+void launch_sigmoid_gate_batch(tw_half* data, const tw_half* gate, int dim, int G, hipStream_t s) {
+    launch_sigmoid_gate(reinterpret_cast<half_t*>(data), dim, H(gate), dim, dim, G, s);
+    check_launch("launch_sigmoid_gate_batch");
+}
+
+void tw_layer_attention_step(const tw_layer_step_args* p, hipStream_t s) {
+    const char* fn = "tw_layer_attention_step";
+    if (!p) { set_error(1, "%s: NULL arguments", fn); return; }
+    if (p->kv_bits != 0 && !check_bits(fn, p->kv_bits)) return;
+    const bool producers = p->q_weight || p->cos_table;
+    t_gate = p->gate;
+    t_gate_stride = p->gate ? p->gate_stride : 0;
+    if (p->kv_bits == 0) {
+        if (producers) {
+            tw_qk_norm_rope_append_attention_batch(p->out, p->q, p->k, p->v, p->q_weight, p->k_weight, p->eps, p->biased,
+                                                   p->cos_table, p->sin_table, p->rope_dim, (tw_half*)p->cache_k,
+                                                   (tw_half*)p->cache_v, p->scratch, p->positions, p->max_seq_len, p->G,
+                                                   p->num_heads, p->num_kv_heads, p->head_dim, p->q_dim, p->kv_dim, s);
+        } else {
+            launch_kv_cache_write_batch((tw_half*)p->cache_k, (tw_half*)p->cache_v, p->k, p->v, p->positions,
+                                        p->max_seq_len, p->G, p->kv_dim, s);
+            launch_gqa_attention_batch(p->out, p->q, (const tw_half*)p->cache_k, (const tw_half*)p->cache_v, p->scratch,
+                                       p->positions, p->max_seq_len, p->G, p->num_heads, p->num_kv_heads, p->head_dim,
+                                       p->q_dim, p->kv_dim, s);
+        }
+    } else if (producers) {
+        tw_qk_norm_rope_turbo_append_attention_batch(
+            p->out, p->q, p->k, p->v, p->q_weight, p->k_weight, p->eps, p->biased, p->cos_table, p->sin_table,
+            p->rope_dim, (uint8_t*)p->cache_k, (uint8_t*)p->cache_v, p->k_norms, p->v_norms, p->rotation, p->scratch,
+            p->positions, p->max_seq_len, p->G, p->num_heads, p->num_kv_heads, p->head_dim, p->q_dim, p->kv_dim,
+            p->kv_bits, s);
+    } else {
+        tw_turbo_append_attention_batch(p->out, p->q, p->k, p->v, (uint8_t*)p->cache_k, (uint8_t*)p->cache_v, p->k_norms,
+                                        p->v_norms, p->rotation, p->scratch, p->positions, p->max_seq_len, p->G,
+                                        p->num_heads, p->num_kv_heads, p->head_dim, p->q_dim, p->kv_dim, p->kv_bits, s);
+    }
+    t_gate = nullptr;
+    t_gate_stride = 0;
 }
 
 void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const uint8_t* ck_q,

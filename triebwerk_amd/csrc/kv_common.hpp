@@ -112,6 +112,11 @@ __device__ __forceinline__ float as_half_value(float x) {
     return (float)(half_t)x;
 }
 
+// sigmoid_gate_batch_kernel's arithmetic (kernels.cu:2993-2994) on an output that has already been rounded to fp16
+__device__ __forceinline__ half_t gated(half_t out, half_t gate) {
+    return (half_t)((float)out / (1.0f + expf(-(float)gate)));
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));

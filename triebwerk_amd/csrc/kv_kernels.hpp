@@ -60,6 +60,9 @@ struct ProducerArgs {
     long long seq_stride_rows;
 };
 void launch_producer(const ProducerArgs& a, hipStream_t s);
+// data[r][i] = half(data[r][i] / (1 + exp(-gate[r][i]))), rows of `dim` halves with their own strides
+void launch_sigmoid_gate(half_t* data, long long data_stride, const half_t* gate, long long gate_stride, int dim,
+                         int rows, hipStream_t s);
 
 // ---------------------------------------------------------------- rotation on the matrix cores
 struct RotArgs {
@@ -123,6 +126,9 @@ struct AttnArgs {
     int balance;            // MFMA scan: may cut the batch by tiles instead of by sequence (ragged lengths)
     int max_slots;          // partials the workspace holds per (sequence, head): >= nsplit
     int slots_from_ws;      // merge: the spare word of partial 0 holds the number of partials (0: even chunks)
+    // optional output gate (gated attention, kernels.cu:2987-2995): out = half(float(half(out)) * sigmoid(gate))
+    const half_t* gate;     // row g at gate + g * gate_stride, laid out like a row of out; NULL = none
+    long long gate_stride;
 };
 
 constexpr int kPartialFloats = kHeadDim + 4;  // acc[128], running max, running sum, 2 pad (16-byte rows)

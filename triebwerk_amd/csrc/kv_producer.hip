@@ -3,7 +3,8 @@
 // position embedding (rope_kernel, 193-235; rope_batch_kernel, 927-961), as kernels of their own
 // with the reference's in-place semantics, and fused with the fp16 append (one launch instead of
 // qk_norm + rope + kv_cache_write).  The fusion into the compressed append lives in
-// kv_rotate.hip and uses norm_rope_values() below on its own register layout.
+// kv_rotate.hip, on that kernel's register layout.  Also here: the sigmoid gate of gated attention
+// (sigmoid_gate_batch_kernel, kernels.cu:2987-2995), which the attention kernels can apply themselves.
 //
 // Bits.  Both steps round to fp16 in between, as the reference's in-place kernels do:
 //   normed = half((float(x) * rms) * w),  rms = 1 / sqrt(sum / 128 + eps), w + 1 when `biased`;
@@ -146,6 +147,39 @@ void launch_producer(const ProducerArgs& a, hipStream_t s) {
     if (vecs <= 0) return;
     const int blocks = (int)((vecs + kProdWaves - 1) / kProdWaves);
     hipLaunchKernelGGL(producer_kernel, dim3(blocks), dim3(kProdWaves * kWave), 0, s, a);
+}
+
+// ---------------------------------------------------------------- gated attention output
+// sigmoid_gate_batch_kernel (kernels.cu:2987-2995) with row strides: 8 halves per lane
+__global__ void __launch_bounds__(256)
+sigmoid_gate_kernel(half_t* data, long long data_stride, const half_t* gate, long long gate_stride, int dim,
+                    int rows, int vec_ok) {
+    const int per_row = (dim + 7) / 8;
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long long)rows * per_row) return;
+    const int r = (int)(idx / per_row), c = (int)(idx - (long long)r * per_row) * 8;
+    half_t* d = data + (long long)r * data_stride + c;
+    const half_t* g = gate + (long long)r * gate_stride + c;
+    if (vec_ok) {
+        union { uint4 u; half_t h[8]; } dv, gv;
+        dv.u = *reinterpret_cast<const uint4*>(d);
+        gv.u = *reinterpret_cast<const uint4*>(g);
+#pragma unroll
+        for (int i = 0; i < 8; i++) dv.h[i] = gated(dv.h[i], gv.h[i]);
+        *reinterpret_cast<uint4*>(d) = dv.u;
+    } else {
+        for (int i = 0; i < 8 && c + i < dim; i++) d[i] = gated(d[i], g[i]);
+    }
+}
+
+void launch_sigmoid_gate(half_t* data, long long data_stride, const half_t* gate, long long gate_stride, int dim,
+                         int rows, hipStream_t s) {
+    if (rows <= 0 || dim <= 0) return;
+    const int vec_ok = (dim % 8 == 0 && data_stride % 8 == 0 && gate_stride % 8 == 0 &&
+                        ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(gate)) & 15u) == 0) ? 1 : 0;
+    const long long n = (long long)rows * ((dim + 7) / 8);
+    hipLaunchKernelGGL(sigmoid_gate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, data, data_stride, gate,
+                       gate_stride, dim, rows, vec_ok);
 }
 
 }  // namespace twkv

@@ -310,7 +310,10 @@ merge_rotate_kernel(AttnArgs a) {
         const int vv = v0 + 4 * kk + r;
         if (vv < total) {
             const int g = vv / a.num_heads, head = vv - g * a.num_heads;
-            a.out[(long long)g * a.q_stride + (long long)head * kHeadDim + 16 * wave + i16] = (half_t)acc[r];
+            const long long col = (long long)head * kHeadDim + 16 * wave + i16;
+            half_t h = (half_t)acc[r];
+            if (a.gate) h = gated(h, a.gate[(long long)g * a.gate_stride + col]);
+            a.out[(long long)g * a.q_stride + col] = h;
         }
     }
 }

@@ -293,3 +293,35 @@ def tw_qk_norm_rope_append_attention_batch(out, q, k_buf, v_buf, q_weight, k_wei
         _ptr(ck, "f16", "ck"), _ptr(cv, "f16", "cv"), _ptr(scratch, "f32", "scratch"), _ptr(pos, "i32", "pos"),
         msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, _stream(stream))
     _done(lib)
+
+
+def launch_sigmoid_gate_batch(data, gate, dim, G, stream=None):
+    lib = _lib.load()
+    lib.launch_sigmoid_gate_batch(_ptr(data, "f16", "data"), _ptr(gate, "f16", "gate"), dim, G, _stream(stream))
+    _done(lib)
+
+
+def tw_layer_attention_step(out, q, k, v, positions, max_seq_len, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim,
+                            cache_k, cache_v, scratch, kv_bits=0, k_norms=None, v_norms=None, rotation=None,
+                            q_weight=None, k_weight=None, eps=1e-6, biased=False, cos_table=None, sin_table=None,
+                            rope_dim=0, gate=None, gate_stride=0, gate_offset=0, stream=None):
+    """Steps 3-6 of a layer (producers, append, attention, gate) through tw_layer_attention_step.
+    `gate` may be the q tensor itself with gate_offset = num_heads*head_dim (gated q projection)."""
+    lib = _lib.load()
+    a = _lib.LayerStepArgs()
+    a.out, a.q, a.k, a.v = _ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(k, "f16", "k"), _ptr(v, "f16", "v")
+    a.G, a.num_heads, a.num_kv_heads, a.head_dim, a.q_dim, a.kv_dim = G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim
+    a.positions, a.max_seq_len = _ptr(positions, "i32", "positions"), max_seq_len
+    a.q_weight, a.k_weight = _ptr(q_weight, "f16", "q_weight"), _ptr(k_weight, "f16", "k_weight")
+    a.eps, a.biased = eps, int(biased)
+    a.cos_table, a.sin_table, a.rope_dim = _ptr(cos_table, "f16", "cos_table"), _ptr(sin_table, "f16", "sin_table"), rope_dim
+    a.kv_bits = kv_bits
+    a.cache_k = _ptr(cache_k, "u8" if kv_bits else "f16", "cache_k")
+    a.cache_v = _ptr(cache_v, "u8" if kv_bits else "f16", "cache_v")
+    a.k_norms, a.v_norms = _ptr(k_norms, "f16", "k_norms"), _ptr(v_norms, "f16", "v_norms")
+    a.rotation, a.scratch = _ptr(rotation, "f16", "rotation"), _ptr(scratch, "f32", "scratch")
+    gp = _ptr(gate, "f16", "gate")
+    a.gate = (gp + 2 * gate_offset) if gp is not None else None
+    a.gate_stride = gate_stride
+    lib.tw_layer_attention_step(_lib.C.byref(a), _stream(stream))
+    _done(lib)
