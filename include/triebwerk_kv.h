@@ -368,6 +368,29 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
 int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end, int T,
                                hipStream_t s);
 
+/* sleep() / wake(), engine.cpp:922-1022: sleep hands the cache memory back (frees an arena the engine
+ * allocated, forgets one the caller owns), drops the captured step and the generation bookkeeping;
+ * wake has nothing to restore for the batch path -- tw_engine_alloc_batch (or tw_engine_set_arena +
+ * tw_engine_alloc_batch) re-creates it on the next use, zeroed. */
+int tw_engine_sleep(tw_engine* e);
+int tw_engine_wake(tw_engine* e);
+int tw_engine_is_allocated(const tw_engine* e);
+
+/* The tail of generate_batch's decode loop (engine.cpp:2350, 2496-2534), for the caller that owns the
+ * sampling: begin_generation sizes a (max_new_tokens, G) token history on the device; record_tokens
+ * copies a step's G tokens (device int32) into it without synchronising; check_stops does nothing on
+ * most steps and, every 8th step and on the last one, waits for the stream, fetches positions and the
+ * history rows not yet seen, extends the outputs of the sequences still running and marks those that
+ * produced eos_token_id or the stop sequence.  It returns 1 when every sequence has finished, 0
+ * otherwise, < 0 on error; *checked says whether the step was a checking one.  output() returns a
+ * sequence's tokens so far (host memory owned by the engine) and whether it has finished. */
+int tw_engine_begin_generation(tw_engine* e, int max_new_tokens, int eos_token_id,
+                               const int* stop_ids_host, int n_stop);
+int tw_engine_record_tokens(tw_engine* e, const int* d_tokens, int step, hipStream_t s);
+int tw_engine_check_stops(tw_engine* e, int step, hipStream_t s, int* checked);
+int tw_engine_output(tw_engine* e, int g, const int** tokens, int* n);
+int tw_engine_host_position(const tw_engine* e, int g); /* positions as of the last check */
+
 #ifdef __cplusplus
 }
 #endif

@@ -912,6 +912,99 @@ def test_engine_decode_steps_with_producers(oracle, kv_bits, mode):
     eng.set_producers(0)
 
 
+def test_engine_sleep_and_wake(oracle):
+    """sleep() hands the cache memory back and drops the captured step; after wake() + alloc_batch the
+    caches are zero again and a captured step works on the new memory."""
+    import torch
+    from triebwerk_amd import Engine
+    r = gen.rng(570)
+    L, H, Hk, G, msl = 2, 16, 8, 3, 32
+    kv_dim, q_dim = Hk * D, H * D
+    eng = Engine(kv_bits=4)
+    eng.set_shape(L, H, Hk, D)
+    d_q = dev(gen.normal_f16(r, (L, G, q_dim))); d_k = dev(gen.normal_f16(r, (L, G, kv_dim))); d_v = dev(gen.normal_f16(r, (L, G, kv_dim)))
+    d_out = torch.zeros((L, G, q_dim), dtype=torch.float16, device="cuda")
+    stream = torch.cuda.Stream()
+    outs = []
+    for cycle in range(2):
+        eng.alloc_batch(G, msl)
+        assert eng.is_allocated()
+        assert not host(eng.cache(0)[0]).any() and not host(eng.positions()).any()
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                eng.decode_step(d_q, d_k, d_v, d_out, use_graph=True, stream=stream)
+        stream.synchronize()
+        assert host(eng.positions()).tolist() == [3] * G
+        assert host(eng.cache(1)[0])[:, :3].any()
+        outs.append(host(d_out).copy())
+        eng.sleep()
+        assert not eng.is_allocated()
+        with pytest.raises(RuntimeError):
+            eng.decode_step(d_q, d_k, d_v, d_out, use_graph=True, stream=stream)
+        eng.wake()
+    assert_bytes_equal(outs[0], outs[1], "same steps after a sleep / wake cycle")
+
+
+def test_engine_stop_check_cadence():
+    """record_tokens + check_stops against a plain restatement of the reference's loop (engine.cpp:2496-2534):
+    checks on steps 7, 15, ... and the last; eos and a two-token stop sequence; sequences that finished keep
+    their output; the loop ends on the first check at which all have finished."""
+    import torch
+    from triebwerk_amd import Engine
+    r = gen.rng(580)
+    L, H, Hk, G, msl, max_new = 1, 4, 2, 6, 64, 21
+    eos, stop = 9, [3, 4]
+    eng = Engine(kv_bits=0)
+    eng.set_shape(L, H, Hk, D)
+    eng.alloc_batch(G, msl)
+    toks = r.integers(0, 12, (max_new, G)).astype(np.int32)
+    toks[:, 5] = 1                      # never stops
+    toks[2, 0] = eos                    # stops early
+    toks[9, 1], toks[10, 1] = 3, 4      # stop sequence across a check boundary? (steps 9, 10 are in one block)
+    toks[7, 2], toks[8, 2] = 3, 4       # stop sequence across the check at step 7
+    eng.begin_generation(max_new, eos, stop)
+    # model
+    outputs = [[] for _ in range(G)]; finished = [False] * G
+    last_checked, want_checks, want_done_step = -1, [], None
+    for step in range(max_new):
+        if not ((step + 1) % 8 == 0 or step + 1 == max_new):
+            continue
+        want_checks.append(step)
+        all_done = True
+        for st in range(last_checked + 1, step + 1):
+            for g in range(G):
+                if finished[g]:
+                    continue
+                t = int(toks[st, g]); outputs[g].append(t)
+                if t == eos or (len(outputs[g]) >= 2 and outputs[g][-2:] == stop):
+                    finished[g] = True
+                if not finished[g]:
+                    all_done = False
+        last_checked = step
+        if all_done:
+            want_done_step = step
+            break
+    stream = torch.cuda.Stream()
+    got_checks, done_step = [], None
+    d_tok = torch.zeros(G, dtype=torch.int32, device="cuda")
+    for step in range(max_new):
+        d_tok.copy_(dev(toks[step]))
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            eng.record_tokens(d_tok, step, stream=stream)
+        done, checked = eng.check_stops(step, stream=stream)
+        if checked:
+            got_checks.append(step)
+        if done:
+            done_step = step
+            break
+    assert got_checks == want_checks and done_step == want_done_step
+    for g in range(G):
+        out, fin = eng.output(g)
+        assert out == outputs[g] and fin == finished[g], g
+    assert not finished[5] and finished[0] and outputs[0] == [int(x) for x in toks[:3, 0]]
+
+
 def test_engine_prefix_broadcast(oracle):
     import torch
     from triebwerk_amd import Engine

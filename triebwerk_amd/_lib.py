@@ -91,6 +91,14 @@ SIGNATURES = {
     "tw_engine_rotation": (P, [P]),
     "tw_engine_set_positions": (I, [P, P, I]),
     "tw_engine_set_producers": (I, [P, I, P, P, C.c_float, I, P, P, I]),
+    "tw_engine_sleep": (I, [P]),
+    "tw_engine_wake": (I, [P]),
+    "tw_engine_is_allocated": (I, [P]),
+    "tw_engine_begin_generation": (I, [P, I, I, P, I]),
+    "tw_engine_record_tokens": (I, [P, P, I, P]),
+    "tw_engine_check_stops": (I, [P, I, P, C.POINTER(I)]),
+    "tw_engine_output": (I, [P, I, C.POINTER(C.POINTER(I)), C.POINTER(I)]),
+    "tw_engine_host_position": (I, [P, I]),
     "tw_engine_layer_step": (I, [P, I, P, P, P, P, P]),
     "tw_engine_decode_step": (I, [P, P, P, P, P, I, P]),
     "tw_engine_broadcast_prefix": (I, [P, I, I, I, I, P]),

@@ -63,6 +63,23 @@ struct tw_engine {
     const void* graph_key[4] = {};
     int graph_G = 0;
 
+    // generation bookkeeping (generate_batch, engine.cpp:2350, 2496-2534)
+    int* d_token_history = nullptr;   // (max_new_tokens, G) device
+    std::vector<int> h_token_history;
+    std::vector<int> h_positions;
+    std::vector<char> h_finished;
+    std::vector<std::vector<int>> outputs;
+    std::vector<int> stop_ids;
+    int eos_token = -1;
+    int max_new_tokens = 0;
+    int last_checked = -1;
+
+    void drop_generation() {
+        if (d_token_history) { hipFree(d_token_history); d_token_history = nullptr; }
+        h_token_history.clear(); h_positions.clear(); h_finished.clear(); outputs.clear(); stop_ids.clear();
+        max_new_tokens = 0; last_checked = -1;
+    }
+
     int kv_dim() const { return shape.num_kv_heads * shape.head_dim; }
     int q_dim() const { return shape.num_heads * shape.head_dim; }
     // KV_DIM_PACKED, engine.cpp:294
@@ -75,6 +92,7 @@ struct tw_engine {
     }
     void drop_arena() {
         drop_graph();  // the capture holds arena addresses, engine.cpp:1440-1442
+        drop_generation();
         if (arena && arena_owned) hipFree(arena);
         arena = nullptr; arena_cap = 0; arena_owned = false;
         G = 0; batch_msl = 0;
@@ -304,6 +322,100 @@ int tw_engine_set_producers(tw_engine* e, int mode, const tw_half* q_norm, const
     e->q_norm = q_norm; e->k_norm = k_norm; e->norm_eps = eps; e->norm_biased = biased ? 1 : 0;
     e->rope_cos = rope_cos; e->rope_sin = rope_sin; e->rope_dim = rope_dim;
     return 0;
+}
+
+// sleep(), engine.cpp:922-983: give the device memory back (the arena when the engine allocated it; a
+// caller's arena is only forgotten) and drop everything that points into it.  wake(), engine.cpp:985-1022,
+// has nothing to restore for the batch path: alloc_batch re-creates it on the next use.
+int tw_engine_sleep(tw_engine* e) {
+    if (e->stream) hipStreamSynchronize(e->stream);
+    e->drop_arena();
+    return 0;
+}
+
+int tw_engine_wake(tw_engine* e) {
+    (void)e;
+    return 0;
+}
+
+int tw_engine_is_allocated(const tw_engine* e) { return e->arena != nullptr && e->G > 0; }
+
+int tw_engine_begin_generation(tw_engine* e, int max_new_tokens, int eos_token_id, const int* stop_ids_host,
+                               int n_stop) {
+    if (!e->arena || e->G == 0 || max_new_tokens < 1 || n_stop < 0) return -1;
+    e->drop_generation();
+    if (hipMalloc((void**)&e->d_token_history, (size_t)max_new_tokens * e->G * sizeof(int)) != hipSuccess) return -2;
+    e->h_token_history.assign((size_t)max_new_tokens * e->G, 0);
+    e->h_positions.assign(e->G, 0);
+    e->h_finished.assign(e->G, 0);
+    e->outputs.assign(e->G, std::vector<int>());
+    e->stop_ids.assign(stop_ids_host, stop_ids_host + n_stop);
+    e->eos_token = eos_token_id;
+    e->max_new_tokens = max_new_tokens;
+    e->last_checked = -1;
+    return 0;
+}
+
+// engine.cpp:2496-2498: the step's tokens go into the history on the device, no synchronisation
+int tw_engine_record_tokens(tw_engine* e, const int* d_tokens, int step, hipStream_t s) {
+    if (!e->d_token_history || step < 0 || step >= e->max_new_tokens) return -1;
+    s = pick(e, s);
+    return hipMemcpyAsync(e->d_token_history + (size_t)step * e->G, d_tokens, (size_t)e->G * sizeof(int),
+                          hipMemcpyDeviceToDevice, s) == hipSuccess ? 0 : -2;
+}
+
+// engine.cpp:2499-2534: every 8th step and on the last one, wait for the stream, fetch positions and the
+// history rows not yet seen, extend the outputs of the sequences still running and mark those that
+// produced the end token or the stop sequence.  Returns 1 when all have finished, 0 otherwise.
+int tw_engine_check_stops(tw_engine* e, int step, hipStream_t s, int* checked) {
+    constexpr int kCheckInterval = 8;      // engine.cpp:2350
+    if (!e->d_token_history || step < 0 || step >= e->max_new_tokens) return -1;
+    const bool should_check = ((step + 1) % kCheckInterval == 0) || (step + 1 == e->max_new_tokens);
+    if (checked) *checked = should_check ? 1 : 0;
+    if (!should_check) return 0;
+    s = pick(e, s);
+    const int G = e->G;
+    if (hipStreamSynchronize(s) != hipSuccess) return -2;
+    if (hipMemcpy(e->h_positions.data(), e->d_positions, (size_t)G * sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)
+        return -2;
+    const int check_start = e->last_checked + 1;
+    const size_t count = (size_t)(step + 1 - check_start) * G;
+    if (hipMemcpy(e->h_token_history.data() + (size_t)check_start * G, e->d_token_history + (size_t)check_start * G,
+                  count * sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)
+        return -2;
+    bool all_done = true;
+    const int stop_len = (int)e->stop_ids.size();
+    for (int st = check_start; st <= step; st++) {
+        for (int g = 0; g < G; g++) {
+            if (e->h_finished[g]) continue;
+            const int tok = e->h_token_history[(size_t)st * G + g];
+            std::vector<int>& out = e->outputs[g];
+            out.push_back(tok);
+            if (tok == e->eos_token) {
+                e->h_finished[g] = 1;
+            } else if (stop_len > 0 && (int)out.size() >= stop_len) {
+                bool match = true;
+                for (int j = 0; j < stop_len; j++) {
+                    if (out[out.size() - stop_len + j] != e->stop_ids[j]) { match = false; break; }
+                }
+                if (match) e->h_finished[g] = 1;
+            }
+            if (!e->h_finished[g]) all_done = false;
+        }
+    }
+    e->last_checked = step;
+    return all_done ? 1 : 0;
+}
+
+int tw_engine_output(tw_engine* e, int g, const int** tokens, int* n) {
+    if (g < 0 || g >= (int)e->outputs.size() || !tokens || !n) return -1;
+    *tokens = e->outputs[g].data();
+    *n = (int)e->outputs[g].size();
+    return e->h_finished[g] ? 1 : 0;
+}
+
+int tw_engine_host_position(const tw_engine* e, int g) {
+    return (g >= 0 && g < (int)e->h_positions.size()) ? e->h_positions[g] : -1;
 }
 
 int tw_engine_layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k,

@@ -138,3 +138,45 @@ class Engine:
         rc = self._lib.tw_engine_broadcast_prefix(self._h, src, dst_begin, dst_end, T, _stream(stream))
         if rc != 0:
             raise RuntimeError(f"broadcast_prefix failed ({rc})")
+
+    # ---- memory lifecycle (engine.cpp:922-1022)
+    def sleep(self) -> None:
+        """Give the cache memory back (the torch arena is released) and drop the captured step."""
+        self._lib.tw_engine_sleep(self._h)
+        self._arena = None
+        self._G = self._msl = 0
+
+    def wake(self) -> None:
+        """Nothing to restore for the batch path: call alloc_batch again."""
+        self._lib.tw_engine_wake(self._h)
+
+    def is_allocated(self) -> bool:
+        return bool(self._lib.tw_engine_is_allocated(self._h))
+
+    # ---- tail of the decode loop (engine.cpp:2350, 2496-2534)
+    def begin_generation(self, max_new_tokens: int, eos_token_id: int, stop_token_ids=()) -> None:
+        ids = (C.c_int * max(len(stop_token_ids), 1))(*[int(x) for x in stop_token_ids])
+        rc = self._lib.tw_engine_begin_generation(self._h, int(max_new_tokens), int(eos_token_id), ids, len(stop_token_ids))
+        if rc != 0:
+            raise RuntimeError(f"begin_generation failed ({rc})")
+
+    def record_tokens(self, tokens, step: int, stream=None) -> None:
+        rc = self._lib.tw_engine_record_tokens(self._h, _ptr(tokens, "i32", "tokens"), int(step), _stream(stream))
+        if rc != 0:
+            raise RuntimeError(f"record_tokens failed ({rc})")
+
+    def check_stops(self, step: int, stream=None):
+        """-> (all_done, checked)"""
+        checked = C.c_int(0)
+        rc = self._lib.tw_engine_check_stops(self._h, int(step), _stream(stream), C.byref(checked))
+        if rc < 0:
+            raise RuntimeError(f"check_stops failed ({rc})")
+        return bool(rc), bool(checked.value)
+
+    def output(self, g: int):
+        """-> (tokens so far, finished)"""
+        ptr, n = C.POINTER(C.c_int)(), C.c_int(0)
+        rc = self._lib.tw_engine_output(self._h, int(g), C.byref(ptr), C.byref(n))
+        if rc < 0:
+            raise IndexError(g)
+        return [ptr[i] for i in range(n.value)], bool(rc)
