@@ -271,6 +271,36 @@ def test_fp16_prefill_attention(kv, oracle):
     assert rel_err(host(out), want) <= TOL
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("H,Hk,T,pad", [(16, 8, 700, 0), (8, 8, 333, 0), (16, 4, 530, 256), (12, 4, 100, 0), (4, 2, 1, 0),
+                                        (4, 2, 17, 0), (16, 8, 64, 0)])
+def test_fp16_prefill_attention_long(kv, oracle, H, Hk, T, pad, variant):
+    """Causal prefill over the fp16 cache: GQA groups 1, 2 and 4 take the matrix-core kernel (variant 0),
+    group 3 and variant 1 the vector-ALU one; block edges (T = 1, 17, 64), a q row stride wider than
+    H*D, outlier keys that move the running maximum late in the row."""
+    import torch
+    r = gen.rng(250 + H + T)
+    msl = T + 5
+    kv_dim, q_dim = Hk * D, H * D + pad
+    ck, cv = build_fp16_cache(r, 1, msl, kv_dim)
+    if T > 40:
+        ck[0, T - 3] = (ck[0, T - 3].astype(np.float32) * 6).astype(np.float16)   # a late, large key
+        ck[0, 35] = (ck[0, 35].astype(np.float32) * 5).astype(np.float16)
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    oracle.gqa_prefill_attention(want, q, ck[0], cv[0], T, msl, H, Hk, D, q_dim, kv_dim)
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * T, dtype=torch.float32, device="cuda")
+    kv.set_attention_variant(variant)
+    try:
+        kv.launch_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), scratch, T, msl, H, Hk, D, q_dim, kv_dim)
+    finally:
+        kv.set_attention_variant(0)
+    got = host(out)
+    assert rel_err(got[:, :H * D], want[:, :H * D]) <= TOL
+    assert not got[:, H * D:].any()
+
+
 # ------------------------------------------------------------------ compressed attention
 @pytest.mark.parametrize("variant", [1, 0])
 @pytest.mark.parametrize("bits", [4, 2])

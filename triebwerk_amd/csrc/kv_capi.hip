@@ -140,6 +140,13 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done =
             g_prof.created++;
         }
     }
+    if (a.bits == 0 && g_variant.load() != 1 && prefill_f16_mfma_usable(a)) {   // fp16 prefill: one MFMA kernel, no splits
+        if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
+        launch_prefill_f16_mfma(a, s);
+        if (prof) hipEventRecord(g_prof.stop[g_prof.used++], s);
+        check_launch(fn);
+        return;
+    }
     const bool mfma = mfma_wanted(a) && prepare_attention_mfma(a, s, !query_done);
     if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
     if (mfma) launch_attention_mfma_scan(a, s);

@@ -144,6 +144,9 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);
 // causal prefill with blocks of query tokens per wave (kv_prefill_mfma.hip); same workspace and merge
 bool prefill_mfma_usable(const AttnArgs& a);
 void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s);
+// causal prefill over the fp16 cache on the matrix cores (kv_prefill_f16_mfma.hip); writes `out` directly
+bool prefill_f16_mfma_usable(const AttnArgs& a);
+void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s);
 // 2-bit decode scan for 8 KV heads whose waves load whole cache rows together (kv_attention_mfma2c.hip)
 bool attention_mfma2c_usable(const AttnArgs& a);
 void launch_attention_mfma2c_scan(const AttnArgs& a, hipStream_t s);

@@ -1,0 +1,218 @@
+// kv_prefill_f16_mfma.hip -- causal prefill attention over the fp16 cache on the matrix cores (gfx950).
+//
+// Replaces gqa_prefill_attention_kernel (kernels.cu:1071-1158): query token t of every head attends
+// cache rows 0..t of its KV head, out = softmax(q.K^T / sqrt(128)) V with the reference's
+// `+ 1e-8` in the normalisation.  This is the one GEMM-shaped piece of the path, so both
+// contractions run as v_mfma_f32_16x16x32_f16 with fp32 accumulation:
+//
+//   S^T[kv token][query] = K . Q^T   A = K rows from LDS, B = Q rows (registers, loaded once)
+//   O[query][dim]       += P . V     A = P (the lane's own S^T values, no transposition),
+//                                    B = V^T from LDS
+//
+// Computing S transposed leaves lane (query n, kg) with the scores of kv tokens 4kg..4kg+3 of both
+// 16-token halves of a tile: exactly the 8 contraction slots the A operand of the second MFMA
+// wants from that lane, once V^T is stored with its 32 token columns in the matching order
+// (slot 8kg + 4s + i <-> token 16s + 4kg + i).  Softmax is online, base 2, with the running
+// maximum raised only when a score exceeds it by 2^5 (then the accumulators are rescaled), so in
+// the steady state a tile costs 16 MFMAs, 8 exponentials per lane and no shuffles.
+//
+// A workgroup of 4 waves takes one KV head and 64 / R query tokens (R = GQA group: wave w serves
+// query head w % R, token sub-block w / R), walks the kv tiles of 32 tokens up to its diagonal and
+// shares each tile through LDS: K row-major (padded rows), V transposed on the way in (each
+// thread interleaves the same 8 dims of two consecutive tokens and writes 8 dwords).  Tiles are
+// double-buffered: the next tile's global loads are issued before the arithmetic and stored to
+// LDS after it, one barrier per tile.  Blocks are launched longest first.
+
+#include "kv_common.hpp"
+#include "kv_kernels.hpp"
+#include "kv_mfma_util.hpp"
+
+namespace twkv {
+
+namespace {
+
+constexpr int kPfWaves = 4;
+constexpr int kPfKRow = 2 * kHeadDim + 16;   // bytes per K row in LDS
+constexpr int kPfVRow = 2 * 32 + 16;         // bytes per V^T row (32 token slots) in LDS
+
+// column of a tile's token in the V^T rows: the contraction slot order of the second MFMA
+__device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 2) + 4 * (token >> 4) + (token & 3); }
+
+}  // namespace
+
+template <int R>
+__global__ void __launch_bounds__(kPfWaves* kWave)
+prefill_f16_mfma_kernel(AttnArgs a, int T) {
+    constexpr int TPW = 16 * kPfWaves / R;                 // query tokens per workgroup
+    __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPfKRow];
+    __shared__ __attribute__((aligned(16))) char v_s[2][kHeadDim * kPfVRow];
+
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid / kWave), lane = tid % kWave;
+    const int ln = lane & 15, kg = lane >> 4;
+    const int nblk = (T + TPW - 1) / TPW;
+    const int tb = nblk - 1 - (int)blockIdx.x;             // longest blocks first
+    const int kvh = blockIdx.y;
+    const int head = kvh * R + wave % R;
+    const int q0 = tb * TPW + 16 * (wave / R);             // this wave's 16 query tokens
+    const int tq = q0 + ln;                                // this lane's query (as a column of S^T)
+    const int wg_last = min(T, (tb + 1) * TPW) - 1;        // last query token of the workgroup
+    const int ntiles = (wg_last >> 5) + 1;
+    const int kv_dim = a.num_kv_heads * kHeadDim;
+    const half_t* kbase = reinterpret_cast<const half_t*>(a.k) + (long long)kvh * kHeadDim;
+    const half_t* vbase = reinterpret_cast<const half_t*>(a.v) + (long long)kvh * kHeadDim;
+
+    // ---- B operand of the first MFMA: Q[tq][32j + 8kg .. +7], j = 0..3
+    half8_t qb[4];
+    {
+        const half_t* qrow = a.q + (long long)min(tq, T - 1) * a.q_stride + (long long)head * kHeadDim + 8 * kg;
+#pragma unroll
+        for (int j = 0; j < 4; j++) qb[j] = *reinterpret_cast<const half8_t*>(qrow + 32 * j);
+    }
+
+    // ---- staging of a tile: thread (r = tid / 16, c = tid % 16) carries 16 bytes (dims 8c..8c+7) of
+    // K rows r and r + 16, and of V rows 2r and 2r + 1 (two consecutive tokens, interleaved on the way
+    // into the transposed tile).  Rows past the last token are clamped (they are masked anyway).
+    const int sr = tid >> 4, sc = tid & 15;
+    auto load_tile = [&](int tile, uint4 (&kr)[2], uint4 (&vr)[2]) {
+        const int last = T - 1;
+        const long long k0 = (long long)min(tile + sr, last) * kv_dim, k1 = (long long)min(tile + sr + 16, last) * kv_dim;
+        const long long v0 = (long long)min(tile + 2 * sr, last) * kv_dim, v1 = (long long)min(tile + 2 * sr + 1, last) * kv_dim;
+        kr[0] = *reinterpret_cast<const uint4*>(kbase + k0 + 8 * sc);
+        kr[1] = *reinterpret_cast<const uint4*>(kbase + k1 + 8 * sc);
+        vr[0] = *reinterpret_cast<const uint4*>(vbase + v0 + 8 * sc);
+        vr[1] = *reinterpret_cast<const uint4*>(vbase + v1 + 8 * sc);
+    };
+    const int vcol = 2 * vt_slot(2 * sr);                  // byte column of the token pair in a V^T row
+    auto stash = [&](int buf, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
+        *reinterpret_cast<uint4*>(&k_s[buf][sr * kPfKRow + 16 * sc]) = kr[0];
+        *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPfKRow + 16 * sc]) = kr[1];
+        const uint32_t va[4] = {vr[0].x, vr[0].y, vr[0].z, vr[0].w};
+        const uint32_t vb[4] = {vr[1].x, vr[1].y, vr[1].z, vr[1].w};
+        char* dst = &v_s[buf][(8 * sc) * kPfVRow + vcol];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
+            *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPfVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
+            *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kPfVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x07060302u);
+        }
+    };
+
+    float4_t o[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = kNegBig, l_run = 0.0f;
+    const float scale2 = kLog2e * kInvSqrtD;
+    constexpr float kRaise = 5.0f;
+
+    uint4 kr[2], vr[2];
+    load_tile(0, kr, vr);
+    stash(0, kr, vr);
+    __syncthreads();
+
+    for (int it = 0; it < ntiles; it++) {
+        const int buf = it & 1;
+        const int tile = 32 * it;
+        const bool more = it + 1 < ntiles;
+        if (more) load_tile(tile + 32, kr, vr);
+
+        if (tile <= q0 + 15 && q0 < T) {                   // the tile reaches this wave's queries (uniform over the wave)
+            // ---- S^T[kv][query] for both 16-token halves
+            float4_t s[2];
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+                const char* krow = &k_s[buf][(16 * sub + ln) * kPfKRow + 16 * kg];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const half8_t ka = *reinterpret_cast<const half8_t*>(krow + 64 * j);
+                    s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[j], s[sub], 0, 0, 0);
+                }
+            }
+            // ---- online softmax for query tq: this lane holds kv tokens tile + 16 sub + 4kg + i
+            float x[8];
+            float mx = kNegBig;
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const bool valid = tile + 16 * sub + 4 * kg + i <= tq;
+                    x[4 * sub + i] = valid ? s[sub][i] * scale2 : kNegBig;
+                    mx = fmaxf(mx, x[4 * sub + i]);
+                }
+            }
+            if (__any(mx > m_run + kRaise)) {              // rare after the first tiles
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {              // accumulator register i belongs to query 4kg + i
+                    const float ai = __shfl(alpha, 4 * kg + i, 64);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) o[j][i] *= ai;
+                }
+            }
+            half8_t pa;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float p = __builtin_amdgcn_exp2f(x[i] - m_run);
+                l_run += p;
+                pa[i] = (half_t)p;
+            }
+            // ---- O[query][dim 16j + ln] += P . V
+            const char* vrow = &v_s[buf][ln * kPfVRow + 16 * kg];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
+                o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, o[j], 0, 0, 0);
+            }
+        }
+
+        if (more) stash(buf ^ 1, kr, vr);
+        __syncthreads();
+    }
+
+    // ---- normalise (kernels.cu:1146: 1 / (sum + 1e-8)) and store; accumulator register i is query 4kg + i
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / (l_run + 1e-8f);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float inv_i = __shfl(inv, 4 * kg + i, 64);
+        const int t = q0 + 4 * kg + i;
+        if (t < T) {
+            const long long col = (long long)head * kHeadDim + ln;
+            half_t* orow = a.out + (long long)t * a.q_stride + col;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                half_t h = (half_t)(o[j][i] * inv_i);
+                if (a.gate) h = gated(h, a.gate[(long long)t * a.gate_stride + col + 16 * j]);
+                orow[16 * j] = h;
+            }
+        }
+    }
+}
+
+// fp16 cache, one sequence, query t attends rows 0..t, GQA group 1, 2 or 4, 16-byte aligned rows
+bool prefill_f16_mfma_usable(const AttnArgs& a) {
+    const int R = a.num_heads / a.num_kv_heads;
+    if (a.bits != 0 || a.pos_mode != kPosIota || a.block_table || a.seq_stride_rows != 0) return false;
+    if (R != 1 && R != 2 && R != 4) return false;
+    if ((a.q_stride & 7) != 0) return false;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.k) | reinterpret_cast<uintptr_t>(a.v);
+    return (bits & 15u) == 0 && a.G >= 1;
+}
+
+void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s) {
+    const int R = a.num_heads / a.num_kv_heads;
+    const int T = a.G;
+    const int tpw = 16 * kPfWaves / R;
+    const dim3 grid((T + tpw - 1) / tpw, a.num_kv_heads), block(kPfWaves * kWave);
+    if (R == 1) hipLaunchKernelGGL(prefill_f16_mfma_kernel<1>, grid, block, 0, s, a, T);
+    else if (R == 2) hipLaunchKernelGGL(prefill_f16_mfma_kernel<2>, grid, block, 0, s, a, T);
+    else hipLaunchKernelGGL(prefill_f16_mfma_kernel<4>, grid, block, 0, s, a, T);
+}
+
+}  // namespace twkv
