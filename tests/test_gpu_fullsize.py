@@ -266,3 +266,30 @@ def test_extremely_ragged_batch(kv, oracle, rotation_fixture, bits):
         err = rel_err_rows(host(out), want)
         assert err.max() <= TOL, f"variant {variant}: max rel err {err.max():.3e} (sequence {err.argmax() // H}, length {lens[err.argmax() // H]})"
     kv.set_attention_variant(0)
+
+
+@pytest.mark.parametrize("H,T", [(16, 2500), (16, 5000), (32, 4100)])
+def test_fp16_prefill_long_prompts_kernel_families_agree(kv, H, T):
+    """Prompt lengths at which the matrix-core prefill kernel switches to mirrored block pairs and to two
+    query blocks per wave, against the vector-ALU kernel (which the small cases pin to the oracle):
+    both within the attention tolerance of each other, row by row."""
+    import torch
+    Hk = 8
+    kv_dim, q_dim = Hk * D, H * D
+    g_ = torch.Generator(device="cuda"); g_.manual_seed(990 + T)
+    q = torch.randn((T, q_dim), generator=g_, device="cuda").to(torch.float16)
+    ck = torch.randn((T, kv_dim), generator=g_, device="cuda").to(torch.float16)
+    cv = torch.randn((T, kv_dim), generator=g_, device="cuda").to(torch.float16)
+    ck[T - 2] *= 5
+    scratch = torch.zeros(H * T * 1024, dtype=torch.float32, device="cuda")
+    outs = []
+    for variant in (0, 1):
+        kv.set_attention_variant(variant)
+        try:
+            out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+            kv.launch_gqa_prefill_attention(out, q, ck, cv, scratch, T, T, H, Hk, D, q_dim, kv_dim)
+            outs.append(host(out))
+        finally:
+            kv.set_attention_variant(0)
+    err = rel_err_rows(outs[0], outs[1])
+    assert err.max() <= TOL, f"max rel err {err.max():.3e} at row {err.argmax() // H}"

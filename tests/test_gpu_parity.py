@@ -301,6 +301,30 @@ def test_fp16_prefill_attention_long(kv, oracle, H, Hk, T, pad, variant):
     assert not got[:, H * D:].any()
 
 
+@pytest.mark.parametrize("form", [1, 2, 3])
+@pytest.mark.parametrize("H,Hk,T", [(16, 8, 300), (8, 8, 129), (16, 4, 97), (16, 8, 31)])
+def test_fp16_prefill_every_form_of_the_mfma_kernel(kv, oracle, H, Hk, T, form):
+    """The matrix-core prefill kernel picks one of three forms from the prompt length (one or two query
+    blocks per wave, with or without mirrored block pairs); each is forced here at lengths that put
+    the diagonal, the middle block of an odd count and a ragged last block in different places."""
+    import torch
+    r = gen.rng(270 + H + T)
+    msl = T
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv = build_fp16_cache(r, 1, msl, kv_dim)
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    oracle.gqa_prefill_attention(want, q, ck[0], cv[0], T, msl, H, Hk, D, q_dim, kv_dim)
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * T, dtype=torch.float32, device="cuda")
+    kv.set_prefill_form(form)
+    try:
+        kv.launch_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), scratch, T, msl, H, Hk, D, q_dim, kv_dim)
+    finally:
+        kv.set_prefill_form(0)
+    assert rel_err(host(out), want) <= TOL
+
+
 # ------------------------------------------------------------------ compressed attention
 @pytest.mark.parametrize("variant", [1, 0])
 @pytest.mark.parametrize("bits", [4, 2])

@@ -60,6 +60,7 @@ SIGNATURES = {
     "tw_kv_set_attention_variant": (None, [I]),
     "tw_kv_get_attention_variant": (I, []),
     "tw_kv_set_num_splits": (None, [I]),
+    "tw_kv_set_prefill_form": (None, [I]),
     "tw_kv_profile_attention": (None, [I]),
     "tw_kv_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_kv_measure_read_bandwidth": (C.c_double, [P, C.c_size_t, I, P]),

@@ -129,6 +129,7 @@ struct Profiler {
 
 // query_done: q_rot is already in the workspace (the fused append + attention entry
 // rotates the query together with the appended rows).
+std::atomic<int> g_prefill_form{0};   // test hook: forces a form of the fp16 MFMA prefill kernel
 bool mfma_wanted(const AttnArgs& a) { return a.bits != 0 && g_variant.load() != 1; }
 
 void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done = false) {
@@ -142,7 +143,7 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done =
     }
     if (a.bits == 0 && g_variant.load() != 1 && prefill_f16_mfma_usable(a)) {   // fp16 prefill: one MFMA kernel, no splits
         if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
-        launch_prefill_f16_mfma(a, s);
+        launch_prefill_f16_mfma(a, s, g_prefill_form.load());
         if (prof) hipEventRecord(g_prof.stop[g_prof.used++], s);
         check_launch(fn);
         return;
@@ -175,6 +176,7 @@ const char* tw_kv_build_info(void) { return "triebwerk_kv gfx950 " __DATE__ " " 
 void tw_kv_set_attention_variant(int v) { g_variant.store(v); }
 int tw_kv_get_attention_variant(void) { return g_variant.load(); }
 void tw_kv_set_num_splits(int n) { g_nsplit_override.store(n); }
+void tw_kv_set_prefill_form(int form) { g_prefill_form.store(form); }
 
 void tw_kv_profile_attention(int enable) {
     g_prof.enabled.store(enable);

@@ -146,7 +146,9 @@ bool prefill_mfma_usable(const AttnArgs& a);
 void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s);
 // causal prefill over the fp16 cache on the matrix cores (kv_prefill_f16_mfma.hip); writes `out` directly
 bool prefill_f16_mfma_usable(const AttnArgs& a);
-void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s);
+// form: 0 = chosen from the prompt length; 1 one query block per wave, 2 the same with mirrored block pairs,
+// 3 two query blocks per wave with mirrored pairs
+void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form);
 // 2-bit decode scan for 8 KV heads whose waves load whole cache rows together (kv_attention_mfma2c.hip)
 bool attention_mfma2c_usable(const AttnArgs& a);
 void launch_attention_mfma2c_scan(const AttnArgs& a, hipStream_t s);

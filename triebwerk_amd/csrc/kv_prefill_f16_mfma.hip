@@ -16,16 +16,20 @@
 // maximum raised only when a score exceeds it by 2^5 (then the accumulators are rescaled), so in
 // the steady state a tile costs 16 MFMAs, 8 exponentials per lane and no shuffles.
 //
-// A workgroup of 4 waves takes one KV head and 64 / R query tokens (R = GQA group: wave w serves
-// query head w % R, token sub-block w / R), walks the kv tiles of 32 tokens up to its diagonal and
-// shares each tile through LDS: K row-major (padded rows), V transposed on the way in (each
-// thread interleaves the same 8 dims of two consecutive tokens and writes 8 dwords).  Tiles are
-// double-buffered: the next tile's global loads are issued before the arithmetic and stored to
-// LDS after it, one barrier per tile.  Blocks are launched longest first.
+// A workgroup of 4 waves takes one KV head and 64 NQ / R query tokens (R = GQA group: wave w serves
+// query head w % R and 16 NQ tokens; with NQ = 2 the two 16-row blocks share every operand read),
+// walks the kv tiles of 32 tokens up to its diagonal and shares each tile through LDS: K row-major
+// (padded rows), V transposed on the way in (each thread interleaves the same 8 dims of two
+// consecutive tokens and writes 8 dwords).  Tiles are double-buffered: the next tile's global loads
+// are issued before the arithmetic and stored to LDS after it, one barrier per tile.  For long
+// prompts a workgroup does a token block and then its mirror image from the other end of the
+// sequence, so causal rows cost every workgroup the same; short prompts take one block each, longest
+// first.
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 #include "kv_mfma_util.hpp"
+
 
 namespace twkv {
 
@@ -40,10 +44,12 @@ __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 
 
 }  // namespace
 
-template <int R>
+// NQ: 16-row query blocks per wave (every K and V operand read feeds NQ MFMAs).  MIRROR: a workgroup does a
+// token block and then its mirror image from the other end of the sequence.
+template <int R, int NQ, bool MIRROR>
 __global__ void __launch_bounds__(kPfWaves* kWave)
 prefill_f16_mfma_kernel(AttnArgs a, int T) {
-    constexpr int TPW = 16 * kPfWaves / R;                 // query tokens per workgroup
+    constexpr int TPW = 16 * NQ * kPfWaves / R;            // query tokens per workgroup pass
     __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPfKRow];
     __shared__ __attribute__((aligned(16))) char v_s[2][kHeadDim * kPfVRow];
 
@@ -51,24 +57,13 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
     const int wave = uniform(tid / kWave), lane = tid % kWave;
     const int ln = lane & 15, kg = lane >> 4;
     const int nblk = (T + TPW - 1) / TPW;
-    const int tb = nblk - 1 - (int)blockIdx.x;             // longest blocks first
     const int kvh = blockIdx.y;
     const int head = kvh * R + wave % R;
-    const int q0 = tb * TPW + 16 * (wave / R);             // this wave's 16 query tokens
-    const int tq = q0 + ln;                                // this lane's query (as a column of S^T)
-    const int wg_last = min(T, (tb + 1) * TPW) - 1;        // last query token of the workgroup
-    const int ntiles = (wg_last >> 5) + 1;
     const int kv_dim = a.num_kv_heads * kHeadDim;
     const half_t* kbase = reinterpret_cast<const half_t*>(a.k) + (long long)kvh * kHeadDim;
     const half_t* vbase = reinterpret_cast<const half_t*>(a.v) + (long long)kvh * kHeadDim;
-
-    // ---- B operand of the first MFMA: Q[tq][32j + 8kg .. +7], j = 0..3
-    half8_t qb[4];
-    {
-        const half_t* qrow = a.q + (long long)min(tq, T - 1) * a.q_stride + (long long)head * kHeadDim + 8 * kg;
-#pragma unroll
-        for (int j = 0; j < 4; j++) qb[j] = *reinterpret_cast<const half8_t*>(qrow + 32 * j);
-    }
+    const float scale2 = kLog2e * kInvSqrtD;
+    constexpr float kRaise = 5.0f;
 
     // ---- staging of a tile: thread (r = tid / 16, c = tid % 16) carries 16 bytes (dims 8c..8c+7) of
     // K rows r and r + 16, and of V rows 2r and 2r + 1 (two consecutive tokens, interleaved on the way
@@ -97,99 +92,132 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
         }
     };
 
-    float4_t o[8];
-#pragma unroll
-    for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float m_run = kNegBig, l_run = 0.0f;
-    const float scale2 = kLog2e * kInvSqrtD;
-    constexpr float kRaise = 5.0f;
+    // A workgroup takes token block blockIdx.x and its mirror image from the other end, one after the
+    // other: with causal rows the two together cost the same for every workgroup.
+    const int first = blockIdx.x, second = nblk - 1 - (int)blockIdx.x;   // without MIRROR: longest blocks first
+    for (int pass = 0; pass < (MIRROR ? 2 : 1); pass++) {
+        if (pass == 1 && second == first) break;           // the middle block of an odd count
+        const int tb = pass == 0 ? second : first;         // the long one first
+        const int q0 = tb * TPW + 16 * NQ * (wave / R);    // this wave's 16 NQ query tokens
+        const int wg_last = min(T, (tb + 1) * TPW) - 1;    // last query token of the pass
+        const int ntiles = (wg_last >> 5) + 1;
 
-    uint4 kr[2], vr[2];
-    load_tile(0, kr, vr);
-    stash(0, kr, vr);
-    __syncthreads();
-
-    for (int it = 0; it < ntiles; it++) {
-        const int buf = it & 1;
-        const int tile = 32 * it;
-        const bool more = it + 1 < ntiles;
-        if (more) load_tile(tile + 32, kr, vr);
-
-        if (tile <= q0 + 15 && q0 < T) {                   // the tile reaches this wave's queries (uniform over the wave)
-            // ---- S^T[kv][query] for both 16-token halves
-            float4_t s[2];
+        // ---- B operands of the first MFMA: Q[q0 + 16 nq + ln][32j + 8kg .. +7], j = 0..3
+        half8_t qb[NQ][4];
 #pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
-                s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
-                const char* krow = &k_s[buf][(16 * sub + ln) * kPfKRow + 16 * kg];
+        for (int nq = 0; nq < NQ; nq++) {
+            const half_t* qrow = a.q + (long long)min(q0 + 16 * nq + ln, T - 1) * a.q_stride + (long long)head * kHeadDim + 8 * kg;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const half8_t ka = *reinterpret_cast<const half8_t*>(krow + 64 * j);
-                    s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[j], s[sub], 0, 0, 0);
-                }
-            }
-            // ---- online softmax for query tq: this lane holds kv tokens tile + 16 sub + 4kg + i
-            float x[8];
-            float mx = kNegBig;
+            for (int j = 0; j < 4; j++) qb[nq][j] = *reinterpret_cast<const half8_t*>(qrow + 32 * j);
+        }
+        float4_t o[NQ][8];
+        float m_run[NQ], l_run[NQ];
 #pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
+        for (int nq = 0; nq < NQ; nq++) {
+            m_run[nq] = kNegBig; l_run[nq] = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const bool valid = tile + 16 * sub + 4 * kg + i <= tq;
-                    x[4 * sub + i] = valid ? s[sub][i] * scale2 : kNegBig;
-                    mx = fmaxf(mx, x[4 * sub + i]);
-                }
-            }
-            if (__any(mx > m_run + kRaise)) {              // rare after the first tiles
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
-                const float m_new = fmaxf(m_run, mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                m_run = m_new;
-                l_run *= alpha;
-#pragma unroll
-                for (int i = 0; i < 4; i++) {              // accumulator register i belongs to query 4kg + i
-                    const float ai = __shfl(alpha, 4 * kg + i, 64);
-#pragma unroll
-                    for (int j = 0; j < 8; j++) o[j][i] *= ai;
-                }
-            }
-            half8_t pa;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float p = __builtin_amdgcn_exp2f(x[i] - m_run);
-                l_run += p;
-                pa[i] = (half_t)p;
-            }
-            // ---- O[query][dim 16j + ln] += P . V
-            const char* vrow = &v_s[buf][ln * kPfVRow + 16 * kg];
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
-                o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, o[j], 0, 0, 0);
-            }
+            for (int j = 0; j < 8; j++) o[nq][j] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
 
-        if (more) stash(buf ^ 1, kr, vr);
+        uint4 kr[2], vr[2];
+        load_tile(0, kr, vr);
+        stash(0, kr, vr);
         __syncthreads();
-    }
 
-    // ---- normalise (kernels.cu:1146: 1 / (sum + 1e-8)) and store; accumulator register i is query 4kg + i
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / (l_run + 1e-8f);
+        for (int it = 0; it < ntiles; it++) {
+            const int buf = it & 1;
+            const int tile = 32 * it;
+            const bool more = it + 1 < ntiles;
+            if (more) load_tile(tile + 32, kr, vr);
+
+            if (tile <= q0 + 16 * NQ - 1 && q0 < T) {      // the tile reaches this wave's queries (uniform over the wave)
+                // ---- S^T[kv][query] for both 16-token halves and all query blocks
+                float4_t s[NQ][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float inv_i = __shfl(inv, 4 * kg + i, 64);
-        const int t = q0 + 4 * kg + i;
-        if (t < T) {
-            const long long col = (long long)head * kHeadDim + ln;
-            half_t* orow = a.out + (long long)t * a.q_stride + col;
+                for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                half_t h = (half_t)(o[j][i] * inv_i);
-                if (a.gate) h = gated(h, a.gate[(long long)t * a.gate_stride + col + 16 * j]);
-                orow[16 * j] = h;
+                    for (int nq = 0; nq < NQ; nq++) s[nq][sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+                    const char* krow = &k_s[buf][(16 * sub + ln) * kPfKRow + 16 * kg];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const half8_t ka = *reinterpret_cast<const half8_t*>(krow + 64 * j);
+#pragma unroll
+                        for (int nq = 0; nq < NQ; nq++)
+                            s[nq][sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[nq][j], s[nq][sub], 0, 0, 0);
+                    }
+                }
+                // ---- online softmax per query: this lane holds kv tokens tile + 16 sub + 4kg + i
+                half8_t pa[NQ];
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) {
+                    const int tq = q0 + 16 * nq + ln;
+                    float x[8];
+                    float mx = kNegBig;
+#pragma unroll
+                    for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const bool valid = tile + 16 * sub + 4 * kg + i <= tq;
+                            x[4 * sub + i] = valid ? s[nq][sub][i] * scale2 : kNegBig;
+                            mx = fmaxf(mx, x[4 * sub + i]);
+                        }
+                    }
+                    if (__any(mx > m_run[nq] + kRaise)) {  // rare after the first tiles
+                        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
+                        const float m_new = fmaxf(m_run[nq], mx);
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[nq] - m_new);
+                        m_run[nq] = m_new;
+                        l_run[nq] *= alpha;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {      // accumulator register i belongs to query 4kg + i
+                            const float ai = __shfl(alpha, 4 * kg + i, 64);
+#pragma unroll
+                            for (int j = 0; j < 8; j++) o[nq][j][i] *= ai;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float p = __builtin_amdgcn_exp2f(x[i] - m_run[nq]);
+                        l_run[nq] += p;
+                        pa[nq][i] = (half_t)p;
+                    }
+                }
+                // ---- O[query][dim 16j + ln] += P . V
+                const char* vrow = &v_s[buf][ln * kPfVRow + 16 * kg];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
+#pragma unroll
+                    for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
+                }
+            }
+
+            if (more) stash(buf ^ 1, kr, vr);
+            __syncthreads();
+        }
+
+        // ---- normalise (kernels.cu:1146: 1 / (sum + 1e-8)) and store; accumulator register i is query 4kg + i
+#pragma unroll
+        for (int nq = 0; nq < NQ; nq++) {
+            float l = l_run[nq];
+            l += __shfl_xor(l, 16, 64);
+            l += __shfl_xor(l, 32, 64);
+            const float inv = 1.0f / (l + 1e-8f);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float inv_i = __shfl(inv, 4 * kg + i, 64);
+                const int t = q0 + 16 * nq + 4 * kg + i;
+                if (t < T) {
+                    const long long col = (long long)head * kHeadDim + ln;
+                    half_t* orow = a.out + (long long)t * a.q_stride + col;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        half_t h = (half_t)(o[nq][j][i] * inv_i);
+                        if (a.gate) h = gated(h, a.gate[(long long)t * a.gate_stride + col + 16 * j]);
+                        orow[16 * j] = h;
+                    }
+                }
             }
         }
     }
@@ -205,14 +233,32 @@ bool prefill_f16_mfma_usable(const AttnArgs& a) {
     return (bits & 15u) == 0 && a.G >= 1;
 }
 
-void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s) {
+void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form) {
     const int R = a.num_heads / a.num_kv_heads;
     const int T = a.G;
-    const int tpw = 16 * kPfWaves / R;
-    const dim3 grid((T + tpw - 1) / tpw, a.num_kv_heads), block(kPfWaves * kWave);
-    if (R == 1) hipLaunchKernelGGL(prefill_f16_mfma_kernel<1>, grid, block, 0, s, a, T);
-    else if (R == 2) hipLaunchKernelGGL(prefill_f16_mfma_kernel<2>, grid, block, 0, s, a, T);
-    else hipLaunchKernelGGL(prefill_f16_mfma_kernel<4>, grid, block, 0, s, a, T);
+    // Long prompts: two query blocks per wave and mirrored block pairs (operand reuse, equal work per
+    // workgroup).  Short ones do not fill the GPU that way and take smaller, then unpaired workgroups
+    // (measured at 16 and 32 heads over 8 KV heads: each form wins from one workgroup per CU upwards).
+    const int cus = compute_units();
+    int mode = 1;
+    {
+        const int nblk2 = (T + 32 * kPfWaves / R - 1) / (32 * kPfWaves / R), nblk1 = (T + 16 * kPfWaves / R - 1) / (16 * kPfWaves / R);
+        if ((nblk2 + 1) / 2 * a.num_kv_heads >= cus) mode = 3;
+        else if ((nblk1 + 1) / 2 * a.num_kv_heads >= cus) mode = 2;
+    }
+    if (form >= 1 && form <= 3) mode = form;               // forced by a test
+    const int nq = mode >= 3 ? 2 : 1;
+    const bool mirror = mode == 2 || mode == 3;
+    const int tpw = 16 * nq * kPfWaves / R;
+    const int nblk = (T + tpw - 1) / tpw;
+    const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(kPfWaves * kWave);
+#define TW_PF_LAUNCH(RR, NN, MM) hipLaunchKernelGGL((prefill_f16_mfma_kernel<RR, NN, MM>), grid, block, 0, s, a, T)
+#define TW_PF_MODES(RR) \
+    do { if (mode == 1) TW_PF_LAUNCH(RR, 1, false); else if (mode == 2) TW_PF_LAUNCH(RR, 1, true); \
+         else TW_PF_LAUNCH(RR, 2, true); } while (0)
+    if (R == 1) TW_PF_MODES(1); else if (R == 2) TW_PF_MODES(2); else TW_PF_MODES(4);
+#undef TW_PF_MODES
+#undef TW_PF_LAUNCH
 }
 
 }  // namespace twkv

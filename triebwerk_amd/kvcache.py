@@ -228,6 +228,10 @@ def set_attention_variant(variant: int) -> None:
     _lib.load().tw_kv_set_attention_variant(int(variant))
 
 
+def set_prefill_form(form: int) -> None:
+    _lib.load().tw_kv_set_prefill_form(int(form))
+
+
 def set_num_splits(nsplit: int) -> None:
     _lib.load().tw_kv_set_num_splits(int(nsplit))
 
