@@ -136,6 +136,58 @@ def cpu_baseline(w, kv_bits, seconds_budget=15.0):
                        f"{os.cpu_count()} logical CPUs visible")
 
 
+def prefill_bench(args):
+    """Causal prefill attention of one sequence, one layer: ms per launch and the matrix-core rate.
+    FLOPs counted: 4 * head_dim per (query head, query token, attended token), causal half only."""
+    import torch
+    from triebwerk_amd import kvcache
+    w = WORKLOADS[args.workload]
+    kv_bits = w["kv_bits"] if args.kv_bits is None else args.kv_bits
+    H, Hk, D, T = w["H"], w["Hk"], 128, args.prefill
+    kvcache.set_attention_variant(args.variant)
+    g = torch.Generator(device="cuda"); g.manual_seed(11)
+    q = torch.randn((T, H * D), generator=g, device="cuda", dtype=torch.float16)
+    out = torch.zeros_like(q)
+    ws = torch.zeros(H * T * min(T, 4096), dtype=torch.float32, device="cuda")
+    if kv_bits:
+        kvp = Hk * D * kv_bits // 8
+        ck = torch.randint(0, 256, (T, kvp), generator=g, device="cuda", dtype=torch.uint8)
+        cv = torch.randint(0, 256, (T, kvp), generator=g, device="cuda", dtype=torch.uint8)
+        kn = (11.3 + 0.7 * torch.randn((T, Hk), generator=g, device="cuda")).to(torch.float16)
+        vn = (11.3 + 0.7 * torch.randn((T, Hk), generator=g, device="cuda")).to(torch.float16)
+        rot = kvcache.make_rotation().cuda()
+
+        def launch():
+            kvcache.launch_turbo_gqa_prefill_attention(out, q, ck, cv, kn, vn, rot, ws, T, T, H, Hk, D, H * D, Hk * D, kv_bits)
+    else:
+        ck = torch.randn((T, Hk * D), generator=g, device="cuda", dtype=torch.float16)
+        cv = torch.randn((T, Hk * D), generator=g, device="cuda", dtype=torch.float16)
+
+        def launch():
+            kvcache.launch_gqa_prefill_attention(out, q, ck, cv, ws, T, T, H, Hk, D, H * D, Hk * D)
+    for _ in range(max(args.warmup, 1)):
+        launch()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        launch()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    flop = 4.0 * D * H * T * (T + 1) / 2
+    tflops = flop / (ms * 1e-3) * 1e-12
+    print(json.dumps({
+        "metric": "prefill-attn prompt tokens/s (one layer)", "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": max(args.warmup, 1), "ms_per_step": ms, "higher_is_better": True,
+        "dtype": "f32 accumulate over f16" if not kv_bits else "f32 accumulate over u8 codes + f16 norms", "data": "synthetic",
+        "config": {"workload": f"causal prefill attention, one sequence, {T} tokens, {H} heads over {Hk} KV heads",
+                   "kv_bits": kv_bits if kv_bits else 16, "variant": args.variant},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s", "frac": tflops / 2500.0,
+                     "flops_per_launch": flop, "traffic": None},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -156,7 +208,13 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device-to-device copy of this many MiB five times (reference for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--prefill", type=int, default=0, metavar="T",
+                    help="instead of the decode step, time causal prefill attention over a T-token prompt of one "
+                         "sequence (one layer's launch, the workload's head counts, --kv-bits cache) and exit")
     args = ap.parse_args()
+    if args.prefill:
+        prefill_bench(args)
+        return
     if args.copy_calibration:
         import torch
         n = args.copy_calibration << 20
