@@ -333,8 +333,9 @@ def main():
     step_bytes = algorithmic_bytes(n_tokens_timed, G * K, L, H, Hk, kv_bits, with_append=True) / K
     step_gbs = step_bytes / (elapsed / K) * 1e-9
 
-    # ---- dominant kernel alone: HIP events on the launch stream around the context-scanning kernel
-    # (eager steps that continue the same decode; the library holds 4096 event pairs)
+    # ---- dominant kernel alone: a pair of HIP events attached to every launch of the context-scanning
+    # kernel on its stream (hipExtLaunchKernelGGL: start = the kernel begins, stop = it ends), in eager
+    # steps that continue the same decode; the library holds 4096 event pairs
     Kp = max(1, min(K, 4096 // L))
     lib.tw_kv_profile_attention(1)
     with torch.cuda.stream(stream):

@@ -296,9 +296,9 @@ static void launch_valu_mode(const AttnArgs& a, hipStream_t s) {
     const int rt = (group % 4 == 0) ? 4 : (group % 2 == 0) ? 2 : 1;
     dim3 grid(a.nsplit, a.num_kv_heads * (group / rt), a.G);
     dim3 block(kAttnThreads);
-    if (rt == 4) hipLaunchKernelGGL((attention_valu_kernel<MODE, 4>), grid, block, 0, s, a);
-    else if (rt == 2) hipLaunchKernelGGL((attention_valu_kernel<MODE, 2>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((attention_valu_kernel<MODE, 1>), grid, block, 0, s, a);
+    if (rt == 4) launch_scan_kernel(attention_valu_kernel<MODE, 4>, grid, block, s, a);
+    else if (rt == 2) launch_scan_kernel(attention_valu_kernel<MODE, 2>, grid, block, s, a);
+    else launch_scan_kernel(attention_valu_kernel<MODE, 1>, grid, block, s, a);
 }
 
 void launch_attention_valu(const AttnArgs& a, hipStream_t s) {

@@ -16,6 +16,11 @@
 
 using namespace twkv;
 
+namespace twkv {
+thread_local hipEvent_t t_scan_start = nullptr;
+thread_local hipEvent_t t_scan_stop = nullptr;
+}  // namespace twkv
+
 // ---------------------------------------------------------------- error state
 namespace {
 thread_local int g_err = 0;
@@ -141,18 +146,18 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done =
             g_prof.created++;
         }
     }
+    // the scan kernel carries the profiler's events itself (see launch_scan_kernel)
+    if (prof) { t_scan_start = g_prof.start[g_prof.used]; t_scan_stop = g_prof.stop[g_prof.used]; g_prof.used++; }
     if (a.bits == 0 && g_variant.load() != 1 && prefill_f16_mfma_usable(a)) {   // fp16 prefill: one MFMA kernel, no splits
-        if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
         launch_prefill_f16_mfma(a, s, g_prefill_form.load());
-        if (prof) hipEventRecord(g_prof.stop[g_prof.used++], s);
+        t_scan_start = t_scan_stop = nullptr;
         check_launch(fn);
         return;
     }
-    const bool mfma = mfma_wanted(a) && prepare_attention_mfma(a, s, !query_done);
-    if (prof) hipEventRecord(g_prof.start[g_prof.used], s);
+    const bool mfma = mfma_wanted(a) && prepare_attention_mfma(a, s, !query_done);   // (its query rotation is not a scan launch)
     if (mfma) launch_attention_mfma_scan(a, s);
     else launch_attention_valu(a, s);
-    if (prof) hipEventRecord(g_prof.stop[g_prof.used++], s);
+    t_scan_start = t_scan_stop = nullptr;
     if (a.nsplit > 1 || a.force_merge) {
         if (!(g_variant.load() != 1 && launch_merge_rotate(a, s))) launch_attention_merge(a, s);
     }

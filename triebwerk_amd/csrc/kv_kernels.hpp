@@ -3,11 +3,24 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "kv_common.hpp"
 
 namespace twkv {
+
+// ---------------------------------------------------------------- timing the context-scanning kernel
+// When the profiler is on, kv_capi.hip hands the scan launch a pair of events; the launch attaches them
+// to the kernel itself (start = the kernel begins, stop = it ends), so their distance is the kernel's
+// duration without the gaps an event recorded before and after a launch would add.
+extern thread_local hipEvent_t t_scan_start;
+extern thread_local hipEvent_t t_scan_stop;
+template <typename... Args, typename F = void (*)(Args...)>
+inline void launch_scan_kernel(F kernel, dim3 grid, dim3 block, hipStream_t s, Args... args) {
+    if (t_scan_start) hipExtLaunchKernelGGL(kernel, grid, block, 0, s, t_scan_start, t_scan_stop, 0, args...);
+    else hipLaunchKernelGGL(kernel, grid, block, 0, s, args...);
+}
 
 // ---------------------------------------------------------------- append
 struct QuantArgs {
