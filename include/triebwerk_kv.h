@@ -163,9 +163,9 @@ int tw_kv_get_attention_variant(void);
 
 /* Split count override for decode attention (0 = automatic). */
 void tw_kv_set_num_splits(int nsplit);
-/* Test hook: force a form of the fp16 matrix-core prefill kernel (0 = choose from the prompt length,
+/* Test hook: force a form of the matrix-core prefill kernels (0 = choose from the prompt length,
  * 1 = one 16-row query block per wave, 2 = the same with mirrored block pairs, 3 = two query blocks
- * per wave with mirrored pairs). */
+ * per wave with mirrored pairs, 4 = compressed cache only: the kernel that expands tiles per wave). */
 void tw_kv_set_prefill_form(int form);
 
 /* Timing of the context-scanning attention kernel alone, with HIP events

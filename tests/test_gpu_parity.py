@@ -465,6 +465,31 @@ def test_turbo_prefill_attention_long(kv, oracle, rotation_fixture, bits, H, Hk,
     kv.set_attention_variant(0)
 
 
+@pytest.mark.parametrize("form", [1, 2, 3, 4])
+@pytest.mark.parametrize("bits,H,Hk,T", [(4, 16, 8, 300), (2, 8, 8, 129), (4, 16, 4, 97), (2, 16, 8, 31)])
+def test_turbo_prefill_every_form(kv, oracle, rotation_fixture, bits, H, Hk, T, form):
+    """Compressed prefill: the three forms of the kernel that expands a tile once per workgroup and (form 4)
+    the kernel that expands per wave, each against the oracle."""
+    import torch
+    r = gen.rng(380 + bits + H + T)
+    msl = T + 3
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, 1, Hk, msl, [T], bits)
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    oracle.turbo_gqa_prefill_attention(want, q, ck[0], cv[0], kn[0], vn[0], rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * max(T, 1024), dtype=torch.float32, device="cuda")
+    kv.set_prefill_form(form)
+    try:
+        kv.launch_turbo_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), dev(kn[0]), dev(vn[0]),
+                                              dev(rotation_fixture), scratch, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+    finally:
+        kv.set_prefill_form(0)
+    err = rel_err(host(out), want)
+    assert err <= TOL, err
+
+
 @pytest.mark.parametrize("bits", [4, 2])
 def test_golden_case_on_gpu(kv, rotation_fixture, bits):
     """Committed vectors: append 37 tokens on the GPU, compare every byte, then attention."""

@@ -27,6 +27,7 @@ SOURCES = [
     "kv_attention_mfma2c.hip",
     "kv_prefill_mfma.hip",
     "kv_prefill_f16_mfma.hip",
+    "kv_prefill_tq_mfma.hip",
     "kv_producer.hip",
     "kv_rotate.hip",
     "kv_capi.hip",

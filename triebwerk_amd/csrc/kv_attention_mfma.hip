@@ -662,6 +662,10 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
 }
 
 void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
+    if (prefill_tq_mfma_usable(a) && !(prefill_form() == 4 && prefill_mfma_usable(a))) {
+        launch_prefill_tq_mfma(a, s, prefill_form());
+        return;
+    }
     if (prefill_mfma_usable(a)) {
         launch_prefill_mfma_scan(a, s);
         return;

@@ -17,6 +17,8 @@
 using namespace twkv;
 
 namespace twkv {
+static std::atomic<int> g_prefill_form{0};   // test hook, see prefill_form()
+int prefill_form() { return g_prefill_form.load(); }
 thread_local hipEvent_t t_scan_start = nullptr;
 thread_local hipEvent_t t_scan_stop = nullptr;
 }  // namespace twkv
@@ -134,11 +136,14 @@ struct Profiler {
 
 // query_done: q_rot is already in the workspace (the fused append + attention entry
 // rotates the query together with the appended rows).
-std::atomic<int> g_prefill_form{0};   // test hook: forces a form of the fp16 MFMA prefill kernel
 bool mfma_wanted(const AttnArgs& a) { return a.bits != 0 && g_variant.load() != 1; }
 
 void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done = false) {
     bool prof = g_prof.enabled.load() != 0 && g_prof.used < kProfSlots;
+    if (prof) {   // events cannot ride on a launch that is only being recorded into a graph
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone) prof = false;
+    }
     if (prof) {
         while (g_prof.created <= g_prof.used) {
             if (hipEventCreate(&g_prof.start[g_prof.created]) != hipSuccess ||

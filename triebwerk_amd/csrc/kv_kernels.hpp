@@ -84,7 +84,8 @@ struct RotArgs {
     long long seg_stride[3];     // halves per source row
     int seg_heads[3];            // head vectors per source row
     int seg_nvec[3];             // rows * heads
-    int seg_units[3];            // work units = ceil(nvec / 16) * 8
+    int seg_units[3];            // work units = ceil(tiles / nper) * 8 (launch_rotate fills this in)
+    int nper;                    // tiles of 16 vectors a wave walks (launch_rotate fills this in)
     int seg_kind[3];             // 0 = quantize into the cache, 1 = query rotation
     uint8_t* seg_codes[3];
     half_t* seg_norms[3];
@@ -162,6 +163,13 @@ bool prefill_f16_mfma_usable(const AttnArgs& a);
 // form: 0 = chosen from the prompt length; 1 one query block per wave, 2 the same with mirrored block pairs,
 // 3 two query blocks per wave with mirrored pairs
 void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form);
+// causal prefill over the compressed cache with tiles expanded once per workgroup (kv_prefill_tq_mfma.hip);
+// same workspace and merge as the scan; form as for launch_prefill_f16_mfma
+bool prefill_tq_mfma_usable(const AttnArgs& a);
+void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form);
+// test hook (tw_kv_set_prefill_form): 0 = automatic; 1-3 force a form of the flash prefill kernels; 4 = the
+// compressed prefill kernel that expands tiles per wave
+int prefill_form();
 // 2-bit decode scan for 8 KV heads whose waves load whole cache rows together (kv_attention_mfma2c.hip)
 bool attention_mfma2c_usable(const AttnArgs& a);
 void launch_attention_mfma2c_scan(const AttnArgs& a, hipStream_t s);

@@ -1,0 +1,324 @@
+// kv_prefill_tq_mfma.hip -- causal prefill attention over the TurboQuant-compressed cache on the matrix cores
+// (gfx950), for prompts: the flash-attention kernel of kv_prefill_f16_mfma.hip (which documents the MFMA
+// tiling, the transposed scores and the softmax) with one difference: a tile of K and V codes is expanded
+// to fp16 centroids ONCE per workgroup on its way into LDS, instead of once per wave as in the decode
+// scan's layout.  64 NQ / R query tokens of R heads then reuse it.
+//
+// Arithmetic (turbo_gqa_prefill_attention_kernel, kernels.cu:1874-1960, in the rotated space):
+//   score[kv][q] = (sum_d c(K code[kv][d]) q_rot[q][d]) * k_norm[kv]          (kernels.cu:1707)
+//   acc[q][d]   += (p * v_norm[kv]) * c(V code[kv][d])                        (kernels.cu:1765)
+// with q_rot = R q pre-scaled by log2(e) / sqrt(128) / alpha (rotate_kernel), centroids stored as
+// fp16(alpha c) (alpha as in the decode scan: all magnitudes round with <= 1.1e-4 relative error), the
+// norms applied in fp32.  The rotated accumulators go to the split workspace as one partial per
+// (query token, head); merge_rotate_kernel normalises and applies R^T.
+
+#include "kv_common.hpp"
+#include "kv_kernels.hpp"
+#include "kv_mfma_util.hpp"
+
+namespace twkv {
+
+namespace {
+
+constexpr int kPtWaves = 4;
+constexpr int kPtKRow = 2 * kHeadDim + 16;   // bytes per expanded K row in LDS
+constexpr int kPtVRow = 2 * 32 + 16;         // bytes per V^T row (32 token slots) in LDS
+constexpr int kPtReplicas = 16;              // copies of the byte -> centroids table (bank conflicts of the expansion)
+
+// column of a tile's token in the V^T rows: the contraction slot order of the second MFMA
+__device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 2) + 4 * (token >> 4) + (token & 3); }
+
+}  // namespace
+
+// NQ: 16-row query blocks per wave (every K and V operand read feeds NQ MFMAs).  MIRROR: a workgroup does a
+// token block and then its mirror image from the other end of the sequence.
+template <int R, int BITS, int NQ, bool MIRROR>
+__global__ void __launch_bounds__(kPtWaves* kWave)
+prefill_tq_mfma_kernel(AttnArgs a, int T) {
+    constexpr int TPW = 16 * NQ * kPtWaves / R;            // query tokens per workgroup pass
+    constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
+    constexpr int kHeadBytes = BITS * 16;                  // bytes of one head in a cache row
+    constexpr int kEntryDwords = BITS == 4 ? 1 : 2;        // a byte holds 2 (4) codes -> 2 (4) halves
+    __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPtKRow];
+    __shared__ __attribute__((aligned(16))) char v_s[2][kHeadDim * kPtVRow];
+    __shared__ __attribute__((aligned(16))) float n_s[2][2][32];          // [buffer][k | v][token]
+    __shared__ __attribute__((aligned(8))) uint32_t tab_s[256 * kPtReplicas * kEntryDwords];
+
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid / kWave), lane = tid % kWave;
+    const int ln = lane & 15, kg = lane >> 4;
+    const int nblk = (T + TPW - 1) / TPW;
+    const int kvh = blockIdx.y;
+    const int head = kvh * R + wave % R;
+    const int row_bytes = a.num_kv_heads * kHeadBytes;
+    const char* kbase = reinterpret_cast<const char*>(a.k) + kvh * kHeadBytes;
+    const char* vbase = reinterpret_cast<const char*>(a.v) + kvh * kHeadBytes;
+    constexpr float kRaise = 5.0f;
+
+    // ---- table: byte -> its codes' centroids (low field first) as fp16(alpha c), kPtReplicas copies
+    for (int i = tid; i < 256 * kPtReplicas; i += kPtWaves * kWave) {
+        const int e = i / kPtReplicas;
+        if constexpr (BITS == 4) {
+            half2_t p = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
+            tab_s[i] = *reinterpret_cast<uint32_t*>(&p);
+        } else {
+            half2_t p0 = {(half_t)(kAlpha * kCentroids2[e & 3]), (half_t)(kAlpha * kCentroids2[(e >> 2) & 3])};
+            half2_t p1 = {(half_t)(kAlpha * kCentroids2[(e >> 4) & 3]), (half_t)(kAlpha * kCentroids2[(e >> 6) & 3])};
+            tab_s[2 * i] = *reinterpret_cast<uint32_t*>(&p0);
+            tab_s[2 * i + 1] = *reinterpret_cast<uint32_t*>(&p1);
+        }
+    }
+    const int rep = lane & (kPtReplicas - 1);
+    // the 8 halves (4 dwords) of 8 consecutive coordinates from their packed codes (4 bytes at 4 bit, 2 at 2 bit)
+    auto expand8 = [&](uint32_t codes, uint32_t (&out)[4]) {
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int b = 0; b < 4; b++) out[b] = tab_s[((codes >> (8 * b)) & 255u) * kPtReplicas + rep];
+        } else {
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                const uint2 v = *reinterpret_cast<const uint2*>(&tab_s[2 * (((codes >> (8 * b)) & 255u) * kPtReplicas + rep)]);
+                out[2 * b] = v.x; out[2 * b + 1] = v.y;
+            }
+        }
+    };
+    auto load_codes = [&](const char* p) -> uint32_t {
+        if constexpr (BITS == 4) return *reinterpret_cast<const uint32_t*>(p);
+        else return *reinterpret_cast<const uint16_t*>(p);
+    };
+
+    // ---- staging of a tile: thread (r = tid / 16, c = tid % 16) carries the codes of coordinates 8c..8c+7 of
+    // K rows r and r + 16, and of V rows 2r and 2r + 1 (two consecutive tokens, interleaved on the way into
+    // the transposed tile); threads 0..63 also carry a norm.  Rows past the last token are clamped (masked anyway).
+    const int sr = tid >> 4, sc = tid & 15;
+    constexpr int kPiece = BITS;                           // bytes of codes of 8 coordinates
+    struct Staged { uint32_t k[2], v[2]; float nrm; };
+    auto load_tile = [&](int tile, Staged& st) {
+        const int last = T - 1;
+        st.k[0] = load_codes(kbase + (long long)min(tile + sr, last) * row_bytes + kPiece * sc);
+        st.k[1] = load_codes(kbase + (long long)min(tile + sr + 16, last) * row_bytes + kPiece * sc);
+        st.v[0] = load_codes(vbase + (long long)min(tile + 2 * sr, last) * row_bytes + kPiece * sc);
+        st.v[1] = load_codes(vbase + (long long)min(tile + 2 * sr + 1, last) * row_bytes + kPiece * sc);
+        if (tid < 64) {
+            const half_t* nb = (tid < 32) ? a.k_norms : a.v_norms;
+            st.nrm = (float)nb[(long long)min(tile + (tid & 31), last) * a.num_kv_heads + kvh];
+        }
+    };
+    const int vcol = 2 * vt_slot(2 * sr);                  // byte column of the token pair in a V^T row
+    auto stash = [&](int buf, const Staged& st) {
+        uint32_t e[4];
+        expand8(st.k[0], e);
+        *reinterpret_cast<uint4*>(&k_s[buf][sr * kPtKRow + 16 * sc]) = uint4{e[0], e[1], e[2], e[3]};
+        expand8(st.k[1], e);
+        *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPtKRow + 16 * sc]) = uint4{e[0], e[1], e[2], e[3]};
+        uint32_t va[4], vb[4];
+        expand8(st.v[0], va);
+        expand8(st.v[1], vb);
+        char* dst = &v_s[buf][(8 * sc) * kPtVRow + vcol];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
+            *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
+            *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x07060302u);
+        }
+        if (tid < 64) n_s[buf][tid >> 5][tid & 31] = st.nrm;
+    };
+    __syncthreads();                                       // the table is there
+
+    // A workgroup takes token block blockIdx.x and its mirror image from the other end, one after the
+    // other: with causal rows the two together cost the same for every workgroup.
+    const int first = blockIdx.x, second = nblk - 1 - (int)blockIdx.x;   // without MIRROR: longest blocks first
+    for (int pass = 0; pass < (MIRROR ? 2 : 1); pass++) {
+        if (pass == 1 && second == first) break;           // the middle block of an odd count
+        const int tb = pass == 0 ? second : first;         // the long one first
+        const int q0 = tb * TPW + 16 * NQ * (wave / R);    // this wave's 16 NQ query tokens
+        const int wg_last = min(T, (tb + 1) * TPW) - 1;    // last query token of the pass
+        const int ntiles = (wg_last >> 5) + 1;
+
+        // ---- B operands of the first MFMA: q_rot[q0 + 16 nq + ln][32j + 8kg .. +7], j = 0..3, as an fp16 value
+        // and what its rounding left over (scores reach tens of base-2 units on caches with outlier channels,
+        // where a 2^-11 relative error of q alone would show in the output)
+        half8_t qb[NQ][4], ql[NQ][4];
+#pragma unroll
+        for (int nq = 0; nq < NQ; nq++) {
+            const float* qrow = a.qrot + ((long long)min(q0 + 16 * nq + ln, T - 1) * a.num_heads + head) * a.ws_stride + 8 * kg;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 v0 = *reinterpret_cast<const float4*>(qrow + 32 * j), v1 = *reinterpret_cast<const float4*>(qrow + 32 * j + 4);
+                const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const half_t hi = (half_t)v[i];
+                    qb[nq][j][i] = hi;
+                    ql[nq][j][i] = (half_t)(v[i] - (float)hi);
+                }
+            }
+        }
+        float4_t o[NQ][8];
+        float m_run[NQ], l_run[NQ];
+#pragma unroll
+        for (int nq = 0; nq < NQ; nq++) {
+            m_run[nq] = kNegBig; l_run[nq] = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) o[nq][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+
+        Staged st;
+        load_tile(0, st);
+        stash(0, st);
+        __syncthreads();
+
+        for (int it = 0; it < ntiles; it++) {
+            const int buf = it & 1;
+            const int tile = 32 * it;
+            const bool more = it + 1 < ntiles;
+            if (more) load_tile(tile + 32, st);
+
+            if (tile <= q0 + 16 * NQ - 1 && q0 < T) {      // the tile reaches this wave's queries (uniform over the wave)
+                // ---- S^T[kv][query] for both 16-token halves and all query blocks
+                float4_t s[NQ][2];
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                    for (int nq = 0; nq < NQ; nq++) s[nq][sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+                    const char* krow = &k_s[buf][(16 * sub + ln) * kPtKRow + 16 * kg];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const half8_t ka = *reinterpret_cast<const half8_t*>(krow + 64 * j);
+#pragma unroll
+                        for (int nq = 0; nq < NQ; nq++) {
+                            s[nq][sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[nq][j], s[nq][sub], 0, 0, 0);
+                            s[nq][sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, ql[nq][j], s[nq][sub], 0, 0, 0);
+                        }
+                    }
+                }
+                // ---- online softmax per query: this lane holds kv tokens tile + 16 sub + 4kg + i
+                float kn[8], vn[8];
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(&n_s[buf][0][16 * sub + 4 * kg]);
+                    const float4 v4 = *reinterpret_cast<const float4*>(&n_s[buf][1][16 * sub + 4 * kg]);
+                    kn[4 * sub] = k4.x; kn[4 * sub + 1] = k4.y; kn[4 * sub + 2] = k4.z; kn[4 * sub + 3] = k4.w;
+                    vn[4 * sub] = v4.x; vn[4 * sub + 1] = v4.y; vn[4 * sub + 2] = v4.z; vn[4 * sub + 3] = v4.w;
+                }
+                half8_t pa[NQ], pl[NQ];                        // p * vn as an fp16 value and its rounding remainder
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) {
+                    const int tq = q0 + 16 * nq + ln;
+                    float x[8];
+                    float mx = kNegBig;
+#pragma unroll
+                    for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const bool valid = tile + 16 * sub + 4 * kg + i <= tq;
+                            x[4 * sub + i] = valid ? s[nq][sub][i] * kn[4 * sub + i] : kNegBig;    // kernels.cu:1707
+                            mx = fmaxf(mx, x[4 * sub + i]);
+                        }
+                    }
+                    if (__any(mx > m_run[nq] + kRaise)) {  // rare after the first tiles
+                        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
+                        const float m_new = fmaxf(m_run[nq], mx);
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[nq] - m_new);
+                        m_run[nq] = m_new;
+                        l_run[nq] *= alpha;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {      // accumulator register i belongs to query 4kg + i
+                            const float ai = __shfl(alpha, 4 * kg + i, 64);
+#pragma unroll
+                            for (int j = 0; j < 8; j++) o[nq][j][i] *= ai;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float p = __builtin_amdgcn_exp2f(x[i] - m_run[nq]);
+                        l_run[nq] += p;
+                        const float pv = p * vn[i];                             // (s * vn) * centroid, kernels.cu:1765
+                        const half_t hi = (half_t)pv;
+                        pa[nq][i] = hi;
+                        pl[nq][i] = (half_t)(pv - (float)hi);
+                    }
+                }
+                // ---- O[query][dim 16j + ln] += P . V
+                const char* vrow = &v_s[buf][ln * kPtVRow + 16 * kg];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPtVRow);
+#pragma unroll
+                    for (int nq = 0; nq < NQ; nq++) {
+                        o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
+                        o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[nq], vb, o[nq][j], 0, 0, 0);
+                    }
+                }
+            }
+
+            if (more) stash(buf ^ 1, st);
+            __syncthreads();
+        }
+
+        // ---- one partial per (query token, head): rotated accumulator, running maximum (base 2) and sum;
+        // the merge normalises (kernels.cu:1946: 1 / (sum + 1e-8)) and rotates back.  Accumulator register i
+        // is query 4kg + i, maximum and sum sit in the lanes whose ln is the query.
+#pragma unroll
+        for (int nq = 0; nq < NQ; nq++) {
+            float l = l_run[nq];
+            l += __shfl_xor(l, 16, 64);
+            l += __shfl_xor(l, 32, 64);
+            const int tq = q0 + 16 * nq + ln;
+            if (kg == 0 && tq < T) {
+                float* part = a.ws + ((long long)tq * a.num_heads + head) * a.ws_stride;
+                part[kHeadDim] = m_run[nq];
+                part[kHeadDim + 1] = l;
+                reinterpret_cast<int*>(part)[kHeadDim + 2] = 1;          // one partial
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int t = q0 + 16 * nq + 4 * kg + i;
+                if (t < T) {
+                    float* part = a.ws + ((long long)t * a.num_heads + head) * a.ws_stride + ln;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) part[16 * j] = o[nq][j][i] * (1.0f / kAlpha);
+                }
+            }
+        }
+    }
+}
+
+
+// compressed cache, one sequence, query t attends rows 0..t, GQA group 1, 2 or 4, workspace with q_rot
+bool prefill_tq_mfma_usable(const AttnArgs& a) {
+    const int R = a.num_heads / a.num_kv_heads;
+    if ((a.bits != 4 && a.bits != 2) || a.pos_mode != kPosIota || a.block_table || a.seq_stride_rows != 0) return false;
+    if (R != 1 && R != 2 && R != 4) return false;
+    return a.ws && a.qrot && a.G >= 1 && (a.ws_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0;
+}
+
+void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form) {
+    const int R = a.num_heads / a.num_kv_heads;
+    const int T = a.G;
+    // forms as for the fp16 prefill kernel: long prompts take two query blocks per wave and mirrored block pairs
+    const int cus = compute_units();
+    int mode = 1;
+    {
+        const int nblk2 = (T + 32 * kPtWaves / R - 1) / (32 * kPtWaves / R), nblk1 = (T + 16 * kPtWaves / R - 1) / (16 * kPtWaves / R);
+        if ((nblk2 + 1) / 2 * a.num_kv_heads >= cus) mode = 3;
+        else if ((nblk1 + 1) / 2 * a.num_kv_heads >= cus) mode = 2;
+    }
+    if (form >= 1 && form <= 3) mode = form;               // forced by a test
+    const int nq = mode >= 3 ? 2 : 1;
+    const bool mirror = mode == 2 || mode == 3;
+    const int tpw = 16 * nq * kPtWaves / R;
+    const int nblk = (T + tpw - 1) / tpw;
+    const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(kPtWaves * kWave);
+#define TW_PT_LAUNCH(RR, BB, NN, MM) launch_scan_kernel(prefill_tq_mfma_kernel<RR, BB, NN, MM>, grid, block, s, a, T)
+#define TW_PT_MODES(RR, BB) \
+    do { if (mode == 1) TW_PT_LAUNCH(RR, BB, 1, false); else if (mode == 2) TW_PT_LAUNCH(RR, BB, 1, true); \
+         else TW_PT_LAUNCH(RR, BB, 2, true); } while (0)
+#define TW_PT_BITS(RR) do { if (a.bits == 4) TW_PT_MODES(RR, 4); else TW_PT_MODES(RR, 2); } while (0)
+    if (R == 1) TW_PT_BITS(1); else if (R == 2) TW_PT_BITS(2); else TW_PT_BITS(4);
+#undef TW_PT_BITS
+#undef TW_PT_MODES
+#undef TW_PT_LAUNCH
+}
+
+}  // namespace twkv

@@ -67,38 +67,51 @@ rotate_kernel(RotArgs a) {
     const int lane = threadIdx.x;
     const int i16 = lane & 15, kk = lane >> 4;
 
-    // ---- which unit
+    // ---- which unit: (segment, group of a.nper vector tiles, block of 16 output coordinates)
     int unit = blockIdx.x;
     int seg = 0;
     while (seg < a.nseg - 1 && unit >= a.seg_units[seg]) { unit -= a.seg_units[seg]; seg++; }
     const int dblk = unit & 7;
-    const int vtile = unit >> 3;
+    const int vgroup = unit >> 3;
     const int nvec = a.seg_nvec[seg];
     const int heads = a.seg_heads[seg];                  // head vectors per source row
     const bool is_query = a.seg_kind[seg] != 0;
+    const bool roped = a.seg_rope[seg] != 0;
+
+    // ---- A operand, once per wave: R row d0 + i16 as 16 pieces of 8 halves
+    const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (dblk * 16 + i16) * kHeadDim);
+    float rv[32];
+#pragma unroll
+    for (int q = 0; q < 16; q++) {
+        uint4 rp = rsrc[q];
+        rv[2 * q] = pick_half(rp, 0, kk);
+        rv[2 * q + 1] = pick_half(rp, 1, kk);
+    }
+
+    // Small launches (decode) give every wave one tile of 16 vectors; large ones (prompts) let a wave keep
+    // its rows of R and walk a.nper tiles.
+    for (int it = 0; it < a.nper; it++) {
+    const int vtile = vgroup * a.nper + it;
+    if (vtile * 16 >= nvec) break;
     const int v = vtile * 16 + i16;
     const int vc = v < nvec ? v : nvec - 1;              // clamp loads, mask stores
     const int row = vc / heads, head = vc - row * heads;
 
-    // ---- operands: R row d0 + i16 and source vector v, both as 16 pieces of 8 halves
-    const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (dblk * 16 + i16) * kHeadDim);
+    // ---- B operand: source vector v as 16 pieces of 8 halves
     const uint4* xsrc = reinterpret_cast<const uint4*>(a.seg_src[seg] + (long long)row * a.seg_stride[seg] +
                                                        (long long)head * kHeadDim);
     // position of this vector's row: needed for the cache row and for the rotary table row, so it is the
     // first thing asked for; everything that depends on it is requested before the operands are used
-    const bool roped = a.seg_rope[seg] != 0;
     const int pos_row = (!is_query || roped) ? a.positions[row] : 0;
     long long crow = 0;
     if (!is_query) {
         if (a.token_list) crow = pos_row;                                // sequence 0, kernels.cu:1499, 1553
         else crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, pos_row);
     }
-    float rv[32], xv[32];
+    float xv[32];
 #pragma unroll
     for (int q = 0; q < 16; q++) {
-        uint4 rp = rsrc[q], xp = xsrc[q];
-        rv[2 * q] = pick_half(rp, 0, kk);
-        rv[2 * q + 1] = pick_half(rp, 1, kk);
+        uint4 xp = xsrc[q];
         xv[2 * q] = pick_half(xp, 0, kk);
         xv[2 * q + 1] = pick_half(xp, 1, kk);
     }
@@ -177,7 +190,7 @@ rotate_kernel(RotArgs a) {
             float4 o = {acc[0] * a.q_scale, acc[1] * a.q_scale, acc[2] * a.q_scale, acc[3] * a.q_scale};
             *reinterpret_cast<float4*>(dst) = o;
         }
-        return;
+        continue;
     }
 
     // ---- quantize the lane's 4 consecutive coordinates d0 + 4kk .. +3 and pack (low field first)
@@ -200,11 +213,26 @@ rotate_kernel(RotArgs a) {
         }
         if (dblk == 0) a.seg_norms[seg][crow * a.num_kv_heads + head] = (half_t)sqrtf(n2 + 1e-12f);
     }
+    }   // tiles of this wave
 }
 
-void launch_rotate(const RotArgs& a, int bits, hipStream_t s) {
+void launch_rotate(const RotArgs& args, int bits, hipStream_t s) {
+    RotArgs a = args;
+    // tiles of 16 vectors per wave: one while the launch is small, more once there are far more tiles than
+    // the GPU holds waves
+    long long tiles = 0;
+    for (int i = 0; i < a.nseg; i++) tiles += (a.seg_nvec[i] + 15) / 16;
+    constexpr long long kWantUnits = 16384;               // 64 single-wave workgroups per CU
+    int nper = (int)((tiles * 8 + kWantUnits - 1) / kWantUnits);
+    if (nper < 1) nper = 1;
+    if (nper > 32) nper = 32;
+    a.nper = nper;
     int units = 0;
-    for (int i = 0; i < a.nseg; i++) units += a.seg_units[i];
+    for (int i = 0; i < a.nseg; i++) {
+        const int t = (a.seg_nvec[i] + 15) / 16;
+        a.seg_units[i] = (t + nper - 1) / nper * 8;
+        units += a.seg_units[i];
+    }
     if (units <= 0) return;
     if (bits == 4) hipLaunchKernelGGL(rotate_kernel<4>, dim3(units), dim3(kWave), 0, s, a);
     else hipLaunchKernelGGL(rotate_kernel<2>, dim3(units), dim3(kWave), 0, s, a);
