@@ -66,25 +66,37 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
     constexpr float kRaise = 5.0f;
 
     // ---- staging of a tile: thread (r = tid / 16, c = tid % 16) carries 16 bytes (dims 8c..8c+7) of
-    // K rows r and r + 16, and of V rows 2r and 2r + 1 (two consecutive tokens, interleaved on the way
-    // into the transposed tile).  Rows past the last token are clamped (they are masked anyway).
+    // K rows r and r + 16; for V, thread (c = tid / 16, r = tid % 16) carries dims 8c..8c+7 of rows 2r and
+    // 2r + 1 (two consecutive tokens, interleaved on the way into the transposed tile).  Rows past the
+    // last token are clamped (they are masked anyway).
     const int sr = tid >> 4, sc = tid & 15;
+    // V: 16 consecutive threads take the 16 token pairs of one dim octet, so that their dwords fill one V^T row
+    // (64 contiguous bytes, all banks different); with the K mapping they would hit rows 8 apart, 8 to a bank
+    const int vr_ = tid & 15, vc_ = tid >> 4;
+    // Buffer loads: descriptor over the T rows of the cache (rows past the last token read as zeros and are
+    // masked anyway), per-thread byte offsets fixed for the whole kernel, the tile's row offset in a scalar.
+    const __amdgpu_buffer_rsrc_t krs = make_rsrc(reinterpret_cast<const char*>(kbase), T * kv_dim * 2 - kvh * kHeadDim * 2);
+    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(reinterpret_cast<const char*>(vbase), T * kv_dim * 2 - kvh * kHeadDim * 2);
+    const int koff0 = (sr * kv_dim + 8 * sc) * 2, koff1 = koff0 + 16 * kv_dim * 2;
+    const int voff0 = (2 * vr_ * kv_dim + 8 * vc_) * 2, voff1 = voff0 + kv_dim * 2;
     auto load_tile = [&](int tile, uint4 (&kr)[2], uint4 (&vr)[2]) {
-        const int last = T - 1;
-        const long long k0 = (long long)min(tile + sr, last) * kv_dim, k1 = (long long)min(tile + sr + 16, last) * kv_dim;
-        const long long v0 = (long long)min(tile + 2 * sr, last) * kv_dim, v1 = (long long)min(tile + 2 * sr + 1, last) * kv_dim;
-        kr[0] = *reinterpret_cast<const uint4*>(kbase + k0 + 8 * sc);
-        kr[1] = *reinterpret_cast<const uint4*>(kbase + k1 + 8 * sc);
-        vr[0] = *reinterpret_cast<const uint4*>(vbase + v0 + 8 * sc);
-        vr[1] = *reinterpret_cast<const uint4*>(vbase + v1 + 8 * sc);
+        const int toff = tile * kv_dim * 2;
+        const uint32x4_t k0 = __builtin_amdgcn_raw_buffer_load_b128(krs, koff0, toff, 0);
+        const uint32x4_t k1 = __builtin_amdgcn_raw_buffer_load_b128(krs, koff1, toff, 0);
+        const uint32x4_t v0 = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff0, toff, 0);
+        const uint32x4_t v1 = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff1, toff, 0);
+        kr[0] = uint4{k0[0], k0[1], k0[2], k0[3]};
+        kr[1] = uint4{k1[0], k1[1], k1[2], k1[3]};
+        vr[0] = uint4{v0[0], v0[1], v0[2], v0[3]};
+        vr[1] = uint4{v1[0], v1[1], v1[2], v1[3]};
     };
-    const int vcol = 2 * vt_slot(2 * sr);                  // byte column of the token pair in a V^T row
+    const int vcol = 2 * vt_slot(2 * vr_);                  // byte column of the token pair in a V^T row
     auto stash = [&](int buf, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
         *reinterpret_cast<uint4*>(&k_s[buf][sr * kPfKRow + 16 * sc]) = kr[0];
         *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPfKRow + 16 * sc]) = kr[1];
         const uint32_t va[4] = {vr[0].x, vr[0].y, vr[0].z, vr[0].w};
         const uint32_t vb[4] = {vr[1].x, vr[1].y, vr[1].z, vr[1].w};
-        char* dst = &v_s[buf][(8 * sc) * kPfVRow + vcol];
+        char* dst = &v_s[buf][(8 * vc_) * kPfVRow + vcol];
 #pragma unroll
         for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPfVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
@@ -152,16 +164,23 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                 for (int nq = 0; nq < NQ; nq++) {
                     const int tq = q0 + 16 * nq + ln;
                     float x[8];
-                    float mx = kNegBig;
 #pragma unroll
                     for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            const bool valid = tile + 16 * sub + 4 * kg + i <= tq;
-                            x[4 * sub + i] = valid ? s[nq][sub][i] * scale2 : kNegBig;
-                            mx = fmaxf(mx, x[4 * sub + i]);
+                        for (int i = 0; i < 4; i++) x[4 * sub + i] = s[nq][sub][i] * scale2;
+                    }
+                    if (tile + 31 > q0 + 16 * nq) {        // the tile crosses this block's diagonal (uniform over the wave)
+#pragma unroll
+                        for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                if (tile + 16 * sub + 4 * kg + i > tq) x[4 * sub + i] = kNegBig;
+                            }
                         }
                     }
+                    float mx = x[0];
+#pragma unroll
+                    for (int i = 1; i < 8; i++) mx = fmaxf(mx, x[i]);
                     if (__any(mx > m_run[nq] + kRaise)) {  // rare after the first tiles
                         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
@@ -230,7 +249,8 @@ bool prefill_f16_mfma_usable(const AttnArgs& a) {
     if (R != 1 && R != 2 && R != 4) return false;
     if ((a.q_stride & 7) != 0) return false;
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.k) | reinterpret_cast<uintptr_t>(a.v);
-    return (bits & 15u) == 0 && a.G >= 1;
+    const long long cache_bytes = (long long)a.G * a.num_kv_heads * kHeadDim * 2;     // one buffer descriptor spans it
+    return (bits & 15u) == 0 && a.G >= 1 && cache_bytes < (1LL << 31);
 }
 
 void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form) {

@@ -82,29 +82,41 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
             }
         }
     };
-    auto load_codes = [&](const char* p) -> uint32_t {
-        if constexpr (BITS == 4) return *reinterpret_cast<const uint32_t*>(p);
-        else return *reinterpret_cast<const uint16_t*>(p);
-    };
 
     // ---- staging of a tile: thread (r = tid / 16, c = tid % 16) carries the codes of coordinates 8c..8c+7 of
-    // K rows r and r + 16, and of V rows 2r and 2r + 1 (two consecutive tokens, interleaved on the way into
-    // the transposed tile); threads 0..63 also carry a norm.  Rows past the last token are clamped (masked anyway).
+    // K rows r and r + 16; for V, thread (c = tid / 16, r = tid % 16) carries those of rows 2r and 2r + 1 (two
+    // consecutive tokens, interleaved on the way into the transposed tile); threads 0..63 also carry a norm.
+    // Rows past the last token are clamped (masked anyway).
     const int sr = tid >> 4, sc = tid & 15;
+    // V: 16 consecutive threads take the 16 token pairs of one dim octet, so that their dwords fill one V^T row
+    // (64 contiguous bytes, all banks different); with the K mapping they would hit rows 8 apart, 8 to a bank
+    const int vr_ = tid & 15, vc_ = tid >> 4;
     constexpr int kPiece = BITS;                           // bytes of codes of 8 coordinates
     struct Staged { uint32_t k[2], v[2]; float nrm; };
-    auto load_tile = [&](int tile, Staged& st) {
-        const int last = T - 1;
-        st.k[0] = load_codes(kbase + (long long)min(tile + sr, last) * row_bytes + kPiece * sc);
-        st.k[1] = load_codes(kbase + (long long)min(tile + sr + 16, last) * row_bytes + kPiece * sc);
-        st.v[0] = load_codes(vbase + (long long)min(tile + 2 * sr, last) * row_bytes + kPiece * sc);
-        st.v[1] = load_codes(vbase + (long long)min(tile + 2 * sr + 1, last) * row_bytes + kPiece * sc);
-        if (tid < 64) {
-            const half_t* nb = (tid < 32) ? a.k_norms : a.v_norms;
-            st.nrm = (float)nb[(long long)min(tile + (tid & 31), last) * a.num_kv_heads + kvh];
-        }
+    // Buffer loads: descriptors over the T rows of the cache (rows past the last token read as zeros and are
+    // masked anyway), per-thread byte offsets fixed for the whole kernel, the tile's row offset in a scalar.
+    const __amdgpu_buffer_rsrc_t krs = make_rsrc(kbase, T * row_bytes - kvh * kHeadBytes);
+    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(vbase, T * row_bytes - kvh * kHeadBytes);
+    const int nrow_bytes = a.num_kv_heads * 2;
+    const __amdgpu_buffer_rsrc_t knrs = make_rsrc(reinterpret_cast<const char*>(a.k_norms) + kvh * 2, T * nrow_bytes - kvh * 2);
+    const __amdgpu_buffer_rsrc_t vnrs = make_rsrc(reinterpret_cast<const char*>(a.v_norms) + kvh * 2, T * nrow_bytes - kvh * 2);
+    const int koff0 = sr * row_bytes + kPiece * sc, koff1 = koff0 + 16 * row_bytes;
+    const int voff0 = 2 * vr_ * row_bytes + kPiece * vc_, voff1 = voff0 + row_bytes;
+    const int noff = (tid & 31) * nrow_bytes;
+    auto load_codes = [&](__amdgpu_buffer_rsrc_t rs, int voff, int soff) -> uint32_t {
+        if constexpr (BITS == 4) return __builtin_amdgcn_raw_buffer_load_b32(rs, voff, soff, 0);
+        else return __builtin_amdgcn_raw_buffer_load_b16(rs, voff, soff, 0);
     };
-    const int vcol = 2 * vt_slot(2 * sr);                  // byte column of the token pair in a V^T row
+    auto load_tile = [&](int tile, Staged& st) {
+        const int toff = tile * row_bytes;
+        st.k[0] = load_codes(krs, koff0, toff);
+        st.k[1] = load_codes(krs, koff1, toff);
+        st.v[0] = load_codes(vrs, voff0, toff);
+        st.v[1] = load_codes(vrs, voff1, toff);
+        if (tid < 32) st.nrm = h2f_bits(__builtin_amdgcn_raw_buffer_load_b16(knrs, noff, tile * nrow_bytes, 0));
+        else if (tid < 64) st.nrm = h2f_bits(__builtin_amdgcn_raw_buffer_load_b16(vnrs, noff, tile * nrow_bytes, 0));
+    };
+    const int vcol = 2 * vt_slot(2 * vr_);                  // byte column of the token pair in a V^T row
     auto stash = [&](int buf, const Staged& st) {
         uint32_t e[4];
         expand8(st.k[0], e);
@@ -114,7 +126,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         uint32_t va[4], vb[4];
         expand8(st.v[0], va);
         expand8(st.v[1], vb);
-        char* dst = &v_s[buf][(8 * sc) * kPtVRow + vcol];
+        char* dst = &v_s[buf][(8 * vc_) * kPtVRow + vcol];
 #pragma unroll
         for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
@@ -205,16 +217,20 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
                 for (int nq = 0; nq < NQ; nq++) {
                     const int tq = q0 + 16 * nq + ln;
                     float x[8];
-                    float mx = kNegBig;
 #pragma unroll
-                    for (int sub = 0; sub < 2; sub++) {
+                    for (int i = 0; i < 8; i++) x[i] = s[nq][i >> 2][i & 3] * kn[i];              // kernels.cu:1707
+                    if (tile + 31 > q0 + 16 * nq) {        // the tile crosses this block's diagonal (uniform over the wave)
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            const bool valid = tile + 16 * sub + 4 * kg + i <= tq;
-                            x[4 * sub + i] = valid ? s[nq][sub][i] * kn[4 * sub + i] : kNegBig;    // kernels.cu:1707
-                            mx = fmaxf(mx, x[4 * sub + i]);
+                        for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                if (tile + 16 * sub + 4 * kg + i > tq) x[4 * sub + i] = kNegBig;
+                            }
                         }
                     }
+                    float mx = x[0];
+#pragma unroll
+                    for (int i = 1; i < 8; i++) mx = fmaxf(mx, x[i]);
                     if (__any(mx > m_run[nq] + kRaise)) {  // rare after the first tiles
                         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
@@ -290,7 +306,9 @@ bool prefill_tq_mfma_usable(const AttnArgs& a) {
     const int R = a.num_heads / a.num_kv_heads;
     if ((a.bits != 4 && a.bits != 2) || a.pos_mode != kPosIota || a.block_table || a.seq_stride_rows != 0) return false;
     if (R != 1 && R != 2 && R != 4) return false;
-    return a.ws && a.qrot && a.G >= 1 && (a.ws_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0;
+    const long long cache_bytes = (long long)a.G * a.num_kv_heads * a.bits * 16;      // one buffer descriptor spans it
+    return a.ws && a.qrot && a.G >= 1 && (a.ws_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0 &&
+           cache_bytes < (1LL << 31);
 }
 
 void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form) {
