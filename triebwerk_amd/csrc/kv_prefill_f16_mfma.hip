@@ -20,8 +20,9 @@
 // query head w % R and 16 NQ tokens; with NQ = 2 the two 16-row blocks share every operand read),
 // walks the kv tiles of 32 tokens up to its diagonal and shares each tile through LDS: K row-major
 // (padded rows), V transposed on the way in (each thread interleaves the same 8 dims of two
-// consecutive tokens and writes 8 dwords).  Tiles are double-buffered: the next tile's global loads
-// are issued before the arithmetic and stored to LDS after it, one barrier per tile.  For long
+// consecutive tokens and writes 8 dwords).  The next tile's global loads are issued before the
+// arithmetic and stored to LDS after it, one barrier per tile; the P.V product of a tile runs one
+// iteration late, under the softmax arithmetic of the next tile (three V buffers, two K buffers).  For long
 // prompts a workgroup does a token block and then its mirror image from the other end of the
 // sequence, so causal rows cost every workgroup the same; short prompts take one block each, longest
 // first.
@@ -47,11 +48,11 @@ __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 
 // NQ: 16-row query blocks per wave (every K and V operand read feeds NQ MFMAs).  MIRROR: a workgroup does a
 // token block and then its mirror image from the other end of the sequence.
 template <int R, int NQ, bool MIRROR>
-__global__ void __launch_bounds__(kPfWaves* kWave)
+__global__ void __launch_bounds__(kPfWaves* kWave, 2)        // two workgroups per CU (three would spill)
 prefill_f16_mfma_kernel(AttnArgs a, int T) {
     constexpr int TPW = 16 * NQ * kPfWaves / R;            // query tokens per workgroup pass
     __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPfKRow];
-    __shared__ __attribute__((aligned(16))) char v_s[2][kHeadDim * kPfVRow];
+    __shared__ __attribute__((aligned(16))) char v_s[3][kHeadDim * kPfVRow];
 
     const int tid = threadIdx.x;
     const int wave = uniform(tid / kWave), lane = tid % kWave;
@@ -91,12 +92,12 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
         vr[1] = uint4{v1[0], v1[1], v1[2], v1[3]};
     };
     const int vcol = 2 * vt_slot(2 * vr_);                  // byte column of the token pair in a V^T row
-    auto stash = [&](int buf, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
+    auto stash = [&](int buf, int vbuf, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
         *reinterpret_cast<uint4*>(&k_s[buf][sr * kPfKRow + 16 * sc]) = kr[0];
         *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPfKRow + 16 * sc]) = kr[1];
         const uint32_t va[4] = {vr[0].x, vr[0].y, vr[0].z, vr[0].w};
         const uint32_t vb[4] = {vr[1].x, vr[1].y, vr[1].z, vr[1].w};
-        char* dst = &v_s[buf][(8 * vc_) * kPfVRow + vcol];
+        char* dst = &v_s[vbuf][(8 * vc_) * kPfVRow + vcol];
 #pragma unroll
         for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPfVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
@@ -131,20 +132,39 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
             for (int j = 0; j < 8; j++) o[nq][j] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
 
+        // ---- O[query][dim 16j + ln] += P . V for one tile
+        auto pv = [&](int vbuf, const half8_t (&pa)[NQ]) {
+            const char* vrow = &v_s[vbuf][ln * kPfVRow + 16 * kg];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
+            }
+        };
+
+        // The loop is skewed by one tile: iteration t computes the scores of tile t, then the P.V product of
+        // tile t - 1 (whose MFMAs do not depend on anything of tile t and run under the softmax arithmetic of
+        // tile t), then the softmax of tile t.  So V tiles live one iteration longer than K tiles: three
+        // V buffers, two K buffers.
+        __syncthreads();                                   // a previous pass may still be reading its last V tile
         uint4 kr[2], vr[2];
         load_tile(0, kr, vr);
-        stash(0, kr, vr);
+        stash(0, 0, kr, vr);
         __syncthreads();
 
+        half8_t pa_prev[NQ];
+        bool have_prev = false;
         for (int it = 0; it < ntiles; it++) {
             const int buf = it & 1;
             const int tile = 32 * it;
             const bool more = it + 1 < ntiles;
             if (more) load_tile(tile + 32, kr, vr);
 
-            if (tile <= q0 + 16 * NQ - 1 && q0 < T) {      // the tile reaches this wave's queries (uniform over the wave)
+            const bool active = tile <= q0 + 16 * NQ - 1 && q0 < T;      // the tile reaches this wave's queries (uniform over the wave)
+            float4_t s[NQ][2];
+            if (active) {
                 // ---- S^T[kv][query] for both 16-token halves and all query blocks
-                float4_t s[NQ][2];
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
@@ -158,8 +178,11 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                             s[nq][sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[nq][j], s[nq][sub], 0, 0, 0);
                     }
                 }
+            }
+            if (have_prev) pv((it + 2) % 3, pa_prev);      // tile it - 1 sits in V buffer (it - 1) % 3
+            have_prev = active;
+            if (active) {
                 // ---- online softmax per query: this lane holds kv tokens tile + 16 sub + 4kg + i
-                half8_t pa[NQ];
 #pragma unroll
                 for (int nq = 0; nq < NQ; nq++) {
                     const int tq = q0 + 16 * nq + ln;
@@ -199,22 +222,15 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                     for (int i = 0; i < 8; i++) {
                         const float p = __builtin_amdgcn_exp2f(x[i] - m_run[nq]);
                         l_run[nq] += p;
-                        pa[nq][i] = (half_t)p;
+                        pa_prev[nq][i] = (half_t)p;
                     }
-                }
-                // ---- O[query][dim 16j + ln] += P . V
-                const char* vrow = &v_s[buf][ln * kPfVRow + 16 * kg];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
-#pragma unroll
-                    for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
                 }
             }
 
-            if (more) stash(buf ^ 1, kr, vr);
+            if (more) stash(buf ^ 1, (it + 1) % 3, kr, vr);
             __syncthreads();
         }
+        if (have_prev) pv((ntiles - 1) % 3, pa_prev);
 
         // ---- normalise (kernels.cu:1146: 1 / (sum + 1e-8)) and store; accumulator register i is query 4kg + i
 #pragma unroll

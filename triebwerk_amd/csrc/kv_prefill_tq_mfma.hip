@@ -23,7 +23,6 @@ namespace {
 constexpr int kPtWaves = 4;
 constexpr int kPtKRow = 2 * kHeadDim + 16;   // bytes per expanded K row in LDS
 constexpr int kPtVRow = 2 * 32 + 16;         // bytes per V^T row (32 token slots) in LDS
-constexpr int kPtReplicas = 16;              // copies of the byte -> centroids table (bank conflicts of the expansion)
 
 // column of a tile's token in the V^T rows: the contraction slot order of the second MFMA
 __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 2) + 4 * (token >> 4) + (token & 3); }
@@ -33,15 +32,16 @@ __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 
 // NQ: 16-row query blocks per wave (every K and V operand read feeds NQ MFMAs).  MIRROR: a workgroup does a
 // token block and then its mirror image from the other end of the sequence.
 template <int R, int BITS, int NQ, bool MIRROR>
-__global__ void __launch_bounds__(kPtWaves* kWave)
+__global__ void __launch_bounds__(kPtWaves* kWave, 2)        // two workgroups per CU: at most 256 registers per lane
 prefill_tq_mfma_kernel(AttnArgs a, int T) {
     constexpr int TPW = 16 * NQ * kPtWaves / R;            // query tokens per workgroup pass
     constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
     constexpr int kHeadBytes = BITS * 16;                  // bytes of one head in a cache row
     constexpr int kEntryDwords = BITS == 4 ? 1 : 2;        // a byte holds 2 (4) codes -> 2 (4) halves
+    constexpr int kPtReplicas = BITS == 4 ? 16 : 8;        // copies of the byte -> centroids table (16 KB either way): fewer bank conflicts in the expansion
     __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPtKRow];
-    __shared__ __attribute__((aligned(16))) char v_s[2][kHeadDim * kPtVRow];
-    __shared__ __attribute__((aligned(16))) float n_s[2][2][32];          // [buffer][k | v][token]
+    __shared__ __attribute__((aligned(16))) char v_s[3][kHeadDim * kPtVRow];
+    __shared__ __attribute__((aligned(16))) float n_s[3][2][32];          // [buffer][k | v][token]
     __shared__ __attribute__((aligned(8))) uint32_t tab_s[256 * kPtReplicas * kEntryDwords];
 
     const int tid = threadIdx.x;
@@ -117,7 +117,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         else if (tid < 64) st.nrm = h2f_bits(__builtin_amdgcn_raw_buffer_load_b16(vnrs, noff, tile * nrow_bytes, 0));
     };
     const int vcol = 2 * vt_slot(2 * vr_);                  // byte column of the token pair in a V^T row
-    auto stash = [&](int buf, const Staged& st) {
+    auto stash = [&](int buf, int vbuf, const Staged& st) {
         uint32_t e[4];
         expand8(st.k[0], e);
         *reinterpret_cast<uint4*>(&k_s[buf][sr * kPtKRow + 16 * sc]) = uint4{e[0], e[1], e[2], e[3]};
@@ -126,13 +126,13 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         uint32_t va[4], vb[4];
         expand8(st.v[0], va);
         expand8(st.v[1], vb);
-        char* dst = &v_s[buf][(8 * vc_) * kPtVRow + vcol];
+        char* dst = &v_s[vbuf][(8 * vc_) * kPtVRow + vcol];
 #pragma unroll
         for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
             *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x07060302u);
         }
-        if (tid < 64) n_s[buf][tid >> 5][tid & 31] = st.nrm;
+        if (tid < 64) n_s[vbuf][tid >> 5][tid & 31] = st.nrm;
     };
     __syncthreads();                                       // the table is there
 
@@ -174,20 +174,40 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
             for (int j = 0; j < 8; j++) o[nq][j] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
 
+        // ---- O[query][dim 16j + ln] += P . V for one tile (value and remainder of p * v_norm)
+        auto pv = [&](int vbuf, const half8_t (&pa)[NQ], const half8_t (&pl)[NQ]) {
+            const char* vrow = &v_s[vbuf][ln * kPtVRow + 16 * kg];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPtVRow);
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) {
+                    o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
+                    o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[nq], vb, o[nq][j], 0, 0, 0);
+                }
+            }
+        };
+
+        // The loop is skewed by one tile as in the fp16 kernel: scores of tile t, then the P.V product of tile
+        // t - 1 under the softmax arithmetic of tile t.  Three V (and norm) buffers, two K buffers.
+        __syncthreads();                                   // a previous pass may still be reading its last V tile
         Staged st;
         load_tile(0, st);
-        stash(0, st);
+        stash(0, 0, st);
         __syncthreads();
 
+        half8_t pa_prev[NQ], pl_prev[NQ];
+        bool have_prev = false;
         for (int it = 0; it < ntiles; it++) {
-            const int buf = it & 1;
+            const int buf = it & 1, nbuf = it % 3;
             const int tile = 32 * it;
             const bool more = it + 1 < ntiles;
             if (more) load_tile(tile + 32, st);
 
-            if (tile <= q0 + 16 * NQ - 1 && q0 < T) {      // the tile reaches this wave's queries (uniform over the wave)
+            const bool active = tile <= q0 + 16 * NQ - 1 && q0 < T;      // the tile reaches this wave's queries (uniform over the wave)
+            float4_t s[NQ][2];
+            if (active) {
                 // ---- S^T[kv][query] for both 16-token halves and all query blocks
-                float4_t s[NQ][2];
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
@@ -203,16 +223,19 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
                         }
                     }
                 }
+            }
+            if (have_prev) pv((it + 2) % 3, pa_prev, pl_prev);           // tile it - 1 sits in V buffer (it - 1) % 3
+            have_prev = active;
+            if (active) {
                 // ---- online softmax per query: this lane holds kv tokens tile + 16 sub + 4kg + i
                 float kn[8], vn[8];
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++) {
-                    const float4 k4 = *reinterpret_cast<const float4*>(&n_s[buf][0][16 * sub + 4 * kg]);
-                    const float4 v4 = *reinterpret_cast<const float4*>(&n_s[buf][1][16 * sub + 4 * kg]);
+                    const float4 k4 = *reinterpret_cast<const float4*>(&n_s[nbuf][0][16 * sub + 4 * kg]);
+                    const float4 v4 = *reinterpret_cast<const float4*>(&n_s[nbuf][1][16 * sub + 4 * kg]);
                     kn[4 * sub] = k4.x; kn[4 * sub + 1] = k4.y; kn[4 * sub + 2] = k4.z; kn[4 * sub + 3] = k4.w;
                     vn[4 * sub] = v4.x; vn[4 * sub + 1] = v4.y; vn[4 * sub + 2] = v4.z; vn[4 * sub + 3] = v4.w;
                 }
-                half8_t pa[NQ], pl[NQ];                        // p * vn as an fp16 value and its rounding remainder
 #pragma unroll
                 for (int nq = 0; nq < NQ; nq++) {
                     const int tq = q0 + 16 * nq + ln;
@@ -249,28 +272,18 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
                     for (int i = 0; i < 8; i++) {
                         const float p = __builtin_amdgcn_exp2f(x[i] - m_run[nq]);
                         l_run[nq] += p;
-                        const float pv = p * vn[i];                             // (s * vn) * centroid, kernels.cu:1765
-                        const half_t hi = (half_t)pv;
-                        pa[nq][i] = hi;
-                        pl[nq][i] = (half_t)(pv - (float)hi);
-                    }
-                }
-                // ---- O[query][dim 16j + ln] += P . V
-                const char* vrow = &v_s[buf][ln * kPtVRow + 16 * kg];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPtVRow);
-#pragma unroll
-                    for (int nq = 0; nq < NQ; nq++) {
-                        o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
-                        o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[nq], vb, o[nq][j], 0, 0, 0);
+                        const float pvn = p * vn[i];                            // (s * vn) * centroid, kernels.cu:1765
+                        const half_t hi = (half_t)pvn;
+                        pa_prev[nq][i] = hi;
+                        pl_prev[nq][i] = (half_t)(pvn - (float)hi);
                     }
                 }
             }
 
-            if (more) stash(buf ^ 1, st);
+            if (more) stash(buf ^ 1, (it + 1) % 3, st);
             __syncthreads();
         }
+        if (have_prev) pv((ntiles - 1) % 3, pa_prev, pl_prev);
 
         // ---- one partial per (query token, head): rotated accumulator, running maximum (base 2) and sum;
         // the merge normalises (kernels.cu:1946: 1 / (sum + 1e-8)) and rotates back.  Accumulator register i
