@@ -182,6 +182,14 @@ int tw_kv_profile_read(double* total_ms, int* launches);
  * the practical ceiling beside the published HBM peak.  Returns 0 on error. */
 double tw_kv_measure_read_bandwidth(const void* dev_buf, size_t bytes, int iters, hipStream_t s);
 
+/* Prefix sharing without one copy per (array, destination): rows [0, T) of sequence `src` go to the same
+ * rows of every sequence in [dst_begin, dst_end) (src itself skipped) for up to 4 arrays laid out
+ * (sequence, row, ...), in one launch.  bases[i]: device pointer of array i, seq_bytes[i]: bytes per sequence
+ * (rows per sequence * row bytes), bytes[i]: bytes to copy per sequence (T * row bytes).  Replaces the
+ * cudaMemcpyAsync loop of engine.cpp:2173-2214.  Returns 0, or -1 on bad arguments. */
+int tw_kv_broadcast_rows(void* const* bases, const size_t* seq_bytes, const size_t* bytes, int narrays,
+                         int src, int dst_begin, int dst_end, hipStream_t s);
+
 /* Floats of workspace the *_ws / paged attention entry points need for a
  * (G, num_heads, max_context) problem at the automatic split count.  The
  * reference-signature launchers instead fit their split count to the

@@ -1084,26 +1084,41 @@ def test_engine_stop_check_cadence():
     assert not finished[5] and finished[0] and outputs[0] == [int(x) for x in toks[:3, 0]]
 
 
-def test_engine_prefix_broadcast(oracle):
+@pytest.mark.parametrize("kv_bits,Hk", [(4, 2), (2, 1), (0, 2), (4, 8)])
+@pytest.mark.parametrize("src,dst", [(0, (1, 4)), (2, (0, 5)), (4, (1, 3))])
+def test_engine_prefix_broadcast(oracle, kv_bits, Hk, src, dst):
+    """Rows [0, T) of the source sequence reach every destination in all arrays of all layers (one launch per
+    layer); the source, sequences outside the range and rows from T on keep their bytes."""
     import torch
     from triebwerk_amd import Engine
-    r = gen.rng(600)
-    L, H, Hk, G, msl, T = 2, 4, 2, 4, 32, 7
-    kv_dim = Hk * D
-    eng = Engine(kv_bits=4)
+    L, H, G, msl, T = 2, 8, 5, 32, 7
+    eng = Engine(kv_bits=kv_bits)
     eng.set_shape(L, H, Hk, D)
     eng.alloc_batch(G, msl)
-    rot = eng.rotation()
-    rows = gen.normal_f16(r, (T, kv_dim))
-    c = eng.cache(0)
-    from triebwerk_amd import kvcache
-    positions = torch.arange(T, dtype=torch.int32, device="cuda")
-    kvcache.launch_turbo_kv_quantize(c[0][0], c[2][0], dev(rows), rot, positions, msl, T, Hk, D, kv_dim, 4)
-    eng.broadcast_prefix(0, 1, G, T)
-    k = host(c[0]); n = host(c[2])
-    for g in range(1, G):
-        assert np.array_equal(k[g, :T], k[0, :T]) and np.array_equal(n[g, :T], n[0, :T])
-        assert not k[g, T:].any()
+    gt = torch.Generator(device="cuda"); gt.manual_seed(600 + kv_bits)
+    before = []
+    for l in range(L):
+        arrs = []
+        for arr in eng.cache(l):
+            if arr is None:
+                continue
+            raw = arr.view(torch.uint8) if arr.dtype != torch.uint8 else arr
+            raw.copy_(torch.randint(0, 256, raw.shape, generator=gt, device="cuda", dtype=torch.uint8))
+            arrs.append(host(raw).copy())
+        before.append(arrs)
+    eng.broadcast_prefix(src, dst[0], dst[1], T)
+    torch.cuda.synchronize()
+    for l in range(L):
+        live = [a for a in eng.cache(l) if a is not None]
+        assert len(live) == (2 if kv_bits == 0 else 4)
+        for arr, was in zip(live, before[l]):
+            now = host(arr.view(torch.uint8) if arr.dtype != torch.uint8 else arr)
+            for g in range(G):
+                if dst[0] <= g < dst[1] and g != src:
+                    assert np.array_equal(now[g, :T], was[src, :T]), (l, g)
+                    assert np.array_equal(now[g, T:], was[g, T:]), (l, g)
+                else:
+                    assert np.array_equal(now[g], was[g]), (l, g)
 
 
 def test_plain_read_bandwidth_probe(kv):

@@ -64,6 +64,7 @@ SIGNATURES = {
     "tw_kv_profile_attention": (None, [I]),
     "tw_kv_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_kv_measure_read_bandwidth": (C.c_double, [P, C.c_size_t, I, P]),
+    "tw_kv_broadcast_rows": (I, [P, P, P, I, I, I, I, P]),
     "tw_attention_workspace_floats": (SZ, [I, I, I]),
     "tw_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_turbo_append_attention_batch": (None, [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),

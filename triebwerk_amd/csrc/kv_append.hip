@@ -192,4 +192,42 @@ void launch_increment(int* positions, int G, hipStream_t s) {
     hipLaunchKernelGGL(increment_positions_kernel, dim3((G + 255) / 256), dim3(256), 0, s, positions, G);
 }
 
+// ---------------------------------------------------------------- prefix broadcast
+// The first T rows of one sequence's arrays copied to the same rows of other sequences: the
+// reference's prefill-once-then-broadcast (engine.cpp:2173-2214) does it with one device-to-device
+// copy per (layer, array, destination); here one launch takes up to four arrays and every destination.
+// blockIdx.y = destination slot, blockIdx.z = array; the x blocks stride over the array's bytes.
+template <typename W>
+__global__ void __launch_bounds__(256)
+broadcast_rows_kernel(BroadcastArgs a) {
+    const int which = blockIdx.z;
+    int g = a.dst_begin + blockIdx.y;
+    if (a.src >= a.dst_begin && a.src < a.dst_end && g >= a.src) g++;   // destination slots skip the source
+    const size_t n = a.bytes[which] / sizeof(W);
+    const W* from = reinterpret_cast<const W*>(a.base[which] + (size_t)a.src * a.seq_bytes[which]);
+    W* to = reinterpret_cast<W*>(a.base[which] + (size_t)g * a.seq_bytes[which]);
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) to[i] = from[i];
+}
+
+void launch_broadcast_rows(const BroadcastArgs& a, hipStream_t s) {
+    int ndst = a.dst_end - a.dst_begin;
+    if (a.src >= a.dst_begin && a.src < a.dst_end) ndst--;
+    if (ndst <= 0 || a.narrays <= 0) return;
+    size_t most = 0;
+    unsigned align = 0;
+    for (int w = 0; w < a.narrays; w++) {
+        most = a.bytes[w] > most ? a.bytes[w] : most;
+        align |= (unsigned)(reinterpret_cast<uintptr_t>(a.base[w]) | a.seq_bytes[w] | a.bytes[w]);
+    }
+    if (most == 0) return;
+    const int width = (align & 15u) == 0 ? 16 : ((align & 3u) == 0 ? 4 : 2);    // rows are fp16 at least
+    size_t blocks = (most / width + 255) / 256;
+    if (blocks > 64) blocks = 64;                          // a block copies up to 4 KB per pass
+    if (blocks < 1) blocks = 1;
+    dim3 grid((unsigned)blocks, (unsigned)ndst, (unsigned)a.narrays);
+    if (width == 16) hipLaunchKernelGGL(broadcast_rows_kernel<uint4>, grid, dim3(256), 0, s, a);
+    else if (width == 4) hipLaunchKernelGGL(broadcast_rows_kernel<uint32_t>, grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(broadcast_rows_kernel<uint16_t>, grid, dim3(256), 0, s, a);
+}
+
 }  // namespace twkv

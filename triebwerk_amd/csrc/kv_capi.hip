@@ -251,6 +251,30 @@ double tw_kv_measure_read_bandwidth(const void* dev_buf, size_t bytes, int iters
     return gbps;
 }
 
+int tw_kv_broadcast_rows(void* const* bases, const size_t* seq_bytes, const size_t* bytes, int narrays,
+                         int src, int dst_begin, int dst_end, hipStream_t s) {
+    if (!bases || !seq_bytes || !bytes || narrays < 0 || narrays > 4 || src < 0 || dst_begin < 0 || dst_end < dst_begin) {
+        set_error(1, "tw_kv_broadcast_rows: bad arguments");
+        return -1;
+    }
+    BroadcastArgs b{};
+    b.src = src; b.dst_begin = dst_begin; b.dst_end = dst_end;
+    for (int i = 0; i < narrays; i++) {
+        if (!bases[i] || bytes[i] > seq_bytes[i] || ((reinterpret_cast<uintptr_t>(bases[i]) | seq_bytes[i] | bytes[i]) & 1u)) {
+            set_error(1, "tw_kv_broadcast_rows: arrays must be fp16-aligned and T rows must fit a sequence");
+            return -1;
+        }
+        if (bytes[i] == 0) continue;
+        b.base[b.narrays] = static_cast<char*>(bases[i]);
+        b.seq_bytes[b.narrays] = seq_bytes[i];
+        b.bytes[b.narrays] = bytes[i];
+        b.narrays++;
+    }
+    launch_broadcast_rows(b, s);
+    check_launch("tw_kv_broadcast_rows");
+    return 0;
+}
+
 size_t tw_attention_workspace_floats(int G, int num_heads, int max_context) {
     (void)max_context;
     return (size_t)G * num_heads * kPagedBlockFloats;

@@ -467,19 +467,21 @@ int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end
     s = pick(e, s);
     const size_t msl = (size_t)e->batch_msl;
     for (int l = 0; l < e->shape.num_layers; l++) {
+        void* bases[4];
+        size_t seq_bytes[4], bytes[4];
+        int n = 0;
         for (int which = 0; which < 4; which++) {
-            char* base = (char*)e->cache[l][which];
-            if (!base) continue;
+            if (!e->cache[l][which]) continue;
             size_t row_bytes;
             if (e->kv_bits == 0) row_bytes = (size_t)e->kv_dim() * 2;
             else row_bytes = which < 2 ? e->kv_dim_packed() : (size_t)e->shape.num_kv_heads * 2;
-            for (int g = dst_begin; g < dst_end; g++) {
-                if (g == src) continue;
-                if (hipMemcpyAsync(base + g * msl * row_bytes, base + src * msl * row_bytes,
-                                   (size_t)T * row_bytes, hipMemcpyDeviceToDevice, s) != hipSuccess)
-                    return -2;
-            }
+            bases[n] = e->cache[l][which];
+            seq_bytes[n] = msl * row_bytes;
+            bytes[n] = (size_t)T * row_bytes;
+            n++;
         }
+        // one launch per layer: every array, every destination
+        if (tw_kv_broadcast_rows(bases, seq_bytes, bytes, n, src, dst_begin, dst_end, s) != 0) return -2;
     }
     return 0;
 }

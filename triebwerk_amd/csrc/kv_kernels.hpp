@@ -46,6 +46,17 @@ void launch_kv_write(half_t* ck, half_t* cv, const half_t* k, const half_t* v,
 void launch_turbo_quantize(const QuantArgs& a, int bits, hipStream_t s);
 void launch_increment(int* positions, int G, hipStream_t s);
 
+// Rows [0, T) of sequence `src` copied to sequences [dst_begin, dst_end) (src itself skipped) in up to four
+// arrays that are laid out (sequence, row, ...): bytes = T * row bytes, seq_bytes = rows per sequence * row bytes.
+struct BroadcastArgs {
+    char* base[4];
+    size_t seq_bytes[4];
+    size_t bytes[4];
+    int narrays;
+    int src, dst_begin, dst_end;
+};
+void launch_broadcast_rows(const BroadcastArgs& a, hipStream_t s);
+
 // ---------------------------------------------------------------- producers of q and k (kv_producer.hip)
 struct ProducerArgs {
     half_t* q;               // (rows, q_stride), transformed in place
