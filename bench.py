@@ -197,6 +197,9 @@ def main():
     ap.add_argument("--kv-bits", type=int, default=None, choices=[0, 2, 4])
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 vector-ALU kernel, 2 MFMA kernel")
     ap.add_argument("--nsplit", type=int, default=0)
+    ap.add_argument("--one-launch", type=int, default=None, choices=[0, 1, 2],
+                    help="decode step of a compressed layer as one kernel: 0 by max_seq_len, 1 whenever possible, 2 never "
+                         "(default: what the engine picks from the spread of the context lengths)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--producers", default="none", choices=["none", "fused", "separate"],
@@ -251,6 +254,8 @@ def main():
     lib = _lib.load()
     torch.cuda.set_device(0)
     kvcache.set_attention_variant(args.variant)
+    if args.one_launch is not None:
+        kvcache.set_decode_fused(args.one_launch)
     kvcache.set_num_splits(args.nsplit)
     eng = Engine(max_seq_len=msl, kv_bits=kv_bits)
     eng.set_shape(L, H, Hk, D)

@@ -168,6 +168,14 @@ void tw_kv_set_num_splits(int nsplit);
  * per wave with mirrored pairs, 4 = compressed cache only: the kernel that expands tiles per wave). */
 void tw_kv_set_prefill_form(int form);
 
+/* tw_turbo_append_attention_batch and the calls built on it can run a layer's decode step as ONE kernel
+ * (append, query rotation, scan, merge, rotate-back; a workgroup owns a sequence's heads) instead of three.
+ * 0 (default): when the contexts are short (by max_seq_len, or by tw_layer_step_args::ctx_max), where launches
+ * dominate, and when ctx_min / ctx_max say the lengths are alike and the batch fills the GPU -- one sequence is one
+ * workgroup's work however long it is; 1: whenever the shape allows it (contiguous compressed cache, GQA group 1, 2
+ * or 4); 2: never.  Process-wide. */
+void tw_kv_set_decode_fused(int mode);
+
 /* Timing of the context-scanning attention kernel alone, with HIP events
  * recorded on the launch stream around that kernel (not around the merge).
  * Enable, run eager launches (not under stream capture; at most 4096 are
@@ -270,6 +278,8 @@ typedef struct tw_layer_step_args {
     float* scratch;            /* G*num_heads*max_seq_len floats */
     const tw_half* gate;       /* row g at gate + g*gate_stride, laid out like a row of out; NULL = none */
     long long gate_stride;
+    int ctx_min, ctx_max;      /* what the host knows of min and max over g of positions[g] + 1; 0, 0 = nothing.
+                                * Only steers the choice between kernels (tw_kv_set_decode_fused), never results. */
 } tw_layer_step_args;
 void tw_layer_attention_step(const tw_layer_step_args* args, hipStream_t s);
 

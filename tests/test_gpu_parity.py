@@ -406,6 +406,41 @@ def test_fused_append_attention_equals_two_calls(kv, oracle, rotation_fixture, b
     assert rel_err(host(out), want) <= TOL
 
 
+@pytest.mark.parametrize("mode", [1, 2])
+@pytest.mark.parametrize("bits", [4, 2])
+@pytest.mark.parametrize("H,Hk,lens", [
+    (16, 8, [0, 1, 31, 32, 33, 511, 512, 513, 1023, 1500, 2047]),          # every tile edge, 11 sequences
+    (32, 8, [5, 64, 700, 1299, 95, 96, 97, 1, 0, 255, 256, 257, 640, 641, 2, 1111]),   # GQA 4, 16 sequences
+    (4, 4, [40, 0, 1000]),                                                   # no grouping, 4 KV heads
+    (4, 2, [3, 77, 1999]), (2, 1, [130, 12]), (8, 2, [300, 301, 1024])])     # few KV heads
+def test_decode_step_in_one_launch(kv, oracle, rotation_fixture, bits, H, Hk, lens, mode):
+    """tw_turbo_append_attention_batch as one kernel (mode 1) and as three (mode 2): the appended rows equal the
+    oracle's bytes, the rest of the cache is untouched, outputs within tolerance of oracle append + attention."""
+    import torch
+    r = gen.rng(900 + bits + H + Hk)
+    G, msl = len(lens), 2048
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits)
+    pos = np.array(lens, np.int32)
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    d_ck, d_cv, d_kn, d_vn = dev(ck), dev(cv), dev(kn), dev(vn)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.set_decode_fused(mode)
+    try:
+        kv.tw_turbo_append_attention_batch(out, dev(q), dev(k), dev(v), d_ck, d_cv, d_kn, d_vn, dev(rotation_fixture),
+                                           scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    finally:
+        kv.set_decode_fused(0)
+    oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(cv, vn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    assert_bytes_equal(host(d_ck), ck, "K codes"); assert_bytes_equal(host(d_cv), cv, "V codes")
+    assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+    assert rel_err(host(out), want) <= TOL
+
+
 @pytest.mark.parametrize("bits", [4, 2])
 def test_turbo_attention_single_and_tiny_scratch(kv, oracle, rotation_fixture, bits):
     """Single-sequence entry point; max_seq_len 40 leaves no room for split partials."""

@@ -27,7 +27,7 @@ class LayerStepArgs(C.Structure):
                 ("q_weight", P), ("k_weight", P), ("eps", C.c_float), ("biased", I),
                 ("cos_table", P), ("sin_table", P), ("rope_dim", I),
                 ("kv_bits", I), ("cache_k", P), ("cache_v", P), ("k_norms", P), ("v_norms", P), ("rotation", P),
-                ("scratch", P), ("gate", P), ("gate_stride", LL)]
+                ("scratch", P), ("gate", P), ("gate_stride", LL), ("ctx_min", I), ("ctx_max", I)]
 
 
 class ModelShape(C.Structure):
@@ -61,6 +61,7 @@ SIGNATURES = {
     "tw_kv_get_attention_variant": (I, []),
     "tw_kv_set_num_splits": (None, [I]),
     "tw_kv_set_prefill_form": (None, [I]),
+    "tw_kv_set_decode_fused": (None, [I]),
     "tw_kv_profile_attention": (None, [I]),
     "tw_kv_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_kv_measure_read_bandwidth": (C.c_double, [P, C.c_size_t, I, P]),

@@ -17,6 +17,7 @@
 using namespace twkv;
 
 namespace twkv {
+static std::atomic<int> g_decode_fused{0};   // tw_kv_set_decode_fused: 0 by context bound, 1 whenever possible, 2 never
 static std::atomic<int> g_prefill_form{0};   // test hook, see prefill_form()
 int prefill_form() { return g_prefill_form.load(); }
 thread_local hipEvent_t t_scan_start = nullptr;
@@ -138,9 +139,11 @@ struct Profiler {
 // rotates the query together with the appended rows).
 bool mfma_wanted(const AttnArgs& a) { return a.bits != 0 && g_variant.load() != 1; }
 
-void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done = false) {
+// When the profiler is on (and the stream is not capturing: events cannot ride on a launch that is only being
+// recorded into a graph) the next scan launch on this thread carries a pair of its events (launch_scan_kernel).
+void attach_profiler(hipStream_t s) {
     bool prof = g_prof.enabled.load() != 0 && g_prof.used < kProfSlots;
-    if (prof) {   // events cannot ride on a launch that is only being recorded into a graph
+    if (prof) {
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone) prof = false;
     }
@@ -151,8 +154,11 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done =
             g_prof.created++;
         }
     }
-    // the scan kernel carries the profiler's events itself (see launch_scan_kernel)
     if (prof) { t_scan_start = g_prof.start[g_prof.used]; t_scan_stop = g_prof.stop[g_prof.used]; g_prof.used++; }
+}
+
+void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done = false) {
+    attach_profiler(s);
     if (a.bits == 0 && g_variant.load() != 1 && prefill_f16_mfma_usable(a)) {   // fp16 prefill: one MFMA kernel, no splits
         launch_prefill_f16_mfma(a, s, g_prefill_form.load());
         t_scan_start = t_scan_stop = nullptr;
@@ -187,6 +193,7 @@ void tw_kv_set_attention_variant(int v) { g_variant.store(v); }
 int tw_kv_get_attention_variant(void) { return g_variant.load(); }
 void tw_kv_set_num_splits(int n) { g_nsplit_override.store(n); }
 void tw_kv_set_prefill_form(int form) { g_prefill_form.store(form); }
+void tw_kv_set_decode_fused(int mode) { g_decode_fused.store(mode); }
 
 void tw_kv_profile_attention(int enable) {
     g_prof.enabled.store(enable);
@@ -500,6 +507,50 @@ void launch_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const uint
     run_attention(a, s, "launch_turbo_gqa_attention_batch");
 }
 
+// Range of positions + 1 over the batch as far as the caller of tw_layer_attention_step knows it on the host
+// (0, 0 = unknown), for the call being set up on this thread.
+static thread_local int t_ctx_min = 0;
+static thread_local int t_ctx_max = 0;
+
+// The whole step in one launch (kv_decode_fused.hip)?  There one workgroup owns a sequence's heads from the first
+// token to the last: it saves two launches and the scan's ramp (~10 us of a layer) and loses to the three-kernel
+// path where that one's balanced walk or its row-wise loads matter.  Taken when
+//   - every wave gets at most 8 tiles (launch-bound whatever the spread of the lengths), or
+//   - the lengths are known to be within 1/8 of each other and the batch gives at least half the CUs a workgroup,
+//     up to the size where the three-kernel path's better streaming rate has made up for its start-up
+//     (measured on MI355X: 4 bit ~1M tokens per launch; 2 bit with 8 KV heads, where the three-kernel path
+//     loads whole rows cooperatively, ~256k).
+// false = not taken.
+static bool try_decode_fused(const AttnArgs& a, const tw_half* k_buf, const tw_half* v_buf, int kv_dim,
+                             uint8_t* ck_q, uint8_t* cv_q, tw_half* k_norms, tw_half* v_norms, int msl,
+                             hipStream_t s, const char* fn) {
+    const int mode = g_decode_fused.load();
+    if (mode == 2 || g_variant.load() == 1) return false;
+    FusedArgs f;
+    memset(&f, 0, sizeof(f));
+    f.k_src = H(k_buf); f.v_src = H(v_buf); f.kv_stride = kv_dim;
+    f.k_codes = ck_q; f.v_codes = cv_q; f.k_norms = H(k_norms); f.v_norms = H(v_norms);
+    if (!decode_fused_usable(a, f)) return false;
+    if (mode == 0) {
+        const int hkw = decode_fused_heads_per_workgroup(a.G, a.num_kv_heads);
+        const int split = 16 / hkw;
+        const long long units = (long long)a.G * (a.num_kv_heads / hkw);
+        const bool known = t_ctx_max > 0;
+        const int bound = known ? t_ctx_max : msl;
+        bool take = bound <= 256 * split;
+        if (!take && known && (long long)(t_ctx_max - t_ctx_min) * 8 <= t_ctx_max && units * 2 >= compute_units_host()) {
+            const long long tokens = (long long)a.G * t_ctx_max;
+            take = tokens <= ((a.bits == 2 && a.num_kv_heads == 8) ? (256LL << 10) : (1LL << 20));
+        }
+        if (!take) return false;
+    }
+    attach_profiler(s);
+    launch_decode_fused(a, f, s);
+    t_scan_start = t_scan_stop = nullptr;
+    check_launch(fn);
+    return true;
+}
+
 void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf,
                                      const tw_half* v_buf, uint8_t* ck_q, uint8_t* cv_q,
                                      tw_half* k_norms, tw_half* v_norms, const tw_half* rotation,
@@ -516,6 +567,7 @@ void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_ha
     fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads,
                 num_kv_heads, bits, as);
     a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    if (try_decode_fused(a, k_buf, v_buf, kv_dim, ck_q, cv_q, k_norms, v_norms, msl, s, fn)) return;
     plan_splits(a, msl, msl);
     // one rotation launch for the appended K and V rows and, when the MFMA scan will run,
     // for the query as well
@@ -730,6 +782,8 @@ void tw_layer_attention_step(const tw_layer_step_args* p, hipStream_t s) {
     const bool producers = p->q_weight || p->cos_table;
     t_gate = p->gate;
     t_gate_stride = p->gate ? p->gate_stride : 0;
+    t_ctx_min = p->ctx_max > 0 ? p->ctx_min : 0;
+    t_ctx_max = p->ctx_max > 0 ? p->ctx_max : 0;
     if (p->kv_bits == 0) {
         if (producers) {
             tw_qk_norm_rope_append_attention_batch(p->out, p->q, p->k, p->v, p->q_weight, p->k_weight, p->eps, p->biased,
@@ -756,6 +810,7 @@ void tw_layer_attention_step(const tw_layer_step_args* p, hipStream_t s) {
     }
     t_gate = nullptr;
     t_gate_stride = 0;
+    t_ctx_min = t_ctx_max = 0;
 }
 
 void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const uint8_t* ck_q,

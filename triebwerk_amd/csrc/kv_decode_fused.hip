@@ -1,0 +1,627 @@
+// kv_decode_fused.hip -- one decode step of one layer over the compressed cache in ONE launch (gfx950):
+// append K and V of the new token (turbo_kv_quantize_batch_kernel, kernels.cu:1563-1636), rotate the query
+// (1671-1681), scan the context (1688-1766), merge the parts of the context, normalise and rotate back
+// (1746, 1769-1775).  forward_layer_batch does this with three launches (engine.cpp:1985-2006) and the
+// three-kernel path of this library (rotate_kernel, attention_mfma_kernel, merge_rotate_kernel) does too;
+// each of those small launches costs ~4.5 us before it does anything and the scan another ~6 us to start
+// and drain, which is a third of a layer at contexts of a few hundred tokens.
+//
+// A workgroup of 16 waves owns one sequence and HKW of its KV heads (HKW = 1, 2, 4 or 8) together with
+// their query heads, so nothing is handed from one workgroup to another:
+//   1. waves 0-7 (all 16 when the unit has more than 16 vectors) rotate the unit's vectors exactly as
+//      rotate_kernel does -- lane i16 = vector (K heads, V heads, query heads), wave = block of 16 output
+//      coordinates, the same v_mfma_f32_16x16x4_f32 chain, so the codes have the same bits -- and store
+//      codes and norms in the cache, the scaled q_rot in LDS; meanwhile every thread fills its piece of the
+//      centroid table;
+//   2. after the barrier wave w scans part w / HKW of the context for head w % HKW with the loop of
+//      attention_mfma_kernel (the table look-ups, MFMA tiling, online softmax are described there).  Loads of
+//      a tile that holds the new token's row are only issued after the barrier (the row was stored by this
+//      workgroup: same CU, same L1); tiles before it are requested up front;
+//   3. the partial results meet in LDS: merge (log-sum-exp), "+1e-8" normalisation, and R^T with the MFMA
+//      chain of merge_rotate_kernel; output gate as there.
+// The waves in the upper wave slots of a CU run ~5 % slower (see kv_common.hpp: kPairShare), so the parts
+// of the upper eight waves get 31/64 of the tiles.
+//
+// One sequence is one workgroup's work whatever its length: right for batches of similar lengths (a
+// rollout's decode steps) and for short contexts; the three-kernel path with its balanced walk stays the
+// choice for ragged long contexts, and the only one for the paged layout.
+
+#include "kv_common.hpp"
+#include "kv_kernels.hpp"
+#include "kv_mfma_util.hpp"
+
+namespace twkv {
+
+namespace {
+
+constexpr int kFusedWaves = 16;
+constexpr int kFusedMaxQ = 32;                 // query heads of a unit: HKW * R <= 8 * 4
+constexpr int kRowFloats = kHeadDim + 4;       // LDS row of a vector: conflict-free 16-byte accesses
+constexpr int kStageStride = 2 * kHeadDim + 16;   // bytes per staged fp16 vector
+static_assert(8 * (2 + 4) * kStageStride <= kFusedMaxQ * kRowFloats * 4, "staged vectors fit the output rows");
+
+__device__ __forceinline__ float pick_half16(const uint4& piece, int e, int kk) {
+    uint32_t lo = e ? piece.z : piece.x;
+    uint32_t hi = e ? piece.w : piece.y;
+    uint32_t w = (kk & 2) ? hi : lo;
+    w = (kk & 1) ? (w >> 16) : (w & 0xffffu);
+    union { uint16_t u; half_t h; } cv;
+    cv.u = (uint16_t)w;
+    return (float)cv.h;
+}
+
+}  // namespace
+
+template <int R, int BITS>
+__global__ void __launch_bounds__(kFusedWaves * kWave)
+decode_fused_kernel(AttnArgs a, FusedArgs f) {
+    constexpr int KW = BITS, VW = BITS;
+    constexpr uint32_t kHeadBytes = BITS * 16;
+    constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
+    __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
+    __shared__ __attribute__((aligned(16))) half_t p_s[kFusedWaves][16][32];
+    __shared__ __attribute__((aligned(16))) float qrot_s[kFusedMaxQ][kHeadDim];
+    __shared__ __attribute__((aligned(16))) float part_s[kFusedWaves][R][kRowFloats];
+    __shared__ __attribute__((aligned(16))) float o_s[kFusedMaxQ][kRowFloats];
+
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid / kWave), lane = tid % kWave;
+    const int ln = lane & 15, kg = lane >> 4;          // names of the scan; the rotations call them i16, kk
+    const int Hk = a.num_kv_heads;
+    const int HKW = f.hkw;
+    const int nhg = Hk / HKW;
+    const int SPLIT = kFusedWaves / HKW;
+
+    // ---- unit of this workgroup.  Workgroups are dealt to the 8 XCDs in turn; the units of one sequence
+    // go to one XCD so that the norm rows they all read (16 bytes per token for 8 heads) come out of one L2.
+    int g, hg;
+    {
+        const int b = (int)blockIdx.x;
+        if ((a.G & 7) == 0) {
+            const int xcd = b & 7, j = b >> 3;
+            g = (j / nhg) * 8 + xcd;
+            hg = j % nhg;
+        } else {
+            g = b / nhg;
+            hg = b % nhg;
+        }
+    }
+    // ---- operands of the rotations first: nothing about them depends on the position.  The unit's vectors
+    // (K heads, V heads, query heads) are fetched once by all threads, 16 bytes each, and staged in LDS;
+    // the rotating waves fetch their 16 rows of R.
+    const int nvec = HKW * (2 + R);
+    const int rot_dblk = wave & 7;
+    const bool rotating = (wave >> 3) * 16 < nvec;
+    auto unit_vector = [&](int vc, int& kind, int& head) -> const half_t* {    // vc < nvec
+        if (vc < HKW) {
+            kind = 0; head = hg * HKW + vc;
+            return f.k_src + (long long)g * f.kv_stride + (long long)head * kHeadDim;
+        }
+        if (vc < 2 * HKW) {
+            kind = 1; head = hg * HKW + vc - HKW;
+            return f.v_src + (long long)g * f.kv_stride + (long long)head * kHeadDim;
+        }
+        kind = 2; head = hg * HKW * R + (vc - 2 * HKW);
+        return a.q + (long long)g * a.q_stride + (long long)head * kHeadDim;
+    };
+    uint4 stage = {0u, 0u, 0u, 0u};                    // piece tid % 16 of vector tid / 16
+    if ((tid >> 4) < nvec) {
+        int kind0, head0;
+        stage = reinterpret_cast<const uint4*>(unit_vector(tid >> 4, kind0, head0))[tid & 15];
+    }
+    float rv[32];                                      // R[16 * rot_dblk + ln][4s + kg]
+    if (rotating) {
+        const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (rot_dblk * 16 + ln) * kHeadDim);
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            uint4 rp = rsrc[q];
+            rv[2 * q] = pick_half16(rp, 0, kg);
+            rv[2 * q + 1] = pick_half16(rp, 1, kg);
+        }
+    }
+
+    const int pos = uniform(a.positions[g]);
+    const int n = pos + 1;
+    const int hk_local = wave % HKW, part = wave / HKW;
+    const int h = hg * HKW + hk_local;                 // KV head of this wave
+
+    // ---- part of the context this wave scans: 32-token tiles, lower waves 33/64 of them
+    int t0, t1;
+    {
+        const int ntile = (n + 31) >> 5;
+        const int halfparts = SPLIT >> 1;              // SPLIT is 2, 4, 8 or 16
+        const int lower = min(ntile, (int)((ntile * kPairShare + 63u) / 64u));
+        int b0, b1;
+        if (part < halfparts) {
+            b0 = lower * part / halfparts;
+            b1 = lower * (part + 1) / halfparts;
+        } else {
+            const int up = ntile - lower, pp = part - halfparts;
+            b0 = lower + up * pp / halfparts;
+            b1 = lower + up * (pp + 1) / halfparts;
+        }
+        t0 = 32 * b0;
+        t1 = min(32 * b1, n);
+    }
+    const int ntiles = t1 > t0 ? (t1 - t0 + 31) >> 5 : 0;
+
+    // ---- scan set-up (as attention_mfma_kernel, contiguous layout)
+    const char* tab_lane = reinterpret_cast<const char*>(tab_s);
+    const uint32_t lane_rep = BITS == 4 ? (uint32_t)lane * 4u : (uint32_t)(lane & 31) * 8u;
+    const uint32_t kvp = (uint32_t)Hk * kHeadBytes;
+    const uint32_t nrow = (uint32_t)Hk * 2u;
+    const uint32_t koff = (uint32_t)(lane >> 2) * kvp + (kHeadBytes / 4) * (uint32_t)(lane & 3);
+    const int ksrc = 4 * (4 * ln + kg);
+    uint32_t voff[VW];
+#pragma unroll
+    for (int i = 0; i < VW; i++) {
+        if (BITS == 4) voff[i] = (uint32_t)(4 * kg + i) * kvp + 4u * (uint32_t)ln;
+        else voff[i] = (uint32_t)(4 * kg + 2 * i + (ln & 1)) * kvp + 4u * (uint32_t)(ln >> 1);
+    }
+    const bool odd = (ln & 1) != 0;
+    const uint32_t sel_keep = odd ? 0x07060302u : 0x05040100u;
+    const uint32_t sel_send = odd ? 0x05040100u : 0x07060302u;
+    const uint32_t sub_bytes = 16u * kvp;
+    const int my_sub = kg >> 1;
+    const bool useful = (kg & 1) == 0;
+    const uint32_t noff = (uint32_t)ln * nrow + (uint32_t)my_sub * 16u * nrow;
+    half_t* p_w = &p_s[wave][0][8 * (ln >> 2) + 4 * my_sub + (ln & 3)];
+    const uint4* p_r = reinterpret_cast<const uint4*>(&p_s[wave][ln][8 * kg]);
+    constexpr float kRaise = 5.0f;
+
+    auto lut32 = [&](uint32_t addr) -> uint32_t { return *reinterpret_cast<const uint32_t*>(tab_lane + addr); };
+    auto lut64 = [&](uint32_t addr) -> uint2 { return *reinterpret_cast<const uint2*>(tab_lane + addr); };
+
+    const long long seq_row0 = (long long)g * a.seq_stride_rows;
+    const char* kseq = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes;
+    const char* vseq = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes;
+    const char* knseq = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
+    const char* vnseq = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
+
+    auto load_k = [&](__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t (&dst)[KW]) {
+        if constexpr (BITS == 4) {
+            uint32x4_t q = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+            dst[0] = q[0]; dst[1] = q[1]; dst[2] = q[2]; dst[3] = q[3];
+        } else {
+            uint32x2_t q = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
+            dst[0] = q[0]; dst[1] = q[1];
+        }
+    };
+    // Descriptors span the rows of the tile that exist (rows past the sequence's end read as zeros).
+    auto issue_k = [&](uint32_t (&kreg)[2][KW], int tile) {
+        __amdgpu_buffer_rsrc_t r = make_rsrc(kseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
+        load_k(r, koff, kreg[0]);
+        load_k(r, koff + sub_bytes, kreg[1]);
+    };
+    auto issue_v = [&](uint32_t (&vreg)[2][VW], int tile) {
+        __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+            for (int i = 0; i < VW; i++)
+                vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)(voff[i] + sub * sub_bytes), 0, 0);
+        }
+    };
+    auto pick = [&](const uint32x4_t& q) -> uint32_t {
+        const int dw = (h & 7) >> 1;
+        uint32_t w = dw == 0 ? q[0] : dw == 1 ? q[1] : dw == 2 ? q[2] : q[3];
+        return (h & 1) ? (w >> 16) : (w & 0xffffu);
+    };
+    auto issue_n = [&](int tile) -> uint32_t {        // fp16 bits of kn (low) and vn (high) of this lane's token
+        const bool wide = (nrow & 15u) == 0;
+        const uint32_t hgrp = (uint32_t)(h >> 3) * 16u;
+        const long long row = seq_row0 + tile;
+        const int rows = max(min(n - tile, 32), 0);
+        if (wide) {
+            __amdgpu_buffer_rsrc_t rk = make_rsrc(reinterpret_cast<const char*>(a.k_norms) + row * nrow, rows * (int)nrow);
+            __amdgpu_buffer_rsrc_t rv = make_rsrc(reinterpret_cast<const char*>(a.v_norms) + row * nrow, rows * (int)nrow);
+            uint32x4_t kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
+            if (useful) {
+                kq = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)(noff + hgrp), 0, 0);
+                vq = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)(noff + hgrp), 0, 0);
+            }
+            return pick(kq) | (pick(vq) << 16);
+        }
+        __amdgpu_buffer_rsrc_t rk = make_rsrc(knseq + row * nrow, rows * (int)nrow);
+        __amdgpu_buffer_rsrc_t rv = make_rsrc(vnseq + row * nrow, rows * (int)nrow);
+        uint32_t kk = __builtin_amdgcn_raw_buffer_load_b16(rk, (int)noff, 0, 0);
+        uint32_t vv = __builtin_amdgcn_raw_buffer_load_b16(rv, (int)noff, 0, 0);
+        return kk | (vv << 16);
+    };
+
+    uint32_t kreg[2][KW];
+    uint32_t vreg[2][VW];
+    uint32_t nreg = 0;
+    // The first tile is requested now unless it holds the row this workgroup is about to store.
+    const bool early = ntiles > 0 && t0 + 32 < n;
+    if (early) {
+        issue_k(kreg, t0);
+        nreg = issue_n(t0);
+        issue_v(vreg, t0);
+    }
+
+    // ---- 1. rotations of the unit's vectors
+    {
+        const int i16 = ln, kk = kg;
+        const int dblk = rot_dblk;
+        // the centroid table while the loads are under way: entry e fills 256 bytes with replicas
+        for (int i = tid * 4; i < kTableWords; i += kFusedWaves * kWave * 4) {
+            const int e = i >> 6;
+            if constexpr (BITS == 4) {
+                half2_t p = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
+                uint32_t w = *reinterpret_cast<uint32_t*>(&p);
+                *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
+            } else {
+                half2_t p0 = {(half_t)(kAlpha * kCentroids2[e & 3]), (half_t)(kAlpha * kCentroids2[(e >> 4) & 3])};
+                half2_t p1 = {(half_t)(kAlpha * kCentroids2[(e >> 2) & 3]), (half_t)(kAlpha * kCentroids2[(e >> 6) & 3])};
+                uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
+                *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
+            }
+        }
+        for (int i = tid; i < kFusedWaves * 16 * 32 / 2; i += kFusedWaves * kWave) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
+
+        // the staged vectors: rows of kStageStride bytes (16-byte aligned; a lane group's 2-byte reads below
+        // fall into 32 different banks), in the space the merged outputs will use at the end
+        char* x_s = reinterpret_cast<char*>(o_s);
+        if ((tid >> 4) < nvec) *reinterpret_cast<uint4*>(x_s + (tid >> 4) * kStageStride + (tid & 15) * 16) = stage;
+        __syncthreads();
+
+        for (int vt = wave >> 3; vt * 16 < nvec; vt += 2) {       // uniform over the wave
+            const int vi = vt * 16 + i16;
+            const int vc = vi < nvec ? vi : nvec - 1;              // clamp reads, mask stores
+            int kind, head;
+            (void)unit_vector(vc, kind, head);
+            const bool is_query = kind == 2;
+            // B operand: coordinate 4s + kk of vector vc
+            float xv[32];
+            const half_t* xrow = reinterpret_cast<const half_t*>(x_s + vc * kStageStride) + kk;
+#pragma unroll
+            for (int s2 = 0; s2 < 32; s2++) xv[s2] = (float)xrow[4 * s2];
+            // sum of squares in the reference's order (kernels.cu:1509-1520), as rotate_kernel
+            float n2 = 0.0f;
+            {
+                float sgrp[4];
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    float t[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) t[j] = xv[8 * w + j] * xv[8 * w + j];
+                    float a0 = t[0] + t[4], a1 = t[1] + t[5], a2 = t[2] + t[6], a3 = t[3] + t[7];
+                    float b0 = a0 + a2, b1 = a1 + a3;
+                    float c = b0 + b1;
+                    float d = c + __shfl_xor(c, 32, 64);
+                    sgrp[w] = d + __shfl_xor(d, 16, 64);
+                }
+                n2 = (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
+            }
+            if (!is_query) {
+                const float inv = 1.0f / sqrtf(n2 + 1e-12f);
+#pragma unroll
+                for (int s = 0; s < 32; s++) xv[s] *= inv;
+            }
+            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 32; s++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(rv[s], xv[s], acc, 0, 0, 0);
+
+            if (is_query && vi < nvec) {
+                float4 o = {acc[0] * f.q_scale, acc[1] * f.q_scale, acc[2] * f.q_scale, acc[3] * f.q_scale};
+                *reinterpret_cast<float4*>(&qrot_s[vc - 2 * HKW][dblk * 16 + 4 * kk]) = o;
+            }
+            uint32_t packed = 0;
+#pragma unroll
+            for (int r = 0; r < 4; r++) packed |= (uint32_t)turbo_quantize(acc[r], BITS) << (r * BITS);
+            constexpr int PB = 4 * BITS;
+            uint32_t p1 = (uint32_t)__shfl((int)packed, i16 + 16, 64);
+            uint32_t p2 = (uint32_t)__shfl((int)packed, i16 + 32, 64);
+            uint32_t p3 = (uint32_t)__shfl((int)packed, i16 + 48, 64);
+            if (kk == 0 && vi < nvec && !is_query) {
+                constexpr int BPH = kHeadDim * BITS / 8;
+                const long long crow = seq_row0 + pos;
+                uint8_t* dst = (kind == 0 ? f.k_codes : f.v_codes) + (crow * Hk + head) * BPH + dblk * (2 * BITS);
+                if (BITS == 4) {
+                    uint2 o = {packed | (p1 << PB), p2 | (p3 << PB)};
+                    *reinterpret_cast<uint2*>(dst) = o;
+                } else {
+                    *reinterpret_cast<uint32_t*>(dst) = packed | (p1 << PB) | (p2 << (2 * PB)) | (p3 << (3 * PB));
+                }
+                if (dblk == 0) (kind == 0 ? f.k_norms : f.v_norms)[crow * Hk + head] = (half_t)sqrtf(n2 + 1e-12f);
+            }
+        }
+    }
+    __syncthreads();        // table, q_rot and the new cache row are in place
+
+    // ---- 2. scan of this wave's part
+    float4_t o[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run[R], l_run[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
+
+    if (ntiles > 0) {
+        if (!early) {
+            issue_k(kreg, t0);
+            nreg = issue_n(t0);
+            issue_v(vreg, t0);
+        }
+        // A operand of the score MFMAs: q_rot[head][32kg + 8j + i], row m = fp16 value of head m, row m + 8
+        // its rounding remainder; the 2-bit table returns the codes of a byte in the order 0,2,1,3
+        half8_t aq[4];
+        {
+            const int hq = ln & 7;
+            const bool lo_part = (ln & 8) != 0;
+            const float* qr = &qrot_s[hk_local * R + (hq < R ? hq : 0)][32 * kg];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
+                float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
+                float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int src = BITS == 4 ? i : ((i & 4) | ((i & 1) << 1) | ((i & 2) >> 1));
+                    float x = (hq < R) ? v[src] : 0.0f;
+                    half_t hi = (half_t)x;
+                    half_t lo = (half_t)(x - (float)hi);
+                    aq[j][i] = lo_part ? lo : hi;
+                }
+            }
+        }
+
+        for (int it = 0; it < ntiles; it++) {
+            const int tile = t0 + 32 * it;
+            const int next_tile = tile + 32;
+            const bool more = it + 1 < ntiles;
+
+            // ---- scores S[head][token] for both sub-tiles
+            float4_t s[2];
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                uint32_t kw[KW];
+#pragma unroll
+                for (int i = 0; i < KW; i++) kw[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(ksrc, (int)kreg[sub][i]);
+                union { uint32_t u[4]; half8_t h; } kv[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if constexpr (BITS == 4) {
+                        const uint32_t w = kw[j];
+                        kv[j].u[0] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0400u));
+                        kv[j].u[1] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0500u));
+                        kv[j].u[2] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0600u));
+                        kv[j].u[3] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0700u));
+                    } else {
+                        const uint32_t w = kw[j >> 1];
+                        const uint32_t sel = (j & 1) ? 0x0c0c0600u : 0x0c0c0400u;
+                        uint2 l0 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel));
+                        uint2 l1 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel + 0x100u));
+                        kv[j].u[0] = l0.x; kv[j].u[1] = l0.y; kv[j].u[2] = l1.x; kv[j].u[3] = l1.y;
+                    }
+                }
+                s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[sub], 0, 0, 0);
+            }
+            if (more) issue_k(kreg, next_tile);
+
+            // ---- online softmax (base 2): this lane owns token ln of sub-tile my_sub
+            const float kn = h2f_bits(nreg & 0xffffu), vn = h2f_bits(nreg >> 16);
+            if (more) nreg = issue_n(next_tile);
+            const bool valid = useful && (tile + 16 * my_sub + ln < t1);
+            float raw[R], x[R];
+            bool raise = false;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                uint32x2_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(s[0][r]), __float_as_uint(s[1][r]), false, false);
+                raw[r] = (__uint_as_float(sw[0]) + __uint_as_float(sw[1])) * kn;    // kernels.cu:1707
+                x[r] = valid ? raw[r] - m_run[r] : kNegBig;
+                raise = raise || (x[r] > kRaise);
+            }
+            if (__any(raise)) {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    float m_new = fmaxf(m_run[r], wave_max(valid ? raw[r] : kNegBig));
+                    float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                    m_run[r] = m_new;
+                    l_run[r] *= alpha;
+                    x[r] = valid ? raw[r] - m_new : kNegBig;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) o[j][r] *= alpha;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float p = __builtin_amdgcn_exp2f(x[r]);
+                l_run[r] += p;
+                float pf = p * vn;                                      // (s * vn) * centroid, kernels.cu:1765
+                half_t hi = (half_t)pf;
+                half_t lo = (half_t)(pf - (float)hi);
+                if (useful) {
+                    p_w[r * 32] = hi;
+                    p_w[(r + 8) * 32] = lo;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            union { uint4 q; half8_t h; } pa;
+            pa.q = *p_r;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+
+            // ---- O[head][dim 8ln + j] += P[head][token] V[token][dim]
+            if constexpr (BITS == 4) {
+                uint32_t xe[4], xo[4];
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                    for (int pr = 0; pr < 2; pr++) {
+                        uint32_t wa = vreg[sub][2 * pr], wb = vreg[sub][2 * pr + 1];
+                        xe[2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                        xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                    }
+                }
+                if (more) issue_v(vreg, next_tile);
+#pragma unroll
+                for (int jp = 0; jp < 4; jp++) {
+                    const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
+                    union { uint32_t u[4]; half8_t h; } be, bo;
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        be.u[q4] = lut32(__builtin_amdgcn_perm(xe[q4], lane_rep, sel));
+                        bo.u[q4] = lut32(__builtin_amdgcn_perm(xo[q4], lane_rep, sel));
+                    }
+                    o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * jp], 0, 0, 0);
+                    o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * jp + 1], 0, 0, 0);
+                }
+            } else {
+                uint32_t ie[2], io[2];
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+                    const uint32_t keep = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_keep);
+                    const uint32_t send = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_send);
+                    const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xf, 0xf, false);  // lane ^ 1
+                    const uint32_t wa = odd ? recv : keep, wb = odd ? keep : recv;
+                    ie[sub] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                    io[sub] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                }
+                if (more) issue_v(vreg, next_tile);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t x0 = (q & 1) ? io[0] : ie[0], x1 = (q & 1) ? io[1] : ie[1];
+                    const uint32_t sel = 0x0c0c0400u + ((uint32_t)(q >> 1) << 8);
+                    uint2 l00 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel));
+                    uint2 l01 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel + 0x200u));
+                    uint2 l10 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel));
+                    uint2 l11 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel + 0x200u));
+                    union { uint32_t u[4]; half8_t h; } be, bo;
+                    be.u[0] = l00.x; be.u[1] = l01.x; be.u[2] = l10.x; be.u[3] = l11.x;
+                    bo.u[0] = l00.y; bo.u[1] = l01.y; bo.u[2] = l10.y; bo.u[3] = l11.y;
+                    o[2 * q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * q], 0, 0, 0);
+                    o[2 * q + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * q + 1], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- 3. the parts meet in LDS.  B operand of the rotate-back first (its loads run under the merge):
+    // R[32kk + s][16*dblk + i16], s = 0..31
+    const int nv = HKW * R;                                  // output vectors of this unit
+    const int dblk = wave & 7;
+    const bool back = (wave >> 3) * 16 < nv;
+    uint16_t rb[32];
+    if (back) {
+        const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.rotation) + (32 * kg) * kHeadDim + 16 * dblk + ln;
+#pragma unroll
+        for (int s = 0; s < 32; s++) rb[s] = rp[s * kHeadDim];
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        l_run[r] = wave_sum(l_run[r]);
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j][r] += __shfl_xor(o[j][r], 32, 64);   // row r + row r+8 (lo part of P)
+    }
+    if (kg == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float* pr = &part_s[wave][r][0];
+            float4 lo4 = {o[0][r] * (1.0f / kAlpha), o[1][r] * (1.0f / kAlpha), o[2][r] * (1.0f / kAlpha), o[3][r] * (1.0f / kAlpha)};
+            float4 hi4 = {o[4][r] * (1.0f / kAlpha), o[5][r] * (1.0f / kAlpha), o[6][r] * (1.0f / kAlpha), o[7][r] * (1.0f / kAlpha)};
+            *reinterpret_cast<float4*>(pr + 8 * ln) = lo4;
+            *reinterpret_cast<float4*>(pr + 8 * ln + 4) = hi4;
+            if (ln == 0) { pr[kHeadDim] = m_run[r]; pr[kHeadDim + 1] = l_run[r]; }
+        }
+    }
+    __syncthreads();
+
+    {   // merge: thread -> (vector tid / 32, coordinates 4 * (tid % 32) .. +3); vector = (local KV head, query head)
+        const int vec = tid >> 5, k4 = (tid & 31) * 4;
+        float4 o4 = {0.f, 0.f, 0.f, 0.f};
+        if (vec < nv) {
+            const int hk_l = vec / R, r = vec - hk_l * R;
+            float mg = kNegBig;
+            for (int p = 0; p < SPLIT; p++) mg = fmaxf(mg, part_s[p * HKW + hk_l][r][kHeadDim]);
+            float lsum = 0.0f;
+            float4 av = {0.f, 0.f, 0.f, 0.f};
+            for (int p = 0; p < SPLIT; p++) {
+                const float* pr = &part_s[p * HKW + hk_l][r][0];
+                const float fs = __builtin_amdgcn_exp2f(pr[kHeadDim] - mg);
+                const float4 c = *reinterpret_cast<const float4*>(pr + k4);
+                lsum = __builtin_fmaf(pr[kHeadDim + 1], fs, lsum);
+                av.x = __builtin_fmaf(c.x, fs, av.x);
+                av.y = __builtin_fmaf(c.y, fs, av.y);
+                av.z = __builtin_fmaf(c.z, fs, av.z);
+                av.w = __builtin_fmaf(c.w, fs, av.w);
+            }
+            const float inv = 1.0f / (lsum + 1e-8f);             // kernels.cu:1746
+            o4 = float4{av.x * inv, av.y * inv, av.z * inv, av.w * inv};
+        }
+        *reinterpret_cast<float4*>(&o_s[vec][k4]) = o4;
+    }
+    __syncthreads();
+
+    // ---- out[vector][d] = sum_k o[vector][k] R[k][d]; lane group kk owns k in [32kk, 32kk+32)
+    for (int vt = wave >> 3; vt * 16 < nv; vt += 2) {
+        float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        const float* orow = &o_s[vt * 16 + ln][32 * kg];
+#pragma unroll
+        for (int s4 = 0; s4 < 8; s4++) {
+            float4 o4 = *reinterpret_cast<const float4*>(orow + 4 * s4);
+            const float ov[4] = {o4.x, o4.y, o4.z, o4.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                union { uint16_t u; half_t h; } cv;
+                cv.u = rb[4 * s4 + j];
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ov[j], (float)cv.h, acc, 0, 0, 0);
+            }
+        }
+        // lane holds out[vector vt*16 + 4kk + r][d = 16*dblk + i16]
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int vec = vt * 16 + 4 * kg + r;
+            if (vec < nv) {
+                const int head = hg * HKW * R + vec;
+                const long long col = (long long)head * kHeadDim + 16 * dblk + ln;
+                half_t hv = (half_t)acc[r];
+                if (a.gate) hv = gated(hv, a.gate[(long long)g * a.gate_stride + col]);
+                a.out[(long long)g * a.q_stride + col] = hv;
+            }
+        }
+    }
+}
+
+// KV heads per workgroup: as many (of 8, 4, 2, 1) as still give every CU a workgroup -- the more heads, the
+// longer the contiguous piece of a cache row one workgroup reads -- and one when the batch is too small for that.
+int decode_fused_heads_per_workgroup(int G, int Hk) {
+    const long long cus = compute_units();
+    for (int c = 8; c > 1; c >>= 1) {
+        if (Hk % c == 0 && (long long)G * (Hk / c) >= cus) return c;
+    }
+    return 1;
+}
+
+bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
+    const int R = a.num_kv_heads > 0 ? a.num_heads / a.num_kv_heads : 0;
+    if (a.bits != 4 && a.bits != 2) return false;
+    if (R != 1 && R != 2 && R != 4) return false;
+    if (a.pos_mode != kPosArray || !a.positions || a.block_table || a.G <= 0) return false;
+    if (a.seq_stride_rows <= 0) return false;
+    auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    if (!al16(a.q) || !al16(f.k_src) || !al16(f.v_src) || !al16(a.rotation)) return false;
+    if ((a.q_stride & 7) != 0 || (f.kv_stride & 7) != 0) return false;
+    if (!al16(a.k) || !al16(a.v)) return false;
+    // the scan addresses a tile through a 32-bit buffer offset from the tile's first row: always small
+    return true;
+}
+
+void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s) {
+    FusedArgs f = f_in;
+    f.hkw = decode_fused_heads_per_workgroup(a.G, a.num_kv_heads);
+    f.q_scale = attention_mfma_q_scale(a.bits);
+    const int R = a.num_heads / a.num_kv_heads;
+    const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw))), b3(kFusedWaves * kWave);
+#define TW_FUSED(RR, BB) launch_scan_kernel(decode_fused_kernel<RR, BB>, g3, b3, s, a, f)
+#define TW_FUSED_R(BB) do { if (R == 1) TW_FUSED(1, BB); else if (R == 2) TW_FUSED(2, BB); else TW_FUSED(4, BB); } while (0)
+    if (a.bits == 4) TW_FUSED_R(4); else TW_FUSED_R(2);
+#undef TW_FUSED_R
+#undef TW_FUSED
+}
+
+}  // namespace twkv

@@ -67,6 +67,10 @@ struct tw_engine {
     int* d_token_history = nullptr;   // (max_new_tokens, G) device
     std::vector<int> h_token_history;
     std::vector<int> h_positions;
+    // range of the device positions as far as the host has seen them (set_positions, reset, + 1 per decode
+    // step); a caller that writes the device array itself makes it stale, which only costs kernel choice
+    bool pos_known = false;
+    int pos_min = 0, pos_max = 0;
     std::vector<char> h_finished;
     std::vector<std::vector<int>> outputs;
     std::vector<int> stop_ids;
@@ -144,6 +148,7 @@ int carve(tw_engine* e, int G, int msl) {
     if (off > e->arena_cap) return -1;
     e->G = G;
     e->batch_msl = msl;
+    e->pos_known = false;        // until reset or set_positions
     if (e->kv_bits > 0) {
         std::vector<tw_half> rot((size_t)e->shape.head_dim * e->shape.head_dim);
         tw_make_rotation_host(rot.data(), e->shape.head_dim, 42u);
@@ -170,35 +175,23 @@ void layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, con
                                            e->rope_dim, s);
     }
     const bool fused = e->producers == 1;
-    if (e->kv_bits == 0) {
-        if (fused) {
-            tw_qk_norm_rope_append_attention_batch(out, qm, k, v, qw, kw, e->norm_eps, e->norm_biased, e->rope_cos,
-                                                   e->rope_sin, e->rope_dim, (tw_half*)e->cache[layer][0],
-                                                   (tw_half*)e->cache[layer][1], e->attn_scores, e->d_positions,
-                                                   e->batch_msl, e->G, m.num_heads, m.num_kv_heads, m.head_dim,
-                                                   e->q_dim(), e->kv_dim(), s);
-            return;
-        }
-        launch_kv_cache_write_batch((tw_half*)e->cache[layer][0], (tw_half*)e->cache[layer][1], k, v,
-                                    e->d_positions, e->batch_msl, e->G, e->kv_dim(), s);
-        launch_gqa_attention_batch(out, q, (const tw_half*)e->cache[layer][0],
-                                   (const tw_half*)e->cache[layer][1], e->attn_scores, e->d_positions,
-                                   e->batch_msl, e->G, m.num_heads, m.num_kv_heads, m.head_dim,
-                                   e->q_dim(), e->kv_dim(), s);
-    } else if (fused) {
-        tw_qk_norm_rope_turbo_append_attention_batch(
-            out, qm, km, v, qw, kw, e->norm_eps, e->norm_biased, e->rope_cos, e->rope_sin, e->rope_dim,
-            (uint8_t*)e->cache[layer][0], (uint8_t*)e->cache[layer][1], (tw_half*)e->cache[layer][2],
-            (tw_half*)e->cache[layer][3], e->d_rotation, e->attn_scores, e->d_positions, e->batch_msl, e->G,
-            m.num_heads, m.num_kv_heads, m.head_dim, e->q_dim(), e->kv_dim(), e->kv_bits, s);
-    } else {
-        tw_turbo_append_attention_batch(out, q, k, v, (uint8_t*)e->cache[layer][0],
-                                        (uint8_t*)e->cache[layer][1], (tw_half*)e->cache[layer][2],
-                                        (tw_half*)e->cache[layer][3], e->d_rotation, e->attn_scores,
-                                        e->d_positions, e->batch_msl, e->G, m.num_heads,
-                                        m.num_kv_heads, m.head_dim, e->q_dim(), e->kv_dim(),
-                                        e->kv_bits, s);
+    tw_layer_step_args p;
+    memset(&p, 0, sizeof(p));
+    p.out = out; p.q = qm; p.k = km; p.v = v;
+    p.G = e->G; p.num_heads = m.num_heads; p.num_kv_heads = m.num_kv_heads; p.head_dim = m.head_dim;
+    p.q_dim = e->q_dim(); p.kv_dim = e->kv_dim();
+    p.positions = e->d_positions; p.max_seq_len = e->batch_msl;
+    if (fused) {
+        p.q_weight = qw; p.k_weight = kw; p.eps = e->norm_eps; p.biased = e->norm_biased;
+        p.cos_table = e->rope_cos; p.sin_table = e->rope_sin; p.rope_dim = e->rope_dim;
     }
+    p.kv_bits = e->kv_bits;
+    p.cache_k = e->cache[layer][0]; p.cache_v = e->cache[layer][1];
+    p.k_norms = (tw_half*)e->cache[layer][2]; p.v_norms = (tw_half*)e->cache[layer][3];
+    p.rotation = e->d_rotation; p.scratch = e->attn_scores;
+    // what the host knows of the context lengths (positions + 1, the appended token included)
+    if (e->pos_known) { p.ctx_min = e->pos_min + 1; p.ctx_max = e->pos_max + 1; }
+    tw_layer_attention_step(&p, s);
 }
 
 void all_layers(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v, tw_half* out,
@@ -294,6 +287,8 @@ int tw_engine_reset(tw_engine* e) {
         }
     }
     hipMemsetAsync(e->d_positions, 0, (size_t)e->G * sizeof(int), s);
+    e->pos_known = true;
+    e->pos_min = e->pos_max = 0;
     return hipStreamSynchronize(s) == hipSuccess ? 0 : -1;
 }
 
@@ -309,7 +304,16 @@ int tw_engine_set_positions(tw_engine* e, const int* host_positions, int G) {
     for (int g = 0; g < G; g++)
         if (host_positions[g] < 0 || host_positions[g] >= e->batch_msl) return -2;
     // engine.cpp:2364
-    return hipMemcpy(e->d_positions, host_positions, (size_t)G * sizeof(int), hipMemcpyHostToDevice) == hipSuccess ? 0 : -3;
+    if (hipMemcpy(e->d_positions, host_positions, (size_t)G * sizeof(int), hipMemcpyHostToDevice) != hipSuccess) return -3;
+    e->pos_known = G == e->G && G > 0;
+    if (e->pos_known) {
+        e->pos_min = e->pos_max = host_positions[0];
+        for (int g = 1; g < G; g++) {
+            e->pos_min = host_positions[g] < e->pos_min ? host_positions[g] : e->pos_min;
+            e->pos_max = host_positions[g] > e->pos_max ? host_positions[g] : e->pos_max;
+        }
+    }
+    return 0;
 }
 
 int tw_engine_set_producers(tw_engine* e, int mode, const tw_half* q_norm, const tw_half* k_norm, float eps,
@@ -433,6 +437,7 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
     tw_kv_clear_error();
     if (!use_graph) {
         all_layers(e, q, k, v, out, s);
+        if (e->pos_known) { e->pos_min++; e->pos_max++; }
         return tw_kv_last_error();
     }
     const void* key[4] = {q, k, v, out};
@@ -458,7 +463,9 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
         e->graph_G = e->G;
         memcpy(e->graph_key, key, sizeof(key));
     }
-    return hipGraphLaunch(e->graph_exec, s) == hipSuccess ? 0 : -7;
+    if (hipGraphLaunch(e->graph_exec, s) != hipSuccess) return -7;
+    if (e->pos_known) { e->pos_min++; e->pos_max++; }
+    return 0;
 }
 
 int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end, int T, hipStream_t s) {

@@ -166,6 +166,23 @@ bool launch_merge_rotate(const AttnArgs& a, hipStream_t s);   // MFMA merge + ro
 bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query);
 float attention_mfma_q_scale(int bits);
 void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);
+// One decode step of a layer in one launch (kv_decode_fused.hip): append the new K and V rows, rotate the
+// query, scan, merge and rotate back.  AttnArgs as for the batch decode over the contiguous compressed
+// cache (positions array; no workspace needed), plus the rows to append and the cache as writable pointers.
+struct FusedArgs {
+    const half_t* k_src;    // (G, kv_stride) fp16 rows of the new token
+    const half_t* v_src;
+    long long kv_stride;
+    uint8_t* k_codes;       // the arrays AttnArgs::k, v, k_norms, v_norms point at
+    uint8_t* v_codes;
+    half_t* k_norms;
+    half_t* v_norms;
+    int hkw;                // KV heads per workgroup (launch_decode_fused fills this in)
+    float q_scale;          // likewise
+};
+bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f);
+int decode_fused_heads_per_workgroup(int G, int num_kv_heads);   // 8, 4, 2 or 1; a workgroup has 16 waves
+void launch_decode_fused(const AttnArgs& a, const FusedArgs& f, hipStream_t s);
 // causal prefill with blocks of query tokens per wave (kv_prefill_mfma.hip); same workspace and merge
 bool prefill_mfma_usable(const AttnArgs& a);
 void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s);

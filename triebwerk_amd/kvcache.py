@@ -232,6 +232,11 @@ def set_prefill_form(form: int) -> None:
     _lib.load().tw_kv_set_prefill_form(int(form))
 
 
+def set_decode_fused(mode: int) -> None:
+    """0: one-launch decode step when max_seq_len <= 2048, 1: whenever the shape allows it, 2: never."""
+    _lib.load().tw_kv_set_decode_fused(int(mode))
+
+
 def set_num_splits(nsplit: int) -> None:
     _lib.load().tw_kv_set_num_splits(int(nsplit))
 
@@ -308,7 +313,7 @@ def launch_sigmoid_gate_batch(data, gate, dim, G, stream=None):
 def tw_layer_attention_step(out, q, k, v, positions, max_seq_len, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim,
                             cache_k, cache_v, scratch, kv_bits=0, k_norms=None, v_norms=None, rotation=None,
                             q_weight=None, k_weight=None, eps=1e-6, biased=False, cos_table=None, sin_table=None,
-                            rope_dim=0, gate=None, gate_stride=0, gate_offset=0, stream=None):
+                            rope_dim=0, gate=None, gate_stride=0, gate_offset=0, ctx_min=0, ctx_max=0, stream=None):
     """Steps 3-6 of a layer (producers, append, attention, gate) through tw_layer_attention_step.
     `gate` may be the q tensor itself with gate_offset = num_heads*head_dim (gated q projection)."""
     lib = _lib.load()
@@ -327,5 +332,6 @@ def tw_layer_attention_step(out, q, k, v, positions, max_seq_len, G, num_heads, 
     gp = _ptr(gate, "f16", "gate")
     a.gate = (gp + 2 * gate_offset) if gp is not None else None
     a.gate_stride = gate_stride
+    a.ctx_min, a.ctx_max = int(ctx_min), int(ctx_max)       # host knowledge of positions + 1; 0, 0 = none
     lib.tw_layer_attention_step(_lib.C.byref(a), _stream(stream))
     _done(lib)
