@@ -752,12 +752,14 @@ def test_producer_rejects_unsupported_shapes(kv):
         kv.launch_rope_batch(q, k, w, w, pos, 16, 2, 2, 2, 128, 256, 256, 96)
 
 
-@pytest.mark.parametrize("variant", [0, 1])
-@pytest.mark.parametrize("bits,H,Hk,norm,rope_dim", [(4, 16, 8, True, 128), (2, 16, 8, True, 128), (4, 32, 8, True, 64),
-                                                     (2, 8, 8, False, 128), (4, 16, 8, True, 0)])
-def test_fused_norm_rope_turbo_step(kv, oracle, rotation_fixture, bits, H, Hk, norm, rope_dim, variant):
+@pytest.mark.parametrize("variant,one_launch", [(0, 1), (0, 2), (1, 0)])
+@pytest.mark.parametrize("bits,H,Hk,norm,rope_dim,biased", [
+    (4, 16, 8, True, 128, False), (2, 16, 8, True, 128, False), (4, 32, 8, True, 64, False), (2, 8, 8, False, 128, False),
+    (4, 16, 8, True, 0, False), (4, 16, 8, True, 48, True), (2, 32, 8, True, 32, True), (4, 8, 2, True, 16, False)])
+def test_fused_norm_rope_turbo_step(kv, oracle, rotation_fixture, bits, H, Hk, norm, rope_dim, biased, variant, one_launch):
     """RMSNorm + RoPE + append + attention in one call == the oracle's four steps: cache bytes bit for
-    bit, output within the attention tolerance.  variant 1 takes the kernels of their own."""
+    bit, output within the attention tolerance.  One kernel for the whole step (one_launch 1), the three-kernel
+    path with the producers inside its rotation launch (2), and variant 1: the kernels of their own."""
     import torch
     r = gen.rng(730 + bits + H + rope_dim)
     G, msl = 9, 384
@@ -773,15 +775,17 @@ def test_fused_norm_rope_turbo_step(kv, oracle, rotation_fixture, bits, H, Hk, n
     out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
     scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
     kv.set_attention_variant(variant)
+    kv.set_decode_fused(one_launch)
     try:
         kv.tw_qk_norm_rope_turbo_append_attention_batch(
-            out, dev(q), dev(k), dev(v), dev(qw) if norm else None, dev(kw) if norm else None, 1e-6, False,
+            out, dev(q), dev(k), dev(v), dev(qw) if norm else None, dev(kw) if norm else None, 1e-6, biased,
             dev(ct) if rope_dim else None, dev(st) if rope_dim else None, rope_dim, d_ck, d_cv, d_kn, d_vn,
             dev(rotation_fixture), scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
     finally:
         kv.set_attention_variant(0)
+        kv.set_decode_fused(0)
     if norm:
-        oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, 1e-6, q_dim, kv_dim, False)
+        oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, 1e-6, q_dim, kv_dim, biased)
     if rope_dim:
         oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, rope_dim)
     oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)

@@ -521,15 +521,18 @@ static thread_local int t_ctx_max = 0;
 //     (measured on MI355X: 4 bit ~1M tokens per launch; 2 bit with 8 KV heads, where the three-kernel path
 //     loads whole rows cooperatively, ~256k).
 // false = not taken.
-static bool try_decode_fused(const AttnArgs& a, const tw_half* k_buf, const tw_half* v_buf, int kv_dim,
-                             uint8_t* ck_q, uint8_t* cv_q, tw_half* k_norms, tw_half* v_norms, int msl,
-                             hipStream_t s, const char* fn) {
-    const int mode = g_decode_fused.load();
-    if (mode == 2 || g_variant.load() == 1) return false;
+static FusedArgs fused_args(const tw_half* k_buf, const tw_half* v_buf, int kv_dim, uint8_t* ck_q, uint8_t* cv_q,
+                            tw_half* k_norms, tw_half* v_norms) {
     FusedArgs f;
     memset(&f, 0, sizeof(f));
     f.k_src = H(k_buf); f.v_src = H(v_buf); f.kv_stride = kv_dim;
     f.k_codes = ck_q; f.v_codes = cv_q; f.k_norms = H(k_norms); f.v_norms = H(v_norms);
+    return f;
+}
+
+static bool try_decode_fused(const AttnArgs& a, const FusedArgs& f, int msl, hipStream_t s, const char* fn) {
+    const int mode = g_decode_fused.load();
+    if (mode == 2 || g_variant.load() == 1) return false;
     if (!decode_fused_usable(a, f)) return false;
     if (mode == 0) {
         const int hkw = decode_fused_heads_per_workgroup(a.G, a.num_kv_heads);
@@ -567,7 +570,7 @@ void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_ha
     fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads,
                 num_kv_heads, bits, as);
     a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
-    if (try_decode_fused(a, k_buf, v_buf, kv_dim, ck_q, cv_q, k_norms, v_norms, msl, s, fn)) return;
+    if (try_decode_fused(a, fused_args(k_buf, v_buf, kv_dim, ck_q, cv_q, k_norms, v_norms), msl, s, fn)) return;
     plan_splits(a, msl, msl);
     // one rotation launch for the appended K and V rows and, when the MFMA scan will run,
     // for the query as well
@@ -693,6 +696,12 @@ void tw_qk_norm_rope_turbo_append_attention_batch(
     fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads,
                 num_kv_heads, bits, as);
     a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    {
+        FusedArgs f = fused_args(k_buf, v_buf, kv_dim, ck_q, cv_q, k_norms, v_norms);
+        f.q_weight = H(q_weight); f.k_weight = H(k_weight); f.eps = eps; f.biased = biased ? 1 : 0;
+        f.cos_table = H(cos_table); f.sin_table = H(sin_table); f.rope_dim = rope_dim;
+        if (try_decode_fused(a, f, msl, s, fn)) return;
+    }
     plan_splits(a, msl, msl);
     const int R = num_heads / num_kv_heads;
     const bool aligned = ((reinterpret_cast<uintptr_t>(q_weight) | reinterpret_cast<uintptr_t>(k_weight) |

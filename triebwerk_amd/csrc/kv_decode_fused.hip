@@ -29,12 +29,17 @@
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 #include "kv_mfma_util.hpp"
+#include "kv_producer_util.hpp"
 
 namespace twkv {
 
 namespace {
 
 constexpr int kFusedWaves = 16;
+#ifndef TW_FUSED_SHARE
+#define TW_FUSED_SHARE 33
+#endif
+constexpr unsigned kFusedShare = TW_FUSED_SHARE;  // 64ths of a sequence's tiles that go to the lower eight waves
 constexpr int kFusedMaxQ = 32;                 // query heads of a unit: HKW * R <= 8 * 4
 constexpr int kRowFloats = kHeadDim + 4;       // LDS row of a vector: conflict-free 16-byte accesses
 constexpr int kStageStride = 2 * kHeadDim + 16;   // bytes per staged fp16 vector
@@ -52,7 +57,7 @@ __device__ __forceinline__ float pick_half16(const uint4& piece, int e, int kk) 
 
 }  // namespace
 
-template <int R, int BITS>
+template <int R, int BITS, bool PROD>
 __global__ void __launch_bounds__(kFusedWaves * kWave)
 decode_fused_kernel(AttnArgs a, FusedArgs f) {
     constexpr int KW = BITS, VW = BITS;
@@ -63,6 +68,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     __shared__ __attribute__((aligned(16))) float qrot_s[kFusedMaxQ][kHeadDim];
     __shared__ __attribute__((aligned(16))) float part_s[kFusedWaves][R][kRowFloats];
     __shared__ __attribute__((aligned(16))) float o_s[kFusedMaxQ][kRowFloats];
+    __shared__ __attribute__((aligned(16))) half_t prod_s[4][kHeadDim];   // k_weight, q_weight, cos row, sin row
 
     const int tid = threadIdx.x;
     const int wave = uniform(tid / kWave), lane = tid % kWave;
@@ -125,12 +131,28 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const int hk_local = wave % HKW, part = wave / HKW;
     const int h = hg * HKW + hk_local;                 // KV head of this wave
 
+    // producers' operands: the two weight vectors and the table rows of this sequence's position, 16 bytes per thread
+    const bool normed = PROD && f.q_weight != nullptr, roped = PROD && f.cos_table != nullptr;
+    uint4 prod = {0u, 0u, 0u, 0u};
+    const int prod_row = tid >> 4, prod_piece = tid & 15;
+    bool prod_live = false;
+    if (PROD && tid < 64) {
+        if (prod_row < 2 && normed) {
+            prod = reinterpret_cast<const uint4*>(prod_row == 0 ? f.k_weight : f.q_weight)[prod_piece];
+            prod_live = true;
+        } else if (prod_row >= 2 && roped && prod_piece < (f.rope_dim >> 4)) {
+            const half_t* tabrow = (prod_row == 2 ? f.cos_table : f.sin_table) + (long long)pos * (f.rope_dim >> 1);
+            prod = reinterpret_cast<const uint4*>(tabrow)[prod_piece];
+            prod_live = true;
+        }
+    }
+
     // ---- part of the context this wave scans: 32-token tiles, lower waves 33/64 of them
     int t0, t1;
     {
         const int ntile = (n + 31) >> 5;
         const int halfparts = SPLIT >> 1;              // SPLIT is 2, 4, 8 or 16
-        const int lower = min(ntile, (int)((ntile * kPairShare + 63u) / 64u));
+        const int lower = min(ntile, (int)((ntile * kFusedShare + 63u) / 64u));
         int b0, b1;
         if (part < halfparts) {
             b0 = lower * part / halfparts;
@@ -146,27 +168,37 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const int ntiles = t1 > t0 ? (t1 - t0 + 31) >> 5 : 0;
 
     // ---- scan set-up (as attention_mfma_kernel, contiguous layout)
+    // Per-lane offsets and selectors.  They are derived twice, before the rotations (for the loads issued up
+    // front) and after them from a laundered copy of the lane number, so that the two sets are separate values:
+    // otherwise they stay live across the rotations, the allocator spills some of them there and reloads them
+    // inside the scan loop, where a reload waits for every load in flight.
     const char* tab_lane = reinterpret_cast<const char*>(tab_s);
-    const uint32_t lane_rep = BITS == 4 ? (uint32_t)lane * 4u : (uint32_t)(lane & 31) * 8u;
     const uint32_t kvp = (uint32_t)Hk * kHeadBytes;
     const uint32_t nrow = (uint32_t)Hk * 2u;
-    const uint32_t koff = (uint32_t)(lane >> 2) * kvp + (kHeadBytes / 4) * (uint32_t)(lane & 3);
-    const int ksrc = 4 * (4 * ln + kg);
-    uint32_t voff[VW];
-#pragma unroll
-    for (int i = 0; i < VW; i++) {
-        if (BITS == 4) voff[i] = (uint32_t)(4 * kg + i) * kvp + 4u * (uint32_t)ln;
-        else voff[i] = (uint32_t)(4 * kg + 2 * i + (ln & 1)) * kvp + 4u * (uint32_t)(ln >> 1);
-    }
-    const bool odd = (ln & 1) != 0;
-    const uint32_t sel_keep = odd ? 0x07060302u : 0x05040100u;
-    const uint32_t sel_send = odd ? 0x05040100u : 0x07060302u;
+    const uint32_t vstep = BITS == 4 ? kvp : 2u * kvp;  // V: dword i of a lane sits vstep bytes after dword 0 (one register for the four)
     const uint32_t sub_bytes = 16u * kvp;
-    const int my_sub = kg >> 1;
-    const bool useful = (kg & 1) == 0;
-    const uint32_t noff = (uint32_t)ln * nrow + (uint32_t)my_sub * 16u * nrow;
-    half_t* p_w = &p_s[wave][0][8 * (ln >> 2) + 4 * my_sub + (ln & 3)];
-    const uint4* p_r = reinterpret_cast<const uint4*>(&p_s[wave][ln][8 * kg]);
+    uint32_t lane_rep, koff, voff0, noff, sel_keep, sel_send;
+    int ksrc, my_sub;
+    bool odd, useful;
+    half_t* p_w;
+    const uint4* p_r;
+    auto derive_lane = [&](int l) {
+        const int ln_ = l & 15, kg_ = l >> 4;
+        lane_rep = BITS == 4 ? (uint32_t)l * 4u : (uint32_t)(l & 31) * 8u;
+        koff = (uint32_t)(l >> 2) * kvp + (kHeadBytes / 4) * (uint32_t)(l & 3);
+        ksrc = 4 * (4 * ln_ + kg_);
+        voff0 = BITS == 4 ? (uint32_t)(4 * kg_) * kvp + 4u * (uint32_t)ln_
+                          : (uint32_t)(4 * kg_ + (ln_ & 1)) * kvp + 4u * (uint32_t)(ln_ >> 1);
+        odd = (ln_ & 1) != 0;
+        sel_keep = odd ? 0x07060302u : 0x05040100u;
+        sel_send = odd ? 0x05040100u : 0x07060302u;
+        my_sub = kg_ >> 1;
+        useful = (kg_ & 1) == 0;
+        noff = (uint32_t)ln_ * nrow + (uint32_t)my_sub * 16u * nrow;
+        p_w = &p_s[wave][0][8 * (ln_ >> 2) + 4 * my_sub + (ln_ & 3)];
+        p_r = reinterpret_cast<const uint4*>(&p_s[wave][ln_][8 * kg_]);
+    };
+    derive_lane(lane);
     constexpr float kRaise = 5.0f;
 
     auto lut32 = [&](uint32_t addr) -> uint32_t { return *reinterpret_cast<const uint32_t*>(tab_lane + addr); };
@@ -199,7 +231,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
             for (int i = 0; i < VW; i++)
-                vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)(voff[i] + sub * sub_bytes), 0, 0);
+                vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)(voff0 + i * vstep + sub * sub_bytes), 0, 0);
         }
     };
     auto pick = [&](const uint32x4_t& q) -> uint32_t {
@@ -264,7 +296,32 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         // fall into 32 different banks), in the space the merged outputs will use at the end
         char* x_s = reinterpret_cast<char*>(o_s);
         if ((tid >> 4) < nvec) *reinterpret_cast<uint4*>(x_s + (tid >> 4) * kStageStride + (tid & 15) * 16) = stage;
+        if (PROD && prod_live) *reinterpret_cast<uint4*>(&prod_s[prod_row][8 * prod_piece]) = prod;
         __syncthreads();
+        if (PROD) {
+            // optional producers on the staged K and query vectors, one vector per wave: per-head RMSNorm
+            // (kernels.cu:880-923), then rotary embedding (927-961), each rounded to fp16 as the reference's
+            // in-place kernels leave it; V vectors stay as they are
+            for (int v = wave; v < nvec; v += kFusedWaves) {
+                int kind, head;
+                (void)unit_vector(v, kind, head);
+                if (kind == 1) continue;                           // uniform over the wave
+                half_t* row = reinterpret_cast<half_t*>(x_s + v * kStageStride);
+                float x0 = (float)row[lane], x1 = (float)row[lane + 64];
+                HeadXform t;
+                t.weight = normed ? &prod_s[0][0] + (kind == 0 ? 0 : kHeadDim) : nullptr;
+                t.eps = f.eps;
+                t.biased = f.biased;
+                t.cos_row = roped ? prod_s[2] : nullptr;
+                t.sin_row = prod_s[3];
+                t.rope_dim = f.rope_dim;
+                t.single_order = 0;
+                xform_head(x0, x1, lane, t);
+                row[lane] = (half_t)x0;                            // both are fp16 values already
+                row[lane + 64] = (half_t)x1;
+            }
+            __syncthreads();
+        }
 
         for (int vt = wave >> 3; vt * 16 < nvec; vt += 2) {       // uniform over the wave
             const int vi = vt * 16 + i16;
@@ -277,9 +334,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             const half_t* xrow = reinterpret_cast<const half_t*>(x_s + vc * kStageStride) + kk;
 #pragma unroll
             for (int s2 = 0; s2 < 32; s2++) xv[s2] = (float)xrow[4 * s2];
-            // sum of squares in the reference's order (kernels.cu:1509-1520), as rotate_kernel
-            float n2 = 0.0f;
-            {
+            // sum of squares in the reference's order (kernels.cu:1509-1520), as rotate_kernel: xv[s] is
+            // coordinate 4s + kk; offsets 16, 8, 4 of the 32-lane tree stay inside a lane, 2 and 1 cross lanes
+            auto tree_sum_sq = [&]() -> float {
                 float sgrp[4];
 #pragma unroll
                 for (int w = 0; w < 4; w++) {
@@ -292,8 +349,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
                     float d = c + __shfl_xor(c, 32, 64);
                     sgrp[w] = d + __shfl_xor(d, 16, 64);
                 }
-                n2 = (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
-            }
+                return (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
+            };
+            const float n2 = tree_sum_sq();
             if (!is_query) {
                 const float inv = 1.0f / sqrtf(n2 + 1e-12f);
 #pragma unroll
@@ -329,6 +387,11 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         }
     }
     __syncthreads();        // table, q_rot and the new cache row are in place
+    {
+        int l2 = lane;
+        asm volatile("" : "+v"(l2));
+        derive_lane(l2);
+    }
 
     // ---- 2. scan of this wave's part
     float4_t o[8];
@@ -607,6 +670,9 @@ bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
     if (!al16(a.q) || !al16(f.k_src) || !al16(f.v_src) || !al16(a.rotation)) return false;
     if ((a.q_stride & 7) != 0 || (f.kv_stride & 7) != 0) return false;
     if (!al16(a.k) || !al16(a.v)) return false;
+    if ((f.q_weight == nullptr) != (f.k_weight == nullptr) || (f.cos_table == nullptr) != (f.sin_table == nullptr)) return false;
+    if (!al16(f.q_weight) || !al16(f.k_weight) || !al16(f.cos_table) || !al16(f.sin_table)) return false;
+    if (f.cos_table && !(f.rope_dim == 128 || (f.rope_dim > 0 && f.rope_dim <= 64 && f.rope_dim % 16 == 0))) return false;
     // the scan addresses a tile through a 32-bit buffer offset from the tile's first row: always small
     return true;
 }
@@ -617,7 +683,10 @@ void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s
     f.q_scale = attention_mfma_q_scale(a.bits);
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw))), b3(kFusedWaves * kWave);
-#define TW_FUSED(RR, BB) launch_scan_kernel(decode_fused_kernel<RR, BB>, g3, b3, s, a, f)
+    const bool prod = f.q_weight != nullptr || f.cos_table != nullptr;
+#define TW_FUSED(RR, BB) \
+    do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true>, g3, b3, s, a, f); \
+         else launch_scan_kernel(decode_fused_kernel<RR, BB, false>, g3, b3, s, a, f); } while (0)
 #define TW_FUSED_R(BB) do { if (R == 1) TW_FUSED(1, BB); else if (R == 2) TW_FUSED(2, BB); else TW_FUSED(4, BB); } while (0)
     if (a.bits == 4) TW_FUSED_R(4); else TW_FUSED_R(2);
 #undef TW_FUSED_R

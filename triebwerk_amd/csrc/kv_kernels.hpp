@@ -179,6 +179,14 @@ struct FusedArgs {
     half_t* v_norms;
     int hkw;                // KV heads per workgroup (launch_decode_fused fills this in)
     float q_scale;          // likewise
+    // optional producers of q and k applied on the way in, as RotArgs has them (V rows stay as they are)
+    const half_t* q_weight; // per-head RMSNorm weights (128); both or neither
+    const half_t* k_weight;
+    float eps;
+    int biased;
+    const half_t* cos_table; // (positions, rope_dim / 2); both or neither
+    const half_t* sin_table;
+    int rope_dim;            // 128, or a multiple of 16 up to 64
 };
 bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f);
 int decode_fused_heads_per_workgroup(int G, int num_kv_heads);   // 8, 4, 2 or 1; a workgroup has 16 waves
