@@ -49,8 +49,9 @@ BYTES_HEAD = {0: 256, 4: 66, 2: 34}  # per (token, kv head): fp16 row | codes + 
 # HBM bytes per launch (read + write) of the context-scanning kernel, from rocprofv3 --pmc FETCH_SIZE
 # and WRITE_SIZE on this file's own run, each counter scaled by what `--copy-calibration` reads for a
 # copy of known size (2.0 and 1.0); summary and commands in profiles/scan_target_hbm_traffic_pmc.txt.
-# Keyed by (workload, kv_bits); a measurement of the kernels as committed with that file, not live.
-MEASURED_TRAFFIC_BYTES = {("target", 4): 560.8e6, ("target", 2): 292.3e6, ("target", 0): 2151.2e6}
+# Keyed by (workload, kv_bits, kernel that ran); a measurement of the kernels as committed with that file, not live.
+MEASURED_TRAFFIC_BYTES = {("target", 4, "one-launch"): 557.8e6, ("target", 4, "scan"): 560.8e6,
+                          ("target", 2, "scan"): 292.2e6, ("target", 0, "scan"): 2151.2e6}
 
 
 def algorithmic_bytes(n_tokens_total: int, G: int, L: int, H: int, Hk: int, kv_bits: int, with_append: bool) -> int:
@@ -342,6 +343,7 @@ def main():
     # kernel on its stream (hipExtLaunchKernelGGL: start = the kernel begins, stop = it ends), in eager
     # steps that continue the same decode; the library holds 4096 event pairs
     Kp = max(1, min(K, 4096 // L))
+    fused_before = lib.tw_kv_decode_fused_launches()
     lib.tw_kv_profile_attention(1)
     with torch.cuda.stream(stream):
         for _ in range(Kp):
@@ -353,7 +355,10 @@ def main():
     assert rc == 0 and launches.value == Kp * L, (rc, launches.value)
     n_tokens_prof = int(sum(int((pos_now + i + 1).sum()) for i in range(Kp)))
     kern_ms = total_ms.value / launches.value
-    launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=False) / (Kp * L)
+    # which kernel those launches were: the whole layer step in one launch (append included), or the scan of the
+    # three-kernel path
+    one_launch = lib.tw_kv_decode_fused_launches() - fused_before == Kp * L
+    launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=one_launch) / (Kp * L)
     achieved = launch_bytes / (kern_ms * 1e-3) * 1e-9
 
     # ---- what a plain contiguous read kernel reaches on this GPU: over 4 GiB, and over exactly the
@@ -404,7 +409,8 @@ def main():
         "step_frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
         "roofline": {
             "bound": "hbm",
-            "kernel": "decode attention (context scan), one launch per layer",
+            "kernel": ("decode step of a layer in one launch (append, query rotation, context scan, merge, rotate-back)"
+                       if one_launch else "decode attention (context scan), one launch per layer"),
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -413,7 +419,8 @@ def main():
             "launch_algorithmic_MB": launch_bytes * 1e-6,
             "plain_read_GBps_4GiB": read_big,
             "plain_read_GBps_same_bytes_per_launch": read_same,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, kv_bits)) if not overridden else None,
+            "traffic": (MEASURED_TRAFFIC_BYTES.get((args.workload, kv_bits, "one-launch" if one_launch else "scan"))
+                        if not overridden and args.producers == "none" else None),
         },
     }
     if not args.no_cpu:

@@ -175,6 +175,9 @@ void tw_kv_set_prefill_form(int form);
  * workgroup's work however long it is; 1: whenever the shape allows it (contiguous compressed cache, GQA group 1, 2
  * or 4); 2: never.  Process-wide. */
 void tw_kv_set_decode_fused(int mode);
+/* Layer steps that took the one-launch kernel since the library was loaded (launches issued or recorded into a
+ * graph under capture): lets a benchmark say which kernel its figures belong to. */
+long long tw_kv_decode_fused_launches(void);
 
 /* Timing of the context-scanning attention kernel alone, with HIP events
  * recorded on the launch stream around that kernel (not around the merge).

@@ -17,6 +17,7 @@
 using namespace twkv;
 
 namespace twkv {
+static std::atomic<long long> g_fused_launches{0};   // one-launch decode steps issued so far (tw_kv_decode_fused_launches)
 static std::atomic<int> g_decode_fused{0};   // tw_kv_set_decode_fused: 0 by context bound, 1 whenever possible, 2 never
 static std::atomic<int> g_prefill_form{0};   // test hook, see prefill_form()
 int prefill_form() { return g_prefill_form.load(); }
@@ -194,6 +195,7 @@ int tw_kv_get_attention_variant(void) { return g_variant.load(); }
 void tw_kv_set_num_splits(int n) { g_nsplit_override.store(n); }
 void tw_kv_set_prefill_form(int form) { g_prefill_form.store(form); }
 void tw_kv_set_decode_fused(int mode) { g_decode_fused.store(mode); }
+long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }
 
 void tw_kv_profile_attention(int enable) {
     g_prof.enabled.store(enable);
@@ -548,6 +550,7 @@ static bool try_decode_fused(const AttnArgs& a, const FusedArgs& f, int msl, hip
         if (!take) return false;
     }
     attach_profiler(s);
+    g_fused_launches.fetch_add(1);
     launch_decode_fused(a, f, s);
     t_scan_start = t_scan_stop = nullptr;
     check_launch(fn);
