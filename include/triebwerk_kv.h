@@ -226,6 +226,15 @@ void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_ha
                                      int num_kv_heads, int head_dim, int q_dim, int kv_dim,
                                      int bits, hipStream_t s);
 
+/* The same for the fp16 cache: what engine.cpp:1979-2003 does with launch_kv_cache_write_batch and
+ * launch_gqa_attention_batch, as one launch (plus the merge of the context chunks when there are several): the
+ * attention kernel takes the new token's K and V rows from k_buf / v_buf and stores them into the cache itself.
+ * Same cache bytes and outputs as the two calls.  (tw_kv_set_decode_fused(2) keeps the two launches.) */
+void tw_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf, const tw_half* v_buf,
+                               tw_half* ck, tw_half* cv, float* as, const int* pos, int msl, int G,
+                               int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                               hipStream_t s);
+
 /* Producers fused into the path (steps 3-5 of forward_layer_batch, engine.cpp:1972-2006, in one
  * call): per-head RMSNorm (q_weight / k_weight, `biased`) and rotary embedding (tables as for
  * launch_rope_batch) of q and k, append of K and V at positions[g], attention over

@@ -222,6 +222,41 @@ def test_fp16_attention_batch_config1(kv, oracle, nsplit):
     assert rel_err(host(out), want) <= TOL
 
 
+@pytest.mark.parametrize("mode", [0, 2])
+@pytest.mark.parametrize("nsplit", [0, 1, 3])
+@pytest.mark.parametrize("H,Hk", [(16, 8), (8, 2), (4, 4), (8, 1)])
+def test_fp16_append_attention_step(kv, oracle, H, Hk, nsplit, mode):
+    """fp16 cache, append + attention in one call: with the append inside the attention launch (mode 0) and
+    as the reference's two launches (mode 2).  Cache bytes equal the oracle's row copy (nothing else
+    touched), outputs within tolerance of the oracle's attention over the appended cache."""
+    import torch
+    r = gen.rng(210 + H + Hk)
+    lens = [0, 1, 15, 16, 63, 64, 65, 255, 256, 700, 1023]
+    G, msl = len(lens), 1024
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+    pos = np.array(lens, np.int32)
+    for g in range(G):
+        ck[g, pos[g]:] = 0; cv[g, pos[g]:] = 0
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    d_ck, d_cv = dev(ck), dev(cv)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.set_num_splits(nsplit)
+    kv.set_decode_fused(mode)
+    try:
+        kv.tw_append_attention_batch(out, dev(q), dev(k), dev(v), d_ck, d_cv, scratch, dev(pos), msl, G, H, Hk, D,
+                                     q_dim, kv_dim)
+    finally:
+        kv.set_num_splits(0)
+        kv.set_decode_fused(0)
+    oracle.kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    assert_bytes_equal(host(d_ck), ck, "K rows"); assert_bytes_equal(host(d_cv), cv, "V rows")
+    assert rel_err(host(out), want) <= TOL
+
+
 def test_fp16_attention_ragged_and_strided(kv, oracle):
     r = gen.rng(202)
     G, H, Hk, msl = 6, 8, 2, 1500   # GQA group 4

@@ -43,11 +43,14 @@ __device__ __forceinline__ int lane_dim(int c, int e) {
 }
 
 // Load and dequantize the lane's 32 values of one cache row (one KV head).
+// fresh: fp16 only, the head's 128 halves come from there instead (the row of the token being appended), or NULL.
 template <int MODE>
 __device__ __forceinline__ void load_vals(const void* __restrict__ base, long long row, int num_kv_heads,
-                                          int h, int c, const float* __restrict__ cent_s, float* vals) {
+                                          int h, int c, const float* __restrict__ cent_s, float* vals,
+                                          const half_t* fresh = nullptr) {
     if (MODE == 0) {
         const half_t* p = reinterpret_cast<const half_t*>(base) + (row * num_kv_heads + h) * kHeadDim;
+        if (fresh) p = fresh;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             half8_t h8 = *reinterpret_cast<const half8_t*>(p + 32 * j + 8 * c);
@@ -93,7 +96,10 @@ __device__ __forceinline__ void store_head(const AttnArgs& a, int g, int head, i
     a.out[(long long)g * a.q_stride + (long long)head * kHeadDim + d] = h;
 }
 
-template <int MODE, int RT>
+// APPEND (fp16 cache, batch decode): the token at positions[g] is not in the cache yet; its rows are a.k_new and
+// a.v_new, read from there by whichever lane meets that token and stored into the cache by the workgroup whose
+// chunk holds it (the one of the KV head's first query-head tile).
+template <int MODE, int RT, bool APPEND>
 __global__ void __launch_bounds__(kAttnThreads)
 attention_valu_kernel(AttnArgs a) {
     __shared__ float q_s[RT][kHeadDim];
@@ -117,6 +123,19 @@ attention_valu_kernel(AttnArgs a) {
     if (t0 >= t1) return;                       // uniform for the workgroup
 
     if (tid < 16) cent_s[tid] = (MODE == 2) ? kCentroids2[tid & 3] : kCentroids4[tid];
+    const half_t* k_fresh = nullptr;
+    const half_t* v_fresh = nullptr;
+    if (APPEND) {
+        k_fresh = a.k_new + (long long)g * a.kv_new_stride + (long long)h * kHeadDim;
+        v_fresh = a.v_new + (long long)g * a.kv_new_stride + (long long)h * kHeadDim;
+        if (t0 <= n - 1 && n - 1 < t1 && blockIdx.y % subs == 0 && tid < 32) {      // 16 pieces of 16 bytes each for K and V
+            const long long row = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, g, n - 1);
+            const half_t* src = (tid < 16 ? k_fresh : v_fresh) + 8 * (tid & 15);
+            half_t* cache = reinterpret_cast<half_t*>(const_cast<void*>(tid < 16 ? a.k : a.v));
+            half_t* dst = cache + (row * a.num_kv_heads + h) * kHeadDim + 8 * (tid & 15);
+            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
+        }
+    }
 
     // Query, rotated for the compressed cache: q_rot = R q (kernels.cu:1671-1681).
     for (int idx = tid; idx < RT * kHeadDim; idx += kAttnThreads) {
@@ -165,7 +184,8 @@ attention_valu_kernel(AttnArgs a) {
             vn = (float)a.v_norms[row * a.num_kv_heads + h];
         }
         float vals[32];
-        load_vals<MODE>(a.k, row, a.num_kv_heads, h, c, cent_s, vals);
+        const bool fresh = APPEND && tc == n - 1;
+        load_vals<MODE>(a.k, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? k_fresh : nullptr);
         float s[RT];
 #pragma unroll
         for (int r = 0; r < RT; r++) {
@@ -176,7 +196,7 @@ attention_valu_kernel(AttnArgs a) {
             dot += __shfl_xor(dot, 2, 64);
             s[r] = dot * (kn * scale);          // kernels.cu:1707
         }
-        load_vals<MODE>(a.v, row, a.num_kv_heads, h, c, cent_s, vals);
+        load_vals<MODE>(a.v, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? v_fresh : nullptr);
         if (valid) {
 #pragma unroll
             for (int r = 0; r < RT; r++) {
@@ -296,9 +316,15 @@ static void launch_valu_mode(const AttnArgs& a, hipStream_t s) {
     const int rt = (group % 4 == 0) ? 4 : (group % 2 == 0) ? 2 : 1;
     dim3 grid(a.nsplit, a.num_kv_heads * (group / rt), a.G);
     dim3 block(kAttnThreads);
-    if (rt == 4) launch_scan_kernel(attention_valu_kernel<MODE, 4>, grid, block, s, a);
-    else if (rt == 2) launch_scan_kernel(attention_valu_kernel<MODE, 2>, grid, block, s, a);
-    else launch_scan_kernel(attention_valu_kernel<MODE, 1>, grid, block, s, a);
+    if (MODE == 0 && a.k_new) {
+        if (rt == 4) launch_scan_kernel(attention_valu_kernel<0, 4, true>, grid, block, s, a);
+        else if (rt == 2) launch_scan_kernel(attention_valu_kernel<0, 2, true>, grid, block, s, a);
+        else launch_scan_kernel(attention_valu_kernel<0, 1, true>, grid, block, s, a);
+        return;
+    }
+    if (rt == 4) launch_scan_kernel(attention_valu_kernel<MODE, 4, false>, grid, block, s, a);
+    else if (rt == 2) launch_scan_kernel(attention_valu_kernel<MODE, 2, false>, grid, block, s, a);
+    else launch_scan_kernel(attention_valu_kernel<MODE, 1, false>, grid, block, s, a);
 }
 
 void launch_attention_valu(const AttnArgs& a, hipStream_t s) {

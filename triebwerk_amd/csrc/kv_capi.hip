@@ -456,6 +456,30 @@ void launch_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half* c
     run_attention(a, s, "launch_gqa_attention_batch");
 }
 
+void tw_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf, const tw_half* v_buf,
+                               tw_half* ck, tw_half* cv, float* as, const int* pos, int msl, int G, int num_heads,
+                               int num_kv_heads, int head_dim, int q_dim, int kv_dim, hipStream_t s) {
+    const char* fn = "tw_append_attention_batch";
+    if (!check_shape(fn, num_heads, num_kv_heads, head_dim)) return;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, kv_dim);
+        return;
+    }
+    const bool aligned = ((reinterpret_cast<uintptr_t>(k_buf) | reinterpret_cast<uintptr_t>(v_buf) |
+                           reinterpret_cast<uintptr_t>(ck) | reinterpret_cast<uintptr_t>(cv)) & 15u) == 0;
+    if (!aligned || g_decode_fused.load() == 2) {       // the two launches of the reference
+        launch_kv_cache_write_batch(ck, cv, k_buf, v_buf, pos, msl, G, kv_dim, s);
+        launch_gqa_attention_batch(out, q, ck, cv, as, pos, msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, s);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck, cv, nullptr, nullptr, nullptr, G, num_heads, num_kv_heads, 0, as);
+    a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    a.k_new = H(k_buf); a.v_new = H(v_buf); a.kv_new_stride = kv_dim;
+    plan_splits(a, msl, msl);
+    run_attention(a, s, fn);
+}
+
 void launch_gqa_prefill_attention(tw_half* out, const tw_half* q, const tw_half* ck,
                                   const tw_half* cv, float* as, int T, int msl, int num_heads,
                                   int num_kv_heads, int head_dim, int q_dim, int kv_dim,
@@ -803,11 +827,9 @@ void tw_layer_attention_step(const tw_layer_step_args* p, hipStream_t s) {
                                                    (tw_half*)p->cache_v, p->scratch, p->positions, p->max_seq_len, p->G,
                                                    p->num_heads, p->num_kv_heads, p->head_dim, p->q_dim, p->kv_dim, s);
         } else {
-            launch_kv_cache_write_batch((tw_half*)p->cache_k, (tw_half*)p->cache_v, p->k, p->v, p->positions,
-                                        p->max_seq_len, p->G, p->kv_dim, s);
-            launch_gqa_attention_batch(p->out, p->q, (const tw_half*)p->cache_k, (const tw_half*)p->cache_v, p->scratch,
-                                       p->positions, p->max_seq_len, p->G, p->num_heads, p->num_kv_heads, p->head_dim,
-                                       p->q_dim, p->kv_dim, s);
+            tw_append_attention_batch(p->out, p->q, p->k, p->v, (tw_half*)p->cache_k, (tw_half*)p->cache_v, p->scratch,
+                                      p->positions, p->max_seq_len, p->G, p->num_heads, p->num_kv_heads, p->head_dim,
+                                      p->q_dim, p->kv_dim, s);
         }
     } else if (producers) {
         tw_qk_norm_rope_turbo_append_attention_batch(

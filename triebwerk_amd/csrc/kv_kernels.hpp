@@ -154,6 +154,12 @@ struct AttnArgs {
     // optional output gate (gated attention, kernels.cu:2987-2995): out = half(float(half(out)) * sigmoid(gate))
     const half_t* gate;     // row g at gate + g * gate_stride, laid out like a row of out; NULL = none
     long long gate_stride;
+    // fp16 cache, batch decode: the K and V rows of the new token (position positions[g]).  The scan takes them
+    // from here instead of the cache and one workgroup per (sequence, KV head) stores them there, which makes
+    // the append part of the attention launch (kv_cache_write_batch_kernel, kernels.cu:964-977).  NULL = none.
+    const half_t* k_new;    // (G, kv_new_stride)
+    const half_t* v_new;
+    long long kv_new_stride;
 };
 
 constexpr int kPartialFloats = kHeadDim + 4;  // acc[128], running max, running sum, 2 pad (16-byte rows)

@@ -276,6 +276,17 @@ def launch_rope(q, k, cos_table, sin_table, pos, max_seq_len, num_heads, num_kv_
     _done(lib)
 
 
+def tw_append_attention_batch(out, q, k_buf, v_buf, ck, cv, scratch, pos, msl, G, num_heads, num_kv_heads, head_dim,
+                              q_dim, kv_dim, stream=None):
+    """fp16 cache: append at pos[g] and attend 0..pos[g] in one launch (engine.cpp:1979-2003)."""
+    lib = _lib.load()
+    lib.tw_append_attention_batch(
+        _ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(k_buf, "f16", "k_buf"), _ptr(v_buf, "f16", "v_buf"),
+        _ptr(ck, "f16", "ck"), _ptr(cv, "f16", "cv"), _ptr(scratch, "f32", "scratch"), _ptr(pos, "i32", "pos"),
+        msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, _stream(stream))
+    _done(lib)
+
+
 def tw_qk_norm_rope_turbo_append_attention_batch(out, q, k_buf, v_buf, q_weight, k_weight, eps, biased, cos_table,
                                                  sin_table, rope_dim, ck_q, cv_q, k_norms, v_norms, rotation,
                                                  scratch, pos, msl, G, num_heads, num_kv_heads, head_dim, q_dim,
