@@ -49,6 +49,72 @@ def rel_err_rows(got, want):
     return np.max(np.abs(got - want), axis=1) / np.max(np.abs(want), axis=1)
 
 
+def build_target_cache(kv, rotation_fixture, bits, G, Hk, ctx, n_base):
+    """The target shape's cache through the T-token append (kernels.cu:1482-1560), one sequence per call;
+    sequence g replicates base sequence g % n_base.  Returns the base rows and the device arrays."""
+    import torch
+    kv_dim = Hk * D
+    kvp = kv_dim * bits // 8
+    msl = ctx
+    r = gen.rng(900 + bits)
+    rot = dev(rotation_fixture)
+    base_k = [gen.kv_rows_with_outliers(r, (ctx, kv_dim), kv_dim)[0] for _ in range(n_base)]
+    base_v = [gen.normal_f16(r, (ctx, kv_dim)) for _ in range(n_base)]
+    d_base_k = [dev(x) for x in base_k]
+    d_base_v = [dev(x) for x in base_v]
+    ck = torch.zeros((G, msl, kvp), dtype=torch.uint8, device="cuda")
+    cv = torch.zeros_like(ck)
+    kn = torch.zeros((G, msl, Hk), dtype=torch.float16, device="cuda")
+    vn = torch.zeros_like(kn)
+    tok = dev(np.arange(ctx, dtype=np.int32))
+    for g in range(G):
+        kv.launch_turbo_kv_quantize(ck[g], kn[g], d_base_k[g % n_base], rot, tok, msl, ctx, Hk, D, kv_dim, bits)
+        kv.launch_turbo_kv_quantize(cv[g], vn[g], d_base_v[g % n_base], rot, tok, msl, ctx, Hk, D, kv_dim, bits)
+    return r, rot, base_k, base_v, ck, cv, kn, vn
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_target_shape_decode_step_in_one_launch(kv, oracle, rotation_fixture, bits):
+    """The benchmark's default path at its full size: one decode step of a layer as one kernel (batch 64, contexts
+    8187..8191 + the appended token).  Appended rows equal the oracle's bytes, every other byte of the cache is
+    untouched, outputs within tolerance of the oracle and of the three-kernel path."""
+    import torch
+    G, H, Hk, ctx = 64, 16, 8, 8192
+    kv_dim, q_dim = Hk * D, H * D
+    msl = ctx
+    r, rot, _, _, ck, cv, kn, vn = build_target_cache(kv, rotation_fixture, bits, G, Hk, ctx, n_base=4)
+    before = [host(x).copy() for x in (ck, cv, kn, vn)]
+    pos = (ctx - 1 - (np.arange(G) % 5)).astype(np.int32)       # the append overwrites row pos[g]
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    outs, caches = {}, {}
+    for mode in (1, 2):
+        c = [dev(x) for x in before]
+        out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+        kv.set_decode_fused(mode)
+        try:
+            kv.tw_turbo_append_attention_batch(out, dev(q), dev(k), dev(v), c[0], c[1], c[2], c[3], rot, scratch, dev(pos),
+                                               msl, G, H, Hk, D, q_dim, kv_dim, bits)
+        finally:
+            kv.set_decode_fused(0)
+        outs[mode] = host(out)
+        caches[mode] = [host(x) for x in c]
+        del c
+    want_c = [x.copy() for x in before]
+    oracle.turbo_kv_quantize_batch(want_c[0], want_c[2], k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(want_c[1], want_c[3], v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    for mode in (1, 2):
+        for got, want_arr, what in zip(caches[mode], want_c, ("K codes", "V codes", "K norms", "V norms")):
+            assert np.array_equal(got.view(np.uint8), want_arr.view(np.uint8)), f"mode {mode}: {what}"
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, want_c[0], want_c[1], want_c[2], want_c[3], rotation_fixture, pos, msl, G,
+                                     H, Hk, D, q_dim, kv_dim, bits)
+    for mode in (1, 2):
+        err = rel_err_rows(outs[mode], want)
+        assert err.max() <= TOL, f"mode {mode}: max rel err {err.max():.3e} at head vector {err.argmax()}"
+    assert rel_err_rows(outs[1], outs[2]).max() <= TOL
+
+
 @pytest.mark.parametrize("bits", [4, 2])
 def test_target_shape_append_and_attention(kv, oracle, rotation_fixture, bits):
     import torch
@@ -57,21 +123,7 @@ def test_target_shape_append_and_attention(kv, oracle, rotation_fixture, bits):
     kvp = kv_dim * bits // 8
     msl = ctx
     n_base = 4                                   # distinct sequences; sequence g replicates g % n_base
-    r = gen.rng(900 + bits)
-    rot = dev(rotation_fixture)
-    base_k = [gen.kv_rows_with_outliers(r, (ctx, kv_dim), kv_dim)[0] for _ in range(n_base)]
-    base_v = [gen.normal_f16(r, (ctx, kv_dim)) for _ in range(n_base)]
-    d_base_k = [dev(x) for x in base_k]
-    d_base_v = [dev(x) for x in base_v]
-
-    ck = torch.zeros((G, msl, kvp), dtype=torch.uint8, device="cuda")
-    cv = torch.zeros_like(ck)
-    kn = torch.zeros((G, msl, Hk), dtype=torch.float16, device="cuda")
-    vn = torch.zeros_like(kn)
-    tok = dev(np.arange(ctx, dtype=np.int32))
-    for g in range(G):                           # T-token append (kernels.cu:1482-1560), one sequence per call
-        kv.launch_turbo_kv_quantize(ck[g], kn[g], d_base_k[g % n_base], rot, tok, msl, ctx, Hk, D, kv_dim, bits)
-        kv.launch_turbo_kv_quantize(cv[g], vn[g], d_base_v[g % n_base], rot, tok, msl, ctx, Hk, D, kv_dim, bits)
+    r, rot, base_k, base_v, ck, cv, kn, vn = build_target_cache(kv, rotation_fixture, bits, G, Hk, ctx, n_base)
     h_ck, h_cv, h_kn, h_vn = host(ck), host(cv), host(kn), host(vn)
 
     # (1) base sequences against the oracle, every byte
