@@ -117,6 +117,14 @@ __device__ __forceinline__ half_t gated(half_t out, half_t gate) {
     return (half_t)((float)out / (1.0f + expf(-(float)gate)));
 }
 
+// Workgroup barrier that orders LDS accesses only: global loads and stores issued before it stay in flight
+// (__syncthreads also waits for every one of them).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));

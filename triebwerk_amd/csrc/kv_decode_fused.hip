@@ -128,6 +128,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         }
     }
 
+    // scaled centroid number lane % 16 (4 bit) or lane % 4 (2 bit), for the table build
+    const float cent_lane = kAlpha * (BITS == 4 ? kCentroids4[lane & 15] : kCentroids2[lane & 3]);
+
     const int pos = uniform(a.positions[g]);
     const int n = pos + 1;
     const int hk_local = wave % HKW, part = wave / HKW;
@@ -275,16 +278,18 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     {
         const int i16 = ln, kk = kg;
         const int dblk = rot_dblk;
-        // the centroid table while the loads are under way: entry e fills 256 bytes with replicas
+        // the centroid table while the loads are under way: entry e fills 256 bytes with replicas.  The centroids
+        // come out of a register by wave shuffle (lane c holds centroid c): indexing the constant array with a
+        // per-lane index is a dependent memory load per look-up, several microseconds for this loop.
         for (int i = tid * 4; i < kTableWords; i += kFusedWaves * kWave * 4) {
             const int e = i >> 6;
             if constexpr (BITS == 4) {
-                half2_t p = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
+                half2_t p = {(half_t)__shfl(cent_lane, e & 15, 64), (half_t)__shfl(cent_lane, e >> 4, 64)};
                 uint32_t w = *reinterpret_cast<uint32_t*>(&p);
                 *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
             } else {
-                half2_t p0 = {(half_t)(kAlpha * kCentroids2[e & 3]), (half_t)(kAlpha * kCentroids2[(e >> 4) & 3])};
-                half2_t p1 = {(half_t)(kAlpha * kCentroids2[(e >> 2) & 3]), (half_t)(kAlpha * kCentroids2[(e >> 6) & 3])};
+                half2_t p0 = {(half_t)__shfl(cent_lane, e & 3, 64), (half_t)__shfl(cent_lane, (e >> 4) & 3, 64)};
+                half2_t p1 = {(half_t)__shfl(cent_lane, (e >> 2) & 3, 64), (half_t)__shfl(cent_lane, (e >> 6) & 3, 64)};
                 uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
                 *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
             }
@@ -296,7 +301,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         char* x_s = reinterpret_cast<char*>(o_s);
         if ((tid >> 4) < nvec) *reinterpret_cast<uint4*>(x_s + (tid >> 4) * kStageStride + (tid & 15) * 16) = stage;
         if (PROD && prod_live) *reinterpret_cast<uint4*>(&prod_s[prod_row][8 * prod_piece]) = prod;
-        __syncthreads();
+        lds_barrier();             // the tile loads issued up front stay in flight
         if (PROD) {
             // optional producers on the staged K and query vectors, one vector per wave: per-head RMSNorm
             // (kernels.cu:880-923), then rotary embedding (927-961), each rounded to fp16 as the reference's
@@ -319,7 +324,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
                 row[lane] = (half_t)x0;                            // both are fp16 values already
                 row[lane + 64] = (half_t)x1;
             }
-            __syncthreads();
+            lds_barrier();
         }
 
         for (int vt = wave >> 3; vt * 16 < nvec; vt += 2) {       // uniform over the wave
@@ -591,7 +596,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             if (ln == 0) { pr[kHeadDim] = m_run[r]; pr[kHeadDim + 1] = l_run[r]; }
         }
     }
-    __syncthreads();
+    lds_barrier();                 // the loads of R above stay in flight
 
     {   // merge: thread -> (vector tid / 32, coordinates 4 * (tid % 32) .. +3); vector = (local KV head, query head)
         const int vec = tid >> 5, k4 = (tid & 31) * 4;
@@ -617,7 +622,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         }
         *reinterpret_cast<float4*>(&o_s[vec][k4]) = o4;
     }
-    __syncthreads();
+    lds_barrier();
 
     // ---- out[vector][d] = sum_k o[vector][k] R[k][d]; lane group kk owns k in [32kk, 32kk+32)
     for (int vt = wave >> 3; vt * 16 < nv; vt += 2) {
