@@ -175,6 +175,12 @@ void tw_kv_set_prefill_form(int form);
  * workgroup's work however long it is; 1: whenever the shape allows it (contiguous compressed cache, GQA group 1, 2
  * or 4); 2: never.  Process-wide. */
 void tw_kv_set_decode_fused(int mode);
+/* The choice mode 0 makes, as a pure function of what the host knows (1 = one launch, 0 = three): G sequences,
+ * cache width `bits`, max_seq_len, and the range of positions + 1 (ctx_max = 0: unknown).  One launch when every
+ * wave gets at most 8 tiles of 32 tokens, or when the lengths are within 1/8 of each other, the batch gives at
+ * least half the CUs a workgroup and the launch stays under ~1M tokens (256k at 2 bit with 8 KV heads).
+ * Alignment of the buffers, which the entry point also checks, is not part of it. */
+int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max);
 /* Layer steps that took the one-launch kernel since the library was loaded (launches issued or recorded into a
  * graph under capture): lets a benchmark say which kernel its figures belong to. */
 long long tw_kv_decode_fused_launches(void);

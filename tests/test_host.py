@@ -93,3 +93,34 @@ def test_host_rotation_is_the_fixture(rotation_fixture):
     from triebwerk_amd import kvcache
     r = kvcache.make_rotation(128, 42).numpy()
     assert np.array_equal(r.view(np.uint16), rotation_fixture.view(np.uint16))
+
+
+def test_decode_step_plan_is_the_documented_rule():
+    """Which decode-step form mode 0 picks, from host knowledge alone (no GPU needed: without a device the
+    library assumes 256 compute units, the MI355X's number)."""
+    from triebwerk_amd import _lib
+    lib = _lib.load()
+    plan = lib.tw_kv_decode_step_plan
+    # the benchmark's target: 64 sequences of 8192 tokens, lengths known and equal -> one launch at 4 bit,
+    # three at 2 bit (the cooperative 2-bit scan streams faster at that size)
+    assert plan(64, 16, 8, 4, 8448, 8192, 8192) == 1
+    assert plan(64, 16, 8, 2, 8448, 8192, 8192) == 0
+    # the same batch with nothing known about the lengths, or known to be ragged: three launches
+    assert plan(64, 16, 8, 4, 8448, 0, 0) == 0
+    assert plan(64, 16, 8, 4, 8448, 512, 8192) == 0
+    # short contexts by max_seq_len alone: at most 8 tiles per wave (2 heads per workgroup -> 8 parts of 256 tokens)
+    assert plan(64, 16, 8, 4, 2048, 0, 0) == 1
+    assert plan(64, 16, 8, 4, 2049, 0, 0) == 0
+    # a rollout: 128 sequences a few hundred tokens long, at either width
+    assert plan(128, 16, 8, 4, 1536, 300, 300) == 1
+    assert plan(128, 16, 8, 2, 1536, 300, 300) == 1
+    # small batches: one head per workgroup, 16 parts; long contexts of few sequences do not fill the GPU
+    assert plan(4, 16, 8, 4, 640, 0, 0) == 1
+    assert plan(4, 16, 8, 4, 16384, 16000, 16000) == 0
+    assert plan(16, 32, 8, 2, 4352, 4097, 4097) == 1          # 2 bit, GQA 4, 65k tokens
+    # beyond a million tokens per launch the three-kernel path has caught up
+    assert plan(256, 16, 8, 4, 8448, 8192, 8192) == 0
+    # shapes the one-launch kernel does not take
+    assert plan(64, 64, 8, 4, 1024, 0, 0) == 0                # GQA group 8
+    assert plan(64, 16, 8, 3, 1024, 0, 0) == 0
+    assert plan(0, 16, 8, 4, 1024, 0, 0) == 0

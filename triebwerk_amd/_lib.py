@@ -63,6 +63,7 @@ SIGNATURES = {
     "tw_kv_set_prefill_form": (None, [I]),
     "tw_kv_set_decode_fused": (None, [I]),
     "tw_kv_decode_fused_launches": (LL, []),
+    "tw_kv_decode_step_plan": (I, [I, I, I, I, I, I, I]),
     "tw_kv_profile_attention": (None, [I]),
     "tw_kv_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_kv_measure_read_bandwidth": (C.c_double, [P, C.c_size_t, I, P]),

@@ -195,6 +195,21 @@ int tw_kv_get_attention_variant(void) { return g_variant.load(); }
 void tw_kv_set_num_splits(int n) { g_nsplit_override.store(n); }
 void tw_kv_set_prefill_form(int form) { g_prefill_form.store(form); }
 void tw_kv_set_decode_fused(int mode) { g_decode_fused.store(mode); }
+
+int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max) {
+    if (G <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || (bits != 2 && bits != 4)) return 0;
+    const int group = num_heads / num_kv_heads;
+    if (group != 1 && group != 2 && group != 4) return 0;
+    const int hkw = decode_fused_heads_per_workgroup(G, num_kv_heads);
+    const int split = 16 / hkw;                                   // parts of the context per head: waves / heads
+    const long long units = (long long)G * (num_kv_heads / hkw);  // workgroups
+    const bool known = ctx_max > 0;
+    const int bound = known ? ctx_max : max_seq_len;
+    if (bound <= 256 * split) return 1;                           // at most 8 tiles of 32 tokens per wave
+    if (!known || (long long)(ctx_max - ctx_min) * 8 > ctx_max || units * 2 < compute_units_host()) return 0;
+    const long long tokens = (long long)G * ctx_max;
+    return tokens <= ((bits == 2 && num_kv_heads == 8) ? (256LL << 10) : (1LL << 20)) ? 1 : 0;
+}
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }
 
 void tw_kv_profile_attention(int enable) {
@@ -560,19 +575,7 @@ static bool try_decode_fused(const AttnArgs& a, const FusedArgs& f, int msl, hip
     const int mode = g_decode_fused.load();
     if (mode == 2 || g_variant.load() == 1) return false;
     if (!decode_fused_usable(a, f)) return false;
-    if (mode == 0) {
-        const int hkw = decode_fused_heads_per_workgroup(a.G, a.num_kv_heads);
-        const int split = 16 / hkw;
-        const long long units = (long long)a.G * (a.num_kv_heads / hkw);
-        const bool known = t_ctx_max > 0;
-        const int bound = known ? t_ctx_max : msl;
-        bool take = bound <= 256 * split;
-        if (!take && known && (long long)(t_ctx_max - t_ctx_min) * 8 <= t_ctx_max && units * 2 >= compute_units_host()) {
-            const long long tokens = (long long)a.G * t_ctx_max;
-            take = tokens <= ((a.bits == 2 && a.num_kv_heads == 8) ? (256LL << 10) : (1LL << 20));
-        }
-        if (!take) return false;
-    }
+    if (mode == 0 && !tw_kv_decode_step_plan(a.G, a.num_heads, a.num_kv_heads, a.bits, msl, t_ctx_min, t_ctx_max)) return false;
     attach_profiler(s);
     g_fused_launches.fetch_add(1);
     launch_decode_fused(a, f, s);
