@@ -288,9 +288,11 @@ merge_rotate_kernel(AttnArgs a) {
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const int c = c0 + j;
-                // else: no workgroup wrote this slot
+                // else: no workgroup wrote this slot.  The address does not wait for that answer (it needs the
+                // partial count or the position, loads of their own): every slot the workspace has room for may be
+                // read, whatever it holds is dropped below.
                 const bool live = c < nslots && (nseg > 0 || chunk_nonempty(n, c, a.nsplit));
-                const float* pc = part + (long long)(live ? c : 0) * kPartialFloats;
+                const float* pc = part + (long long)(c < a.max_slots ? c : 0) * kPartialFloats;
                 mc[j] = pc[kHeadDim];
                 lc[j] = pc[kHeadDim + 1];
                 pc4[j] = *reinterpret_cast<const float4*>(pc + k4);
