@@ -16,9 +16,8 @@
 //      cache, the scaled q_rot in LDS;
 //   2. after the barrier wave w scans every SPLIT-th tile of the context (SPLIT = 16 / HKW, starting at tile
 //      w / HKW) for head w % HKW with the loop of attention_mfma_kernel (the table look-ups, MFMA tiling,
-//      online softmax are described there).  Loads of a tile that holds the new token's row are only issued
-//      after the barrier (the row was stored by this workgroup: same CU, same L1); a first tile before it is
-//      requested up front;
+//      online softmax are described there).  All its loads are issued after the barrier: the new token's row
+//      was stored by this workgroup (same CU, same L1), which a workgroup-scope barrier makes visible;
 //   3. the partial results meet in LDS: merge (log-sum-exp), "+1e-8" normalisation, and R^T with the MFMA
 //      chain of merge_rotate_kernel; output gate as there.
 // The waves in the upper wave slots of a CU run ~5 % slower (see kv_common.hpp: kPairShare), so the parts
@@ -170,10 +169,10 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const int first_tile = tile_at(0);
 
     // ---- scan set-up (as attention_mfma_kernel, contiguous layout)
-    // Per-lane offsets and selectors.  They are derived twice, before the rotations (for the loads issued up
-    // front) and after them from a laundered copy of the lane number, so that the two sets are separate values:
-    // otherwise they stay live across the rotations, the allocator spills some of them there and reloads them
-    // inside the scan loop, where a reload waits for every load in flight.
+    // Per-lane offsets and selectors.  They are derived after the rotations from a laundered copy of the lane
+    // number: computed from the lane number itself they are hoisted to the top of the kernel, stay live across
+    // the rotations, and the allocator spills some of them there and reloads them inside the scan loop, where a
+    // reload waits for every load in flight.
     const char* tab_lane = reinterpret_cast<const char*>(tab_s);
     const uint32_t kvp = (uint32_t)Hk * kHeadBytes;
     const uint32_t nrow = (uint32_t)Hk * 2u;
@@ -200,7 +199,6 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         p_w = &p_s[wave][0][8 * (ln_ >> 2) + 4 * my_sub + (ln_ & 3)];
         p_r = reinterpret_cast<const uint4*>(&p_s[wave][ln_][8 * kg_]);
     };
-    derive_lane(lane);
     constexpr float kRaise = 5.0f;
 
     auto lut32 = [&](uint32_t addr) -> uint32_t { return *reinterpret_cast<const uint32_t*>(tab_lane + addr); };
@@ -266,13 +264,10 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     uint32_t kreg[2][KW];
     uint32_t vreg[2][VW];
     uint32_t nreg = 0;
-    // The first tile is requested now unless it holds the row this workgroup is about to store.
-    const bool early = ntiles > 0 && first_tile + 32 < n;
-    if (early) {
-        issue_k(kreg, first_tile);
-        nreg = issue_n(first_tile);
-        issue_v(vreg, first_tile);
-    }
+    // (Tiles are only requested after the rotations.  Asking for the first one up front, where it does not hold
+    // the row this workgroup is about to store, made short contexts 0.5 us slower per launch and long ones no
+    // faster; pulling further tiles towards the caches during the prologue cost 2 us per tile: what the
+    // prologue waits for then queues behind them.)
 
     // ---- 1. rotations of the unit's vectors
     {
@@ -406,11 +401,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
 
     if (ntiles > 0) {
-        if (!early) {
-            issue_k(kreg, first_tile);
-            nreg = issue_n(first_tile);
-            issue_v(vreg, first_tile);
-        }
+        issue_k(kreg, first_tile);
+        nreg = issue_n(first_tile);
+        issue_v(vreg, first_tile);
         // A operand of the score MFMAs: q_rot[head][32kg + 8j + i], row m = fp16 value of head m, row m + 8
         // its rounding remainder; the 2-bit table returns the codes of a byte in the order 0,2,1,3
         half8_t aq[4];
