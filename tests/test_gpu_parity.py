@@ -477,6 +477,53 @@ def test_decode_step_in_one_launch(kv, oracle, rotation_fixture, bits, H, Hk, le
 
 
 @pytest.mark.parametrize("bits", [4, 2])
+@pytest.mark.parametrize("G,H,Hk,producers", [(64, 16, 8, False), (128, 16, 8, True), (256, 16, 8, False), (264, 32, 8, True),
+                                              (520, 8, 8, False), (130, 8, 2, True)])
+def test_decode_step_in_one_launch_every_head_grouping(kv, oracle, rotation_fixture, bits, G, H, Hk, producers):
+    """The one-launch step with 2, 4 and 8 KV heads per workgroup (batches of 64, 128 and 256 and more sequences on a
+    256-CU GPU; 8 heads make units of more than 16 vectors, two rotation tiles), batch sizes that are and are not
+    multiples of 8 (the workgroup numbering differs), with and without the producers: cache bytes and outputs
+    against the oracle."""
+    import torch
+    r = gen.rng(950 + bits + G)
+    msl = 96
+    kv_dim, q_dim = Hk * D, H * D
+    lens = [int(x) for x in r.integers(0, msl - 1, size=G)]
+    lens[0], lens[1], lens[G - 1] = 0, msl - 1, 33
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits, outliers=False)
+    pos = np.array(lens, np.int32)
+    q, k, qw, kw = producer_inputs(r, G, H, Hk, q_dim, kv_dim)
+    v = gen.normal_f16(r, (G, kv_dim))
+    ct, st = rope_tables(msl, 128)
+    d_ck, d_cv, d_kn, d_vn = dev(ck), dev(cv), dev(kn), dev(vn)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    launches = kv._lib.load().tw_kv_decode_fused_launches()
+    kv.set_decode_fused(1)
+    try:
+        if producers:
+            kv.tw_qk_norm_rope_turbo_append_attention_batch(
+                out, dev(q), dev(k), dev(v), dev(qw), dev(kw), 1e-6, False, dev(ct), dev(st), 128, d_ck, d_cv, d_kn, d_vn,
+                dev(rotation_fixture), scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
+        else:
+            kv.tw_turbo_append_attention_batch(out, dev(q), dev(k), dev(v), d_ck, d_cv, d_kn, d_vn, dev(rotation_fixture),
+                                               scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    finally:
+        kv.set_decode_fused(0)
+    assert kv._lib.load().tw_kv_decode_fused_launches() == launches + 1      # it was the one-launch kernel
+    if producers:
+        oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, G, 1e-6, q_dim, kv_dim, False)
+        oracle.rope_batch(q, k, ct, st, pos, msl, G, H, Hk, D, q_dim, kv_dim, 128)
+    oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(cv, vn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    assert_bytes_equal(host(d_ck), ck, "K codes"); assert_bytes_equal(host(d_cv), cv, "V codes")
+    assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+    assert rel_err(host(out), want) <= TOL
+
+
+@pytest.mark.parametrize("bits", [4, 2])
 def test_turbo_attention_single_and_tiny_scratch(kv, oracle, rotation_fixture, bits):
     """Single-sequence entry point; max_seq_len 40 leaves no room for split partials."""
     r = gen.rng(320 + bits)
