@@ -31,6 +31,7 @@
 #include "kv_kernels.hpp"
 #include "kv_mfma_util.hpp"
 #include "kv_producer_util.hpp"
+#include "kv_rotate_util.hpp"
 
 namespace twkv {
 
@@ -45,16 +46,6 @@ constexpr int kFusedMaxQ = 32;                 // query heads of a unit: HKW * R
 constexpr int kRowFloats = kHeadDim + 4;       // LDS row of a vector: conflict-free 16-byte accesses
 constexpr int kStageStride = 2 * kHeadDim + 16;   // bytes per staged fp16 vector
 static_assert(8 * (2 + 4) * kStageStride <= kFusedMaxQ * kRowFloats * 4, "staged vectors fit the output rows");
-
-__device__ __forceinline__ float pick_half16(const uint4& piece, int e, int kk) {
-    uint32_t lo = e ? piece.z : piece.x;
-    uint32_t hi = e ? piece.w : piece.y;
-    uint32_t w = (kk & 2) ? hi : lo;
-    w = (kk & 1) ? (w >> 16) : (w & 0xffffu);
-    union { uint16_t u; half_t h; } cv;
-    cv.u = (uint16_t)w;
-    return (float)cv.h;
-}
 
 }  // namespace
 
@@ -122,8 +113,8 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
 #pragma unroll
         for (int q = 0; q < 16; q++) {
             uint4 rp = rsrc[q];
-            rv[2 * q] = pick_half16(rp, 0, kg);
-            rv[2 * q + 1] = pick_half16(rp, 1, kg);
+            rv[2 * q] = pick_half(rp, 0, kg);
+            rv[2 * q + 1] = pick_half(rp, 1, kg);
         }
     }
 
@@ -333,24 +324,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             const half_t* xrow = reinterpret_cast<const half_t*>(x_s + vc * kStageStride) + kk;
 #pragma unroll
             for (int s2 = 0; s2 < 32; s2++) xv[s2] = (float)xrow[4 * s2];
-            // sum of squares in the reference's order (kernels.cu:1509-1520), as rotate_kernel: xv[s] is
-            // coordinate 4s + kk; offsets 16, 8, 4 of the 32-lane tree stay inside a lane, 2 and 1 cross lanes
-            auto tree_sum_sq = [&]() -> float {
-                float sgrp[4];
-#pragma unroll
-                for (int w = 0; w < 4; w++) {
-                    float t[8];
-#pragma unroll
-                    for (int j = 0; j < 8; j++) t[j] = xv[8 * w + j] * xv[8 * w + j];
-                    float a0 = t[0] + t[4], a1 = t[1] + t[5], a2 = t[2] + t[6], a3 = t[3] + t[7];
-                    float b0 = a0 + a2, b1 = a1 + a3;
-                    float c = b0 + b1;
-                    float d = c + __shfl_xor(c, 32, 64);
-                    sgrp[w] = d + __shfl_xor(d, 16, 64);
-                }
-                return (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
-            };
-            const float n2 = tree_sum_sq();
+            const float n2 = rotation_tree_sum_sq(xv);                 // the reference's order, as rotate_kernel
             if (!is_query) {
                 const float inv = 1.0f / sqrtf(n2 + 1e-12f);
 #pragma unroll

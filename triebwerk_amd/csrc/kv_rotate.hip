@@ -27,22 +27,11 @@
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
+#include "kv_rotate_util.hpp"
 
 namespace twkv {
 
 namespace {
-
-// fp16 at index (4s + kk) of a row held as 16 x (8 halves): s = 2*q + e picks dword
-// (2e + kk/2) of 16-byte piece q, half kk%2.
-__device__ __forceinline__ float pick_half(const uint4& piece, int e, int kk) {
-    uint32_t lo = e ? piece.z : piece.x;
-    uint32_t hi = e ? piece.w : piece.y;
-    uint32_t w = (kk & 2) ? hi : lo;
-    w = (kk & 1) ? (w >> 16) : (w & 0xffffu);
-    union { uint16_t u; half_t h; } cv;
-    cv.u = (uint16_t)w;
-    return (float)cv.h;
-}
 
 // Rotary embedding of a vector held as xv[s] = coordinate 4s + kk: coordinate d < HALF pairs with d + HALF
 // (same lane, HALF4 = HALF / 4 registers further on); fp16 rounding as in rope_batch_kernel
@@ -128,29 +117,11 @@ rotate_kernel(RotArgs a) {
         }
     }
 
-    // sum of squares in the reference's order: xv[s] is coordinate 4s + kk; group w holds s = 8w..8w+7
-    auto tree_sum_sq = [&]() -> float {
-        float sgrp[4];
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-            float t[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) t[j] = xv[8 * w + j] * xv[8 * w + j];
-            // offset 16: positions i and i+16 are local j and j+4; offset 8: j and j+2; offset 4: j and j+1
-            float a0 = t[0] + t[4], a1 = t[1] + t[5], a2 = t[2] + t[6], a3 = t[3] + t[7];
-            float b0 = a0 + a2, b1 = a1 + a3;
-            float c = b0 + b1;                                   // c_kk of the tree
-            float d = c + __shfl_xor(c, 32, 64);                 // offset 2: c0+c2 | c1+c3
-            sgrp[w] = d + __shfl_xor(d, 16, 64);                 // offset 1: d0+d1
-        }
-        return (sgrp[0] + sgrp[2]) + (sgrp[1] + sgrp[3]);
-    };
-
     // ---- optional producers: per-head RMSNorm (kernels.cu:880-923), then rotary embedding (927-961),
     // each rounded to fp16 as the in-place kernels of the reference leave it
     if (a.seg_weight[seg]) {
 #pragma clang fp contract(off)      // (x * rms) * w: two fp32 roundings, then the one to fp16
-        const float rms = 1.0f / sqrtf(tree_sum_sq() / (float)kHeadDim + a.eps);
+        const float rms = 1.0f / sqrtf(rotation_tree_sum_sq(xv) / (float)kHeadDim + a.eps);
         const uint4* wsrc = reinterpret_cast<const uint4*>(a.seg_weight[seg]);
 #pragma unroll
         for (int q = 0; q < 16; q++) {
@@ -173,7 +144,7 @@ rotate_kernel(RotArgs a) {
 
     float n2 = 0.0f;
     if (!is_query) {
-        n2 = tree_sum_sq();
+        n2 = rotation_tree_sum_sq(xv);
         const float inv = 1.0f / sqrtf(n2 + 1e-12f);
 #pragma unroll
         for (int s = 0; s < 32; s++) xv[s] *= inv;
