@@ -20,10 +20,16 @@
 //   A operand = R rows   : lane (i = lane%16, kk = lane/16) holds R[d0+i][4s+kk], s = 0..31
 //   B operand = vectors  : the same lane holds u[v0+i][4s+kk]
 //   D[16 x 16]           : lane holds y[d0 + 4*(lane/16) + r][v0 + lane%16], r = 0..3
-// A wave needs nothing from any other wave (no LDS, no barrier), so a launch is
-// ceil(vectors/16) * 8 independent single-wave workgroups that spread over the chip;
-// that matters because these launches are small (a few thousand vectors) and
-// latency-bound.
+// A wave needs nothing from any other wave, so a launch is ceil(vectors/16) * 8 independent single-wave
+// workgroups that spread over the chip; that matters because the launches of a decode step are small (a few
+// thousand vectors) and latency-bound.  The 8 waves that share a tile of vectors are numbered so that they land
+// on one XCD (workgroup b runs on XCD b % 8), whose L2 then serves 7 of their 8 reads of it.
+//
+// Operand loads.  In the MFMA layout a lane wants every fourth half of a 256-byte row, and 16 lanes want 16
+// different rows: asked for directly that is 16 loads per lane of which a quarter is used, each touching 16
+// cache lines, and the address path of the CU becomes the limit of a big launch.  So a tile (16 rows, 4 KB)
+// comes in as 4 fully used 16-byte pieces per lane, is written to LDS with the halves regrouped
+// ([kk][row][s]), and each lane reads back its 32 halves as 4 x 16 bytes.
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
@@ -48,11 +54,47 @@ __device__ __forceinline__ void rope_registers(float (&xv)[32], const uint4 (&cp
     }
 }
 
+// An operand tile in LDS: row kk * 16 + i holds the halves 4s + kk, s = 0..31, of row i of the tile; 16 bytes
+// of padding per row keep the 16-byte reads of 16 lanes on different banks.
+constexpr int kOperandRow = 20;                           // dwords
+
+// raw[j] = 16-byte piece j * 64 + lane of the tile (piece q = lane % 16 of row 4j + lane / 16): its halves
+// e and 4 + e go to row e * 16 + (4j + lane / 16), dword q.
+__device__ __forceinline__ void stage_operand_tile(uint32_t* tile, const uint4 (&raw)[4], int lane) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t* dst = tile + (4 * j + (lane >> 4)) * kOperandRow + (lane & 15);
+        dst[0 * 16 * kOperandRow] = (raw[j].x & 0xffffu) | (raw[j].z << 16);
+        dst[1 * 16 * kOperandRow] = (raw[j].x >> 16) | (raw[j].z & 0xffff0000u);
+        dst[2 * 16 * kOperandRow] = (raw[j].y & 0xffffu) | (raw[j].w << 16);
+        dst[3 * 16 * kOperandRow] = (raw[j].y >> 16) | (raw[j].w & 0xffff0000u);
+    }
+}
+
+// Lane kk * 16 + i reads row kk * 16 + i: out[s] = coordinate 4s + kk of row i.
+__device__ __forceinline__ void read_operand_tile(const uint32_t* tile, int lane, float (&out)[32]) {
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const uint4 p = *reinterpret_cast<const uint4*>(tile + lane * kOperandRow + 4 * t);
+        const uint32_t w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            union { uint32_t u; half_t h[2]; } cv;
+            cv.u = w[e];
+            out[8 * t + 2 * e] = (float)cv.h[0];
+            out[8 * t + 2 * e + 1] = (float)cv.h[1];
+        }
+    }
+}
+
 }  // namespace
 
-template <int BITS>
+// PROD: the producers of q and k may be switched on (their operands cost 64 registers and a third of the
+// occupancy, which only the big launches of a prompt notice).
+template <int BITS, bool PROD>
 __global__ void __launch_bounds__(kWave)
 rotate_kernel(RotArgs a) {
+    __shared__ __attribute__((aligned(16))) uint32_t x_s[kWave * kOperandRow];
     const int lane = threadIdx.x;
     const int i16 = lane & 15, kk = lane >> 4;
 
@@ -60,50 +102,71 @@ rotate_kernel(RotArgs a) {
     int unit = blockIdx.x;
     int seg = 0;
     while (seg < a.nseg - 1 && unit >= a.seg_units[seg]) { unit -= a.seg_units[seg]; seg++; }
-    const int dblk = unit & 7;
-    const int vgroup = unit >> 3;
+    // Units of a segment in blocks of 64 = 8 tile groups x 8 coordinate blocks, the coordinate blocks of one
+    // tile group 8 workgroups apart (same XCD; every segment starts at a multiple of 8); what is left over at the
+    // end of the segment is numbered plainly.
+    int dblk = unit & 7, vgroup = unit >> 3;
+    if (unit < (a.seg_units[seg] >> 6) << 6) {
+        vgroup = (unit >> 6) * 8 + (unit & 7);
+        dblk = (unit >> 3) & 7;
+    }
     const int nvec = a.seg_nvec[seg];
     const int heads = a.seg_heads[seg];                  // head vectors per source row
     const bool is_query = a.seg_kind[seg] != 0;
-    const bool roped = a.seg_rope[seg] != 0;
+    const bool roped = PROD && a.seg_rope[seg] != 0;
 
-    // ---- A operand, once per wave: R row d0 + i16 as 16 pieces of 8 halves
-    const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (dblk * 16 + i16) * kHeadDim);
-    float rv[32];
+    // ---- A operand, once per wave: R rows d0 .. d0 + 15 (4 KB in a row); requested now, staged after the
+    // first tile of vectors has been requested too
+    uint4 raw[4];
 #pragma unroll
-    for (int q = 0; q < 16; q++) {
-        uint4 rp = rsrc[q];
-        rv[2 * q] = pick_half(rp, 0, kk);
-        rv[2 * q + 1] = pick_half(rp, 1, kk);
-    }
+    for (int j = 0; j < 4; j++)
+        raw[j] = reinterpret_cast<const uint4*>(a.rotation + dblk * 16 * kHeadDim)[j * kWave + lane];
+
+    // 16-byte piece j * 64 + lane of a tile of vectors: piece lane % 16 of vector 4j + lane / 16
+    const half_t* src = a.seg_src[seg];
+    const long long stride = a.seg_stride[seg];
+    auto request_tile = [&](int vtile, uint4 (&dst)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int vi = min(vtile * 16 + 4 * j + (lane >> 4), nvec - 1);
+            const int ri = vi / heads, hi = vi - ri * heads;
+            dst[j] = reinterpret_cast<const uint4*>(src + (long long)ri * stride + (long long)hi * kHeadDim)[lane & 15];
+        }
+    };
+    const int vtile0 = vgroup * a.nper;
+    if (vtile0 * 16 >= nvec) return;
+    uint4 xraw[4];
+    request_tile(vtile0, xraw);
+
+    float rv[32];
+    stage_operand_tile(x_s, raw, lane);
+    lds_barrier();
+    read_operand_tile(x_s, lane, rv);
 
     // Small launches (decode) give every wave one tile of 16 vectors; large ones (prompts) let a wave keep
-    // its rows of R and walk a.nper tiles.
+    // its rows of R and walk a.nper tiles, the next tile requested while this one is worked on.
     for (int it = 0; it < a.nper; it++) {
-    const int vtile = vgroup * a.nper + it;
+    const int vtile = vtile0 + it;
     if (vtile * 16 >= nvec) break;
     const int v = vtile * 16 + i16;
     const int vc = v < nvec ? v : nvec - 1;              // clamp loads, mask stores
     const int row = vc / heads, head = vc - row * heads;
 
-    // ---- B operand: source vector v as 16 pieces of 8 halves
-    const uint4* xsrc = reinterpret_cast<const uint4*>(a.seg_src[seg] + (long long)row * a.seg_stride[seg] +
-                                                       (long long)head * kHeadDim);
-    // position of this vector's row: needed for the cache row and for the rotary table row, so it is the
-    // first thing asked for; everything that depends on it is requested before the operands are used
+    // position of this vector's row: needed for the cache row and for the rotary table row, so it is asked for
+    // early; everything that depends on it is requested before the operands are used
     const int pos_row = (!is_query || roped) ? a.positions[row] : 0;
     long long crow = 0;
     if (!is_query) {
         if (a.token_list) crow = pos_row;                                // sequence 0, kernels.cu:1499, 1553
         else crow = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, row, pos_row);
     }
+    // ---- B operand: the tile's vectors through LDS
+    lds_barrier();                                        // the reads of the previous tile (or of R) are done
+    stage_operand_tile(x_s, xraw, lane);
+    if (it + 1 < a.nper) request_tile(vtile + 1, xraw);   // clamped to the last vector: never out of bounds
+    lds_barrier();
     float xv[32];
-#pragma unroll
-    for (int q = 0; q < 16; q++) {
-        uint4 xp = xsrc[q];
-        xv[2 * q] = pick_half(xp, 0, kk);
-        xv[2 * q + 1] = pick_half(xp, 1, kk);
-    }
+    read_operand_tile(x_s, lane, xv);
 
     // rotary table row of this position: rope_dim / 2 halves = rope_dim / 16 pieces
     uint4 cpiece[8], spiece[8];
@@ -119,7 +182,7 @@ rotate_kernel(RotArgs a) {
 
     // ---- optional producers: per-head RMSNorm (kernels.cu:880-923), then rotary embedding (927-961),
     // each rounded to fp16 as the in-place kernels of the reference leave it
-    if (a.seg_weight[seg]) {
+    if (PROD && a.seg_weight[seg]) {
 #pragma clang fp contract(off)      // (x * rms) * w: two fp32 roundings, then the one to fp16
         const float rms = 1.0f / sqrtf(rotation_tree_sum_sq(xv) / (float)kHeadDim + a.eps);
         const uint4* wsrc = reinterpret_cast<const uint4*>(a.seg_weight[seg]);
@@ -205,8 +268,15 @@ void launch_rotate(const RotArgs& args, int bits, hipStream_t s) {
         units += a.seg_units[i];
     }
     if (units <= 0) return;
-    if (bits == 4) hipLaunchKernelGGL(rotate_kernel<4>, dim3(units), dim3(kWave), 0, s, a);
-    else hipLaunchKernelGGL(rotate_kernel<2>, dim3(units), dim3(kWave), 0, s, a);
+    bool prod = false;
+    for (int i = 0; i < a.nseg; i++) prod = prod || a.seg_weight[i] != nullptr || a.seg_rope[i] != 0;
+    if (bits == 4) {
+        if (prod) hipLaunchKernelGGL((rotate_kernel<4, true>), dim3(units), dim3(kWave), 0, s, a);
+        else hipLaunchKernelGGL((rotate_kernel<4, false>), dim3(units), dim3(kWave), 0, s, a);
+    } else {
+        if (prod) hipLaunchKernelGGL((rotate_kernel<2, true>), dim3(units), dim3(kWave), 0, s, a);
+        else hipLaunchKernelGGL((rotate_kernel<2, false>), dim3(units), dim3(kWave), 0, s, a);
+    }
 }
 
 // ---------------------------------------------------------------- split merge + rotate-back
@@ -259,11 +329,13 @@ merge_rotate_kernel(AttnArgs a) {
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const int c = c0 + j;
-                // else: no workgroup wrote this slot.  The address does not wait for that answer (it needs the
-                // partial count or the position, loads of their own): every slot the workspace has room for may be
-                // read, whatever it holds is dropped below.
+                // else: no workgroup wrote this slot.  With a fixed split (a decode step) the address does not wait
+                // for that answer, which needs the position, a load of its own: every slot the workspace has room
+                // for may be read, and what it holds is dropped below.  With the count in the workspace (a prompt,
+                // mostly one slot) only the slots written are read.
                 const bool live = c < nslots && (nseg > 0 || chunk_nonempty(n, c, a.nsplit));
-                const float* pc = part + (long long)(c < a.max_slots ? c : 0) * kPartialFloats;
+                const bool fetch = a.slots_from_ws ? live : c < a.max_slots;
+                const float* pc = part + (long long)(fetch ? c : 0) * kPartialFloats;
                 mc[j] = pc[kHeadDim];
                 lc[j] = pc[kHeadDim + 1];
                 pc4[j] = *reinterpret_cast<const float4*>(pc + k4);
