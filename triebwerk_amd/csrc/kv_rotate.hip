@@ -31,6 +31,9 @@
 // comes in as 4 fully used 16-byte pieces per lane, is written to LDS with the halves regrouped
 // ([kk][row][s]), and each lane reads back its 32 halves as 4 x 16 bytes.
 
+#include <algorithm>
+#include <type_traits>
+
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 #include "kv_rotate_util.hpp"
@@ -290,13 +293,12 @@ constexpr int kMergeVecs = 16;
 constexpr int kMergeStride = kHeadDim + 4;     // floats per LDS row: conflict-free 16-byte reads
 
 __global__ void __launch_bounds__(8 * kWave)
-merge_rotate_kernel(AttnArgs a) {
+merge_rotate_kernel(AttnArgs a, int nper) {
     __shared__ __attribute__((aligned(16))) float o_s[kMergeVecs][kMergeStride];
     const int tid = threadIdx.x;
     const int wave = tid / kWave, lane = tid % kWave;
     const int i16 = lane & 15, kk = lane >> 4;
     const int total = a.G * a.num_heads;
-    const int v0 = blockIdx.x * kMergeVecs;
 
     // B operand first (its loads overlap the merge): R[32kk + s][16*wave + i16], s = 0..31
     uint16_t rb[32];
@@ -305,6 +307,12 @@ merge_rotate_kernel(AttnArgs a) {
 #pragma unroll
         for (int s = 0; s < 32; s++) rb[s] = rp[s * kHeadDim];
     }
+
+    // A workgroup keeps its block of R and walks nper tiles of 16 vectors (1 in a decode step, more for a prompt).
+    for (int it = 0; it < nper; it++) {
+    const int v0 = (blockIdx.x * nper + it) * kMergeVecs;
+    if (v0 >= total) break;
+    if (it > 0) __syncthreads();                      // the previous tile's vectors have been read
 
     // ---- merge: thread -> (vector tid/32, coordinates 4*(tid%32) .. +3)
     {
@@ -317,22 +325,21 @@ merge_rotate_kernel(AttnArgs a) {
         else n = g + 1;
         const float* part = a.ws + (long long)vv * a.ws_stride;
         const int nseg = a.slots_from_ws ? reinterpret_cast<const int*>(part)[kHeadDim + 2] : 0;
-        // Chunks in blocks of 8 with every load of a block issued before the first use, so a
-        // block costs one memory latency rather than one per chunk; the running maximum is
-        // carried across blocks as in an online softmax.
+        // Slots in blocks with every load of a block issued before the first use, so a block costs one memory
+        // latency rather than one per slot; the running maximum is carried across blocks as in an online softmax.
         float mg = -1e30f, lsum = 0.0f;
         float4 av = {0.f, 0.f, 0.f, 0.f};
         const int nslots = nseg > 0 ? nseg : a.nsplit;
-        for (int c0 = 0; c0 < nslots; c0 += 8) {
-            float mc[8], lc[8];
-            float4 pc4[8];
+        auto merge_block = [&](int c0, auto width) {
+            constexpr int W = decltype(width)::value;
+            float mc[W], lc[W];
+            float4 pc4[W];
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
+            for (int j = 0; j < W; j++) {
                 const int c = c0 + j;
                 // else: no workgroup wrote this slot.  With a fixed split (a decode step) the address does not wait
                 // for that answer, which needs the position, a load of its own: every slot the workspace has room
-                // for may be read, and what it holds is dropped below.  With the count in the workspace (a prompt,
-                // mostly one slot) only the slots written are read.
+                // for may be read, and what it holds is dropped below.
                 const bool live = c < nslots && (nseg > 0 || chunk_nonempty(n, c, a.nsplit));
                 const bool fetch = a.slots_from_ws ? live : c < a.max_slots;
                 const float* pc = part + (long long)(fetch ? c : 0) * kPartialFloats;
@@ -343,12 +350,12 @@ merge_rotate_kernel(AttnArgs a) {
             }
             float mb = mg;
 #pragma unroll
-            for (int j = 0; j < 8; j++) mb = fmaxf(mb, mc[j]);
+            for (int j = 0; j < W; j++) mb = fmaxf(mb, mc[j]);
             const float fo = a.m_log2 ? __builtin_amdgcn_exp2f(mg - mb) : __expf(mg - mb);
             lsum *= fo; av.x *= fo; av.y *= fo; av.z *= fo; av.w *= fo;
             mg = mb;
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
+            for (int j = 0; j < W; j++) {
                 float f = a.m_log2 ? __builtin_amdgcn_exp2f(mc[j] - mg) : __expf(mc[j] - mg);
                 lsum = __builtin_fmaf(lc[j], f, lsum);
                 av.x = __builtin_fmaf(pc4[j].x, f, av.x);
@@ -356,6 +363,12 @@ merge_rotate_kernel(AttnArgs a) {
                 av.z = __builtin_fmaf(pc4[j].z, f, av.z);
                 av.w = __builtin_fmaf(pc4[j].w, f, av.w);
             }
+        };
+        // blocks of 8; a count of 1 or 2 (a prompt: the workspace says how many) is not padded to 8 loads
+        if (nslots <= 2) {
+            merge_block(0, std::integral_constant<int, 2>{});
+        } else {
+            for (int c0 = 0; c0 < nslots; c0 += 8) merge_block(c0, std::integral_constant<int, 8>{});
         }
         const float inv = 1.0f / (lsum + 1e-8f);
         float4 o4 = {av.x * inv, av.y * inv, av.z * inv, av.w * inv};
@@ -389,6 +402,7 @@ merge_rotate_kernel(AttnArgs a) {
             a.out[(long long)g * a.q_stride + col] = h;
         }
     }
+    }   // tiles of this workgroup
 }
 
 bool launch_merge_rotate(const AttnArgs& a, hipStream_t s) {
@@ -396,7 +410,10 @@ bool launch_merge_rotate(const AttnArgs& a, hipStream_t s) {
     if ((reinterpret_cast<uintptr_t>(a.ws) & 15u) != 0 || (a.ws_stride & 3) != 0) return false;
     const int total = a.G * a.num_heads;
     if (total <= 0) return true;
-    hipLaunchKernelGGL(merge_rotate_kernel, dim3((total + kMergeVecs - 1) / kMergeVecs), dim3(8 * kWave), 0, s, a);
+    // one tile per workgroup until there are 8 workgroups per CU, then up to 8
+    const int tiles = (total + kMergeVecs - 1) / kMergeVecs;
+    const int nper = std::max(1, std::min(8, tiles / 2048));
+    hipLaunchKernelGGL(merge_rotate_kernel, dim3((tiles + nper - 1) / nper), dim3(8 * kWave), 0, s, a, nper);
     return true;
 }
 
