@@ -661,18 +661,20 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     return true;
 }
 
-void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
+// Returns whether the output is finished (the prompt kernel normalises and rotates back itself); otherwise the
+// partials wait in the workspace for the merge.
+bool launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     if (prefill_tq_mfma_usable(a) && !(prefill_form() == 4 && prefill_mfma_usable(a))) {
         launch_prefill_tq_mfma(a, s, prefill_form());
-        return;
+        return true;
     }
     if (prefill_mfma_usable(a)) {
         launch_prefill_mfma_scan(a, s);
-        return;
+        return false;
     }
     if (attention_mfma2c_usable(a)) {
         launch_attention_mfma2c_scan(a, s);
-        return;
+        return false;
     }
     const int waves = scan_waves(a);
     const int hgroups = a.num_kv_heads / waves;
@@ -698,6 +700,7 @@ void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     }
 #undef TW_LAUNCH_R
 #undef TW_LAUNCH
+    return false;
 }
 
 }  // namespace twkv

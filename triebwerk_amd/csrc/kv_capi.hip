@@ -167,10 +167,11 @@ void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done =
         return;
     }
     const bool mfma = mfma_wanted(a) && prepare_attention_mfma(a, s, !query_done);   // (its query rotation is not a scan launch)
-    if (mfma) launch_attention_mfma_scan(a, s);
+    bool finished = false;
+    if (mfma) finished = launch_attention_mfma_scan(a, s);
     else launch_attention_valu(a, s);
     t_scan_start = t_scan_stop = nullptr;
-    if (a.nsplit > 1 || a.force_merge) {
+    if (!finished && (a.nsplit > 1 || a.force_merge)) {
         if (!(g_variant.load() != 1 && launch_merge_rotate(a, s))) launch_attention_merge(a, s);
     }
     check_launch(fn);

@@ -171,7 +171,7 @@ bool launch_merge_rotate(const AttnArgs& a, hipStream_t s);   // MFMA merge + ro
 // prepare = shape check + query rotation (false = shape not covered), then the scan.
 bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query);
 float attention_mfma_q_scale(int bits);
-void launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);
+bool launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s);   // true: the output is finished, no merge
 // One decode step of a layer in one launch (kv_decode_fused.hip): append the new K and V rows, rotate the
 // query, scan, merge and rotate back.  AttnArgs as for the batch decode over the contiguous compressed
 // cache (positions array; no workspace needed), plus the rows to append and the cache as writable pointers.

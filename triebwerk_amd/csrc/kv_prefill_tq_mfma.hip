@@ -9,8 +9,11 @@
 //   acc[q][d]   += (p * v_norm[kv]) * c(V code[kv][d])                        (kernels.cu:1765)
 // with q_rot = R q pre-scaled by log2(e) / sqrt(128) / alpha (rotate_kernel), centroids stored as
 // fp16(alpha c) (alpha as in the decode scan: all magnitudes round with <= 1.1e-4 relative error), the
-// norms applied in fp32.  The rotated accumulators go to the split workspace as one partial per
-// (query token, head); merge_rotate_kernel normalises and applies R^T.
+// norms applied in fp32.  A workgroup sees the whole context of its query tokens, so it also finishes them:
+// normalisation (kernels.cu:1946) and the rotation back out of the rotated space (kernels.cu:1949-1957) on the
+// matrix cores, the accumulator split into an fp16 value and its remainder; no partials, no merge launch.
+// The accumulators are kept transposed (O^T[dim][query], the operands of the second MFMA swapped), which puts a
+// query's running maximum, sum and accumulators in the same lanes and makes O^T the B operand of the rotation.
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
@@ -23,6 +26,9 @@ namespace {
 constexpr int kPtWaves = 4;
 constexpr int kPtKRow = 2 * kHeadDim + 16;   // bytes per expanded K row in LDS
 constexpr int kPtVRow = 2 * 32 + 16;         // bytes per V^T row (32 token slots) in LDS
+constexpr int kPtVTile = kHeadDim * kPtVRow; // bytes of a V^T tile
+constexpr int kPtVBytes = 2 * kHeadDim * kHeadDim;   // >= 3 tiles, and the 128 x 128 fp16 rotation
+static_assert(kPtVBytes >= 3 * kPtVTile, "three V tiles fit");
 
 // column of a tile's token in the V^T rows: the contraction slot order of the second MFMA
 __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 2) + 4 * (token >> 4) + (token & 3); }
@@ -40,7 +46,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
     constexpr int kEntryDwords = BITS == 4 ? 1 : 2;        // a byte holds 2 (4) codes -> 2 (4) halves
     constexpr int kPtReplicas = BITS == 4 ? 16 : 8;        // copies of the byte -> centroids table (16 KB either way): fewer bank conflicts in the expansion
     __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPtKRow];
-    __shared__ __attribute__((aligned(16))) char v_s[3][kHeadDim * kPtVRow];
+    __shared__ __attribute__((aligned(16))) char v_s[kPtVBytes];           // 3 V^T tiles; in the epilogue the rotation
     __shared__ __attribute__((aligned(16))) float n_s[3][2][32];          // [buffer][k | v][token]
     __shared__ __attribute__((aligned(8))) uint32_t tab_s[256 * kPtReplicas * kEntryDwords];
 
@@ -126,7 +132,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         uint32_t va[4], vb[4];
         expand8(st.v[0], va);
         expand8(st.v[1], vb);
-        char* dst = &v_s[vbuf][(8 * vc_) * kPtVRow + vcol];
+        char* dst = &v_s[vbuf * kPtVTile + (8 * vc_) * kPtVRow + vcol];
 #pragma unroll
         for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
@@ -174,16 +180,16 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
             for (int j = 0; j < 8; j++) o[nq][j] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
 
-        // ---- O[query][dim 16j + ln] += P . V for one tile (value and remainder of p * v_norm)
+        // ---- O^T[dim 16j + 4kg + i][query ln] += V^T . P^T for one tile (value and remainder of p * v_norm)
         auto pv = [&](int vbuf, const half8_t (&pa)[NQ], const half8_t (&pl)[NQ]) {
-            const char* vrow = &v_s[vbuf][ln * kPtVRow + 16 * kg];
+            const char* vrow = &v_s[vbuf * kPtVTile + ln * kPtVRow + 16 * kg];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPtVRow);
 #pragma unroll
                 for (int nq = 0; nq < NQ; nq++) {
-                    o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
-                    o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl[nq], vb, o[nq][j], 0, 0, 0);
+                    o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb, pa[nq], o[nq][j], 0, 0, 0);
+                    o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb, pl[nq], o[nq][j], 0, 0, 0);
                 }
             }
         };
@@ -262,10 +268,9 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
                         m_run[nq] = m_new;
                         l_run[nq] *= alpha;
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {      // accumulator register i belongs to query 4kg + i
-                            const float ai = __shfl(alpha, 4 * kg + i, 64);
+                        for (int j = 0; j < 8; j++) {      // the lane's accumulators all belong to query ln
 #pragma unroll
-                            for (int j = 0; j < 8; j++) o[nq][j][i] *= ai;
+                            for (int i = 0; i < 4; i++) o[nq][j][i] *= alpha;
                         }
                     }
 #pragma unroll
@@ -285,28 +290,72 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         }
         if (have_prev) pv((ntiles - 1) % 3, pa_prev, pl_prev);
 
-        // ---- one partial per (query token, head): rotated accumulator, running maximum (base 2) and sum;
-        // the merge normalises (kernels.cu:1946: 1 / (sum + 1e-8)) and rotates back.  Accumulator register i
-        // is query 4kg + i, maximum and sum sit in the lanes whose ln is the query.
+        // ---- epilogue: out[q][d] = sum_k R[k][d] o[q][k] / (sum + 1e-8) (kernels.cu:1946-1957) as
+        // out^T = R^T . O^T.  The rotation goes into the V buffers in operand order: 16-byte entry
+        // (db * 4 + t) * 64 + lane holds R[k][16 db + ln] for the 8 k that lane (ln, kg) carries in step t,
+        // k = 32t + 16 (e / 4) + 4kg + e % 4 -- the dims its accumulators o[.][2t + e / 4][e % 4] belong to.
+        __syncthreads();                                   // every wave is done with the V tiles
+        {
+            // thread -> rows k = 16r + tid / 16, r = 0..7, columns 8c .. 8c + 7 with c = tid % 16; of k only r is
+            // not fixed per thread, and r moves the destination by whole steps t = r / 2 and halves 4 (r % 2)
+            const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation) + tid;
+            const int krow = tid >> 4, c = tid & 15;
+            char* dst0 = &v_s[(c >> 1) * 4096 + ((krow >> 2) & 3) * 256 + (c & 1) * 128 + 2 * (krow & 3)];
+#pragma unroll
+            for (int r = 0; r < 8; r++) {
+                const uint4 rp = rsrc[r * (kPtWaves * kWave)];
+                const uint32_t w[4] = {rp.x, rp.y, rp.z, rp.w};
+#pragma unroll
+                for (int x = 0; x < 8; x++)
+                    *reinterpret_cast<uint16_t*>(dst0 + (r >> 1) * 1024 + (r & 1) * 8 + x * 16) = (uint16_t)(w[x >> 1] >> (16 * (x & 1)));
+            }
+        }
+        __syncthreads();
+        half8_t oh[NQ][4], ol[NQ][4];
 #pragma unroll
         for (int nq = 0; nq < NQ; nq++) {
             float l = l_run[nq];
             l += __shfl_xor(l, 16, 64);
             l += __shfl_xor(l, 32, 64);
-            const int tq = q0 + 16 * nq + ln;
-            if (kg == 0 && tq < T) {
-                float* part = a.ws + ((long long)tq * a.num_heads + head) * a.ws_stride;
-                part[kHeadDim] = m_run[nq];
-                part[kHeadDim + 1] = l;
-                reinterpret_cast<int*>(part)[kHeadDim + 2] = 1;          // one partial
+            const float inv = (1.0f / kAlpha) / (l + 1e-8f);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float x = o[nq][2 * t + (e >> 2)][e & 3] * inv;
+                    const half_t hi = (half_t)x;
+                    oh[nq][t][e] = hi;
+                    ol[nq][t][e] = (half_t)(x - (float)hi);
+                }
             }
+        }
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int t = q0 + 16 * nq + 4 * kg + i;
-                if (t < T) {
-                    float* part = a.ws + ((long long)t * a.num_heads + head) * a.ws_stride + ln;
+        for (int db = 0; db < 8; db++) {
+            float4_t y[NQ];
 #pragma unroll
-                    for (int j = 0; j < 8; j++) part[16 * j] = o[nq][j][i] * (1.0f / kAlpha);
+            for (int nq = 0; nq < NQ; nq++) y[nq] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const half8_t ra = *reinterpret_cast<const half8_t*>(&v_s[((db * 4 + t) * 64 + lane) * 16]);
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) {
+                    y[nq] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ra, oh[nq][t], y[nq], 0, 0, 0);
+                    y[nq] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ra, ol[nq][t], y[nq], 0, 0, 0);
+                }
+            }
+            // lane holds out[tq][head][16 db + 4kg + i], i = 0..3, of its query token tq
+#pragma unroll
+            for (int nq = 0; nq < NQ; nq++) {
+                const int tq = q0 + 16 * nq + ln;
+                if (tq < T) {
+                    const long long col = (long long)head * kHeadDim + 16 * db + 4 * kg;
+                    half_t h[4] = {(half_t)y[nq][0], (half_t)y[nq][1], (half_t)y[nq][2], (half_t)y[nq][3]};
+                    if (a.gate) {
+                        const half_t* grow = a.gate + (long long)tq * a.gate_stride + col;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) h[i] = gated(h[i], grow[i]);
+                    }
+                    *reinterpret_cast<uint2*>(a.out + (long long)tq * a.q_stride + col) = *reinterpret_cast<const uint2*>(h);
                 }
             }
         }
@@ -320,8 +369,10 @@ bool prefill_tq_mfma_usable(const AttnArgs& a) {
     if ((a.bits != 4 && a.bits != 2) || a.pos_mode != kPosIota || a.block_table || a.seq_stride_rows != 0) return false;
     if (R != 1 && R != 2 && R != 4) return false;
     const long long cache_bytes = (long long)a.G * a.num_kv_heads * a.bits * 16;      // one buffer descriptor spans it
+    // out is written 4 halves at a time, the rotation read 16 bytes at a time
     return a.ws && a.qrot && a.G >= 1 && (a.ws_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0 &&
-           cache_bytes < (1LL << 31);
+           (reinterpret_cast<uintptr_t>(a.out) & 7u) == 0 && (a.q_stride & 3) == 0 &&
+           (reinterpret_cast<uintptr_t>(a.rotation) & 15u) == 0 && cache_bytes < (1LL << 31);
 }
 
 void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form) {
