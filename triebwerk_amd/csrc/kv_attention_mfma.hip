@@ -627,6 +627,13 @@ float attention_mfma_q_scale(int bits) {
     return kLog2e * kInvSqrtD / (bits == 4 ? kAlpha4 : kAlpha2);
 }
 
+namespace {
+// a prompt over the compressed cache goes to the kernel that expands a tile once per workgroup
+bool takes_prefill_tq(const AttnArgs& a) {
+    return prefill_tq_mfma_usable(a) && !(prefill_form() == 4 && prefill_mfma_usable(a));
+}
+}  // namespace
+
 // Shape check; with rotate_query also q_rot = R q (kernels.cu:1671-1681) into the workspace.
 bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     const int R = a.num_heads / a.num_kv_heads;
@@ -642,7 +649,7 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     a.slots_from_ws = 1;
     // ragged batches: cut the work by tiles, not by sequence (decided on the device from the positions)
     a.balance = (a.num_kv_heads == scan_waves(a) && a.G <= kMaxBalanceSeqs && a.max_slots >= 3 && a.G > 1) ? 1 : 0;
-    if (rotate_query) {
+    if (rotate_query && !takes_prefill_tq(a)) {           // (that kernel rotates its queries itself)
         RotArgs r;
         memset(&r, 0, sizeof(r));
         r.nseg = 1;
@@ -664,7 +671,7 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
 // Returns whether the output is finished (the prompt kernel normalises and rotates back itself); otherwise the
 // partials wait in the workspace for the merge.
 bool launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
-    if (prefill_tq_mfma_usable(a) && !(prefill_form() == 4 && prefill_mfma_usable(a))) {
+    if (takes_prefill_tq(a)) {
         launch_prefill_tq_mfma(a, s, prefill_form());
         return true;
     }

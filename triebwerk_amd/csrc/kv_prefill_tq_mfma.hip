@@ -7,7 +7,7 @@
 // Arithmetic (turbo_gqa_prefill_attention_kernel, kernels.cu:1874-1960, in the rotated space):
 //   score[kv][q] = (sum_d c(K code[kv][d]) q_rot[q][d]) * k_norm[kv]          (kernels.cu:1707)
 //   acc[q][d]   += (p * v_norm[kv]) * c(V code[kv][d])                        (kernels.cu:1765)
-// with q_rot = R q pre-scaled by log2(e) / sqrt(128) / alpha (rotate_kernel), centroids stored as
+// with q_rot = R q pre-scaled by log2(e) / sqrt(128) / alpha (made in the kernel), centroids stored as
 // fp16(alpha c) (alpha as in the decode scan: all magnitudes round with <= 1.1e-4 relative error), the
 // norms applied in fp32.  A workgroup sees the whole context of its query tokens, so it also finishes them:
 // normalisation (kernels.cu:1946) and the rotation back out of the rotated space (kernels.cu:1949-1957) on the
@@ -42,6 +42,7 @@ __global__ void __launch_bounds__(kPtWaves* kWave, 2)        // two workgroups p
 prefill_tq_mfma_kernel(AttnArgs a, int T) {
     constexpr int TPW = 16 * NQ * kPtWaves / R;            // query tokens per workgroup pass
     constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
+    constexpr float kQScale = kLog2e * kInvSqrtD / kAlpha;   // score scale of kernels.cu:1707 in base 2, table scale undone
     constexpr int kHeadBytes = BITS * 16;                  // bytes of one head in a cache row
     constexpr int kEntryDwords = BITS == 4 ? 1 : 2;        // a byte holds 2 (4) codes -> 2 (4) halves
     constexpr int kPtReplicas = BITS == 4 ? 16 : 8;        // copies of the byte -> centroids table (16 KB either way): fewer bank conflicts in the expansion
@@ -154,20 +155,45 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
 
         // ---- B operands of the first MFMA: q_rot[q0 + 16 nq + ln][32j + 8kg .. +7], j = 0..3, as an fp16 value
         // and what its rounding left over (scores reach tens of base-2 units on caches with outlier channels,
-        // where a 2^-11 relative error of q alone would show in the output)
+        // where a 2^-11 relative error of q alone would show in the output).  q_rot = R q (kernels.cu:1671-1681)
+        // is made here, on the matrix cores: q_rot^T[d][query] = R[d][.] . q^T, 16 rows d at a time, the rows
+        // picked so that the result lands where the operand wants it -- accumulator row 4kg + i of block (j, h)
+        // is d = 32j + 8kg + 4h + i.  Both factors are exact in fp16 and the sum is kept in fp32.
         half8_t qb[NQ][4], ql[NQ][4];
+        {
+            half8_t qv[NQ][4];                             // q[query ln][32t + 8kg .. +7]
 #pragma unroll
-        for (int nq = 0; nq < NQ; nq++) {
-            const float* qrow = a.qrot + ((long long)min(q0 + 16 * nq + ln, T - 1) * a.num_heads + head) * a.ws_stride + 8 * kg;
+            for (int nq = 0; nq < NQ; nq++) {
+                const half_t* qsrc = a.q + (long long)min(q0 + 16 * nq + ln, T - 1) * a.q_stride + head * kHeadDim + 8 * kg;
+#pragma unroll
+                for (int t = 0; t < 4; t++) qv[nq][t] = *reinterpret_cast<const half8_t*>(qsrc + 32 * t);
+            }
+            int rrow = 8 * (ln >> 2) + (ln & 3);           // row of R this lane feeds within a block, less 32j + 4h
+            asm volatile("" : "+v"(rrow));                 // per pass: the 32 loads below are not kept across passes
+            const half_t* rsrc = a.rotation + rrow * kHeadDim + 8 * kg;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float4 v0 = *reinterpret_cast<const float4*>(qrow + 32 * j), v1 = *reinterpret_cast<const float4*>(qrow + 32 * j + 4);
-                const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const half_t hi = (half_t)v[i];
-                    qb[nq][j][i] = hi;
-                    ql[nq][j][i] = (half_t)(v[i] - (float)hi);
+                for (int h = 0; h < 2; h++) {
+                    float4_t y[NQ];
+#pragma unroll
+                    for (int nq = 0; nq < NQ; nq++) y[nq] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const half8_t ra = *reinterpret_cast<const half8_t*>(rsrc + (32 * j + 4 * h) * kHeadDim + 32 * t);
+#pragma unroll
+                        for (int nq = 0; nq < NQ; nq++) y[nq] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ra, qv[nq][t], y[nq], 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int nq = 0; nq < NQ; nq++) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const float x = y[nq][i] * kQScale;
+                            const half_t hi = (half_t)x;
+                            qb[nq][j][4 * h + i] = hi;
+                            ql[nq][j][4 * h + i] = (half_t)(x - (float)hi);
+                        }
+                    }
                 }
             }
         }
@@ -363,15 +389,15 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
 }
 
 
-// compressed cache, one sequence, query t attends rows 0..t, GQA group 1, 2 or 4, workspace with q_rot
+// compressed cache, one sequence, query t attends rows 0..t, GQA group 1, 2 or 4
 bool prefill_tq_mfma_usable(const AttnArgs& a) {
     const int R = a.num_heads / a.num_kv_heads;
     if ((a.bits != 4 && a.bits != 2) || a.pos_mode != kPosIota || a.block_table || a.seq_stride_rows != 0) return false;
     if (R != 1 && R != 2 && R != 4) return false;
     const long long cache_bytes = (long long)a.G * a.num_kv_heads * a.bits * 16;      // one buffer descriptor spans it
-    // out is written 4 halves at a time, the rotation read 16 bytes at a time
-    return a.ws && a.qrot && a.G >= 1 && (a.ws_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0 &&
-           (reinterpret_cast<uintptr_t>(a.out) & 7u) == 0 && (a.q_stride & 3) == 0 &&
+    // q and the rotation are read 16 bytes at a time, out is written 4 halves at a time
+    return a.G >= 1 && (reinterpret_cast<uintptr_t>(a.q) & 15u) == 0 && (a.q_stride & 7) == 0 &&
+           (reinterpret_cast<uintptr_t>(a.out) & 7u) == 0 &&
            (reinterpret_cast<uintptr_t>(a.rotation) & 15u) == 0 && cache_bytes < (1LL << 31);
 }
 
