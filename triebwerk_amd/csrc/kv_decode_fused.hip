@@ -56,9 +56,14 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     constexpr uint32_t kHeadBytes = BITS * 16;
     constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
-    __shared__ __attribute__((aligned(16))) half_t p_s[kFusedWaves][16][32];
+    // the scan's probabilities and partials; before the scan the same space holds R as 8 operand tiles
+    constexpr int kPBytes = kFusedWaves * 16 * 32 * 2, kPartBytes = kFusedWaves * R * kRowFloats * 4;
+    constexpr int kRotBytes = 8 * kOperandTileDwords * 4;
+    __shared__ __attribute__((aligned(16))) char scan_s[kPBytes + kPartBytes > kRotBytes ? kPBytes + kPartBytes : kRotBytes];
+    half_t (*p_s)[16][32] = reinterpret_cast<half_t (*)[16][32]>(scan_s);
+    float (*part_s)[R][kRowFloats] = reinterpret_cast<float (*)[R][kRowFloats]>(scan_s + kPBytes);
+    uint32_t* rot_s = reinterpret_cast<uint32_t*>(scan_s);
     __shared__ __attribute__((aligned(16))) float qrot_s[kFusedMaxQ][kHeadDim];
-    __shared__ __attribute__((aligned(16))) float part_s[kFusedWaves][R][kRowFloats];
     __shared__ __attribute__((aligned(16))) float o_s[kFusedMaxQ][kRowFloats];
     __shared__ __attribute__((aligned(16))) half_t prod_s[4][kHeadDim];   // k_weight, q_weight, cos row, sin row
 
@@ -107,15 +112,13 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         int kind0, head0;
         stage = reinterpret_cast<const uint4*>(unit_vector(tid >> 4, kind0, head0))[tid & 15];
     }
-    float rv[32];                                      // R[16 * rot_dblk + ln][4s + kg]
-    if (rotating) {
-        const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation + (rot_dblk * 16 + ln) * kHeadDim);
+    // R: wave w < 8 fetches rows 16w .. 16w + 15 (4 KB in a row, 4 fully used pieces per lane) and stages them
+    // as an operand tile; the rotating waves read their operand from there
+    uint4 rraw[4] = {};
+    if (wave < 8) {
 #pragma unroll
-        for (int q = 0; q < 16; q++) {
-            uint4 rp = rsrc[q];
-            rv[2 * q] = pick_half(rp, 0, kg);
-            rv[2 * q + 1] = pick_half(rp, 1, kg);
-        }
+        for (int j = 0; j < 4; j++)
+            rraw[j] = reinterpret_cast<const uint4*>(a.rotation + wave * 16 * kHeadDim)[j * kWave + lane];
     }
 
     // scaled centroid number lane % 16 (4 bit) or lane % 4 (2 bit), for the table build
@@ -280,14 +283,16 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
                 *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
             }
         }
-        for (int i = tid; i < kFusedWaves * 16 * 32 / 2; i += kFusedWaves * kWave) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
 
         // the staged vectors: rows of kStageStride bytes (16-byte aligned; a lane group's 2-byte reads below
         // fall into 32 different banks), in the space the merged outputs will use at the end
         char* x_s = reinterpret_cast<char*>(o_s);
         if ((tid >> 4) < nvec) *reinterpret_cast<uint4*>(x_s + (tid >> 4) * kStageStride + (tid & 15) * 16) = stage;
         if (PROD && prod_live) *reinterpret_cast<uint4*>(&prod_s[prod_row][8 * prod_piece]) = prod;
-        lds_barrier();             // the tile loads issued up front stay in flight
+        if (wave < 8) stage_operand_tile(rot_s + wave * kOperandTileDwords, rraw, lane);
+        lds_barrier();
+        float rv[32];                                      // R[16 * rot_dblk + ln][4s + kg]
+        if (rotating) read_operand_tile(rot_s + rot_dblk * kOperandTileDwords, lane, rv);
         if (PROD) {
             // optional producers on the staged K and query vectors, one vector per wave: per-head RMSNorm
             // (kernels.cu:880-923), then rotary embedding (927-961), each rounded to fp16 as the reference's
@@ -359,7 +364,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             }
         }
     }
-    __syncthreads();        // table, q_rot and the new cache row are in place
+    __syncthreads();        // table, q_rot and the new cache row are in place; R has been read
+    // the wave's slice of the probabilities starts at zero (no other wave touches it)
+    *reinterpret_cast<uint4*>(&p_s[wave][0][0] + 8 * lane) = uint4{0u, 0u, 0u, 0u};
     {
         int l2 = lane;
         asm volatile("" : "+v"(l2));

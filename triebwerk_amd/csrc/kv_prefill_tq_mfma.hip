@@ -376,11 +376,6 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
                 if (tq < T) {
                     const long long col = (long long)head * kHeadDim + 16 * db + 4 * kg;
                     half_t h[4] = {(half_t)y[nq][0], (half_t)y[nq][1], (half_t)y[nq][2], (half_t)y[nq][3]};
-                    if (a.gate) {
-                        const half_t* grow = a.gate + (long long)tq * a.gate_stride + col;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) h[i] = gated(h[i], grow[i]);
-                    }
                     *reinterpret_cast<uint2*>(a.out + (long long)tq * a.q_stride + col) = *reinterpret_cast<const uint2*>(h);
                 }
             }
@@ -397,7 +392,7 @@ bool prefill_tq_mfma_usable(const AttnArgs& a) {
     const long long cache_bytes = (long long)a.G * a.num_kv_heads * a.bits * 16;      // one buffer descriptor spans it
     // q and the rotation are read 16 bytes at a time, out is written 4 halves at a time
     return a.G >= 1 && (reinterpret_cast<uintptr_t>(a.q) & 15u) == 0 && (a.q_stride & 7) == 0 &&
-           (reinterpret_cast<uintptr_t>(a.out) & 7u) == 0 &&
+           (reinterpret_cast<uintptr_t>(a.out) & 7u) == 0 && !a.gate &&        // (no caller gates a prompt's output)
            (reinterpret_cast<uintptr_t>(a.rotation) & 15u) == 0 && cache_bytes < (1LL << 31);
 }
 

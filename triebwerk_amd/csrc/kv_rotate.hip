@@ -29,7 +29,7 @@
 // different rows: asked for directly that is 16 loads per lane of which a quarter is used, each touching 16
 // cache lines, and the address path of the CU becomes the limit of a big launch.  So a tile (16 rows, 4 KB)
 // comes in as 4 fully used 16-byte pieces per lane, is written to LDS with the halves regrouped
-// ([kk][row][s]), and each lane reads back its 32 halves as 4 x 16 bytes.
+// ([kk][row][s], kv_rotate_util.hpp), and each lane reads back its 32 halves as 4 x 16 bytes.
 
 #include <algorithm>
 #include <type_traits>
@@ -57,39 +57,6 @@ __device__ __forceinline__ void rope_registers(float (&xv)[32], const uint4 (&cp
     }
 }
 
-// An operand tile in LDS: row kk * 16 + i holds the halves 4s + kk, s = 0..31, of row i of the tile; 16 bytes
-// of padding per row keep the 16-byte reads of 16 lanes on different banks.
-constexpr int kOperandRow = 20;                           // dwords
-
-// raw[j] = 16-byte piece j * 64 + lane of the tile (piece q = lane % 16 of row 4j + lane / 16): its halves
-// e and 4 + e go to row e * 16 + (4j + lane / 16), dword q.
-__device__ __forceinline__ void stage_operand_tile(uint32_t* tile, const uint4 (&raw)[4], int lane) {
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        uint32_t* dst = tile + (4 * j + (lane >> 4)) * kOperandRow + (lane & 15);
-        dst[0 * 16 * kOperandRow] = (raw[j].x & 0xffffu) | (raw[j].z << 16);
-        dst[1 * 16 * kOperandRow] = (raw[j].x >> 16) | (raw[j].z & 0xffff0000u);
-        dst[2 * 16 * kOperandRow] = (raw[j].y & 0xffffu) | (raw[j].w << 16);
-        dst[3 * 16 * kOperandRow] = (raw[j].y >> 16) | (raw[j].w & 0xffff0000u);
-    }
-}
-
-// Lane kk * 16 + i reads row kk * 16 + i: out[s] = coordinate 4s + kk of row i.
-__device__ __forceinline__ void read_operand_tile(const uint32_t* tile, int lane, float (&out)[32]) {
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        const uint4 p = *reinterpret_cast<const uint4*>(tile + lane * kOperandRow + 4 * t);
-        const uint32_t w[4] = {p.x, p.y, p.z, p.w};
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            union { uint32_t u; half_t h[2]; } cv;
-            cv.u = w[e];
-            out[8 * t + 2 * e] = (float)cv.h[0];
-            out[8 * t + 2 * e + 1] = (float)cv.h[1];
-        }
-    }
-}
-
 }  // namespace
 
 // PROD: the producers of q and k may be switched on (their operands cost 64 registers and a third of the
@@ -97,7 +64,7 @@ __device__ __forceinline__ void read_operand_tile(const uint32_t* tile, int lane
 template <int BITS, bool PROD>
 __global__ void __launch_bounds__(kWave)
 rotate_kernel(RotArgs a) {
-    __shared__ __attribute__((aligned(16))) uint32_t x_s[kWave * kOperandRow];
+    __shared__ __attribute__((aligned(16))) uint32_t x_s[kOperandTileDwords];
     const int lane = threadIdx.x;
     const int i16 = lane & 15, kk = lane >> 4;
 
