@@ -258,9 +258,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     uint32_t kreg[2][KW];
     uint32_t vreg[2][VW];
     uint32_t nreg = 0;
-    // (Tiles are only requested after the rotations.  Asking for the first one up front, where it does not hold
-    // the row this workgroup is about to store, made short contexts 0.5 us slower per launch and long ones no
-    // faster; pulling further tiles towards the caches during the prologue cost 2 us per tile: what the
+    // (Tiles are only requested after the rotations.  Asking for the first one up front, without the row this
+    // workgroup is about to store, made launches 0.4 to 0.9 us slower at every context length, also with R
+    // arriving in 4 coalesced pieces per lane; pulling further tiles towards the caches during the prologue cost 2 us per tile: what the
     // prologue waits for then queues behind them.)
 
     // ---- 1. rotations of the unit's vectors
@@ -542,7 +542,8 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         }
     }
 
-    // ---- 3. the parts meet in LDS.  B operand of the rotate-back first (its loads run under the merge):
+    // ---- 3. the parts meet in LDS.  B operand of the rotate-back first (its loads run under the merge, and stay
+    // hidden there: R brought in coalesced and passed through LDS instead was 0.25 us slower per launch):
     // R[32kk + s][16*dblk + i16], s = 0..31
     const int nv = HKW * R;                                  // output vectors of this unit
     const int dblk = wave & 7;
