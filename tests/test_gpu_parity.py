@@ -607,6 +607,32 @@ def test_turbo_prefill_every_form(kv, oracle, rotation_fixture, bits, H, Hk, T, 
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("bits,H,Hk,T,pad", [(4, 16, 8, 333, 64), (2, 8, 4, 200, 8), (4, 8, 4, 150, 4), (2, 4, 4, 95, 1024)])
+def test_turbo_prefill_strided_rows_scratch_untouched(kv, oracle, rotation_fixture, bits, H, Hk, T, pad):
+    """Compressed prefill with rows of q and out wider than the heads (q_dim = H * 128 + pad; a pad of 4 halves
+    leaves the rows 8-byte aligned only, which the matrix-core prompt kernel does not take).  That kernel keeps
+    nothing in the scratch: it comes back as it went in.  The padding of out stays untouched."""
+    import torch
+    r = gen.rng(390 + bits + H + T)
+    msl = T + 5
+    kv_dim, q_dim = Hk * D, H * D + pad
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, 1, Hk, msl, [T], bits)
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.full((T, q_dim), 7.0, np.float16)
+    oracle.turbo_gqa_prefill_attention(want, q, ck[0], cv[0], kn[0], vn[0], rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+    assert (want[:, H * D:] == 7.0).all()
+    out = torch.full((T, q_dim), 7.0, dtype=torch.float16, device="cuda")
+    scratch = torch.full((T * H * T,), float("nan"), dtype=torch.float32, device="cuda")
+    kv.launch_turbo_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), dev(kn[0]), dev(vn[0]),
+                                          dev(rotation_fixture), scratch, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+    got = host(out)
+    if pad % 8 == 0:
+        assert bool(torch.isnan(scratch).all())
+    assert (got[:, H * D:] == 7.0).all()
+    err = rel_err(got[:, :H * D], want[:, :H * D])
+    assert err <= TOL, err
+
+
 @pytest.mark.parametrize("bits", [4, 2])
 def test_golden_case_on_gpu(kv, rotation_fixture, bits):
     """Committed vectors: append 37 tokens on the GPU, compare every byte, then attention."""

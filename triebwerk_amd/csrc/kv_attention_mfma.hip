@@ -639,6 +639,7 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     const int R = a.num_heads / a.num_kv_heads;
     if (a.bits != 4 && a.bits != 2) return false;
     if (R != 1 && R != 2 && R != 4) return false;
+    if (takes_prefill_tq(a)) return true;                  // that kernel needs no workspace and rotates its queries itself
     // needs the split workspace with room for q_rot behind each block's partials
     if (!a.ws || !a.qrot) return false;
     if ((reinterpret_cast<uintptr_t>(a.qrot) & 15u) != 0 || (a.ws_stride & 3) != 0) return false;
@@ -649,7 +650,7 @@ bool prepare_attention_mfma(AttnArgs& a, hipStream_t s, bool rotate_query) {
     a.slots_from_ws = 1;
     // ragged batches: cut the work by tiles, not by sequence (decided on the device from the positions)
     a.balance = (a.num_kv_heads == scan_waves(a) && a.G <= kMaxBalanceSeqs && a.max_slots >= 3 && a.G > 1) ? 1 : 0;
-    if (rotate_query && !takes_prefill_tq(a)) {           // (that kernel rotates its queries itself)
+    if (rotate_query) {
         RotArgs r;
         memset(&r, 0, sizeof(r));
         r.nseg = 1;
