@@ -345,3 +345,40 @@ def test_fp16_prefill_long_prompts_kernel_families_agree(kv, H, T):
             kv.set_attention_variant(0)
     err = rel_err_rows(outs[0], outs[1])
     assert err.max() <= TOL, f"max rel err {err.max():.3e} at row {err.argmax() // H}"
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_compressed_prefill_8192_tokens(kv, oracle, rotation_fixture, bits):
+    """A prompt of 8192 tokens over the compressed cache (16 heads over 8 KV heads): the cache comes from the
+    T-token append, the matrix-core prompt kernel (one launch: query rotation, attention, rotation back) is
+    compared row by row with the vector-ALU kernel, and rows at the ends, at tile and block borders and in
+    the middle with the oracle's decode attention at that position over the same cache (prefill row t is
+    decode at position t, kernels.cu:1874-1960 against 1641-1870)."""
+    import torch
+    H, Hk, T = 16, 8, 8192
+    kv_dim, q_dim = Hk * D, H * D
+    r, rot, base_k, base_v, ck, cv, kn, vn = build_target_cache(kv, rotation_fixture, bits, 1, Hk, T, 1)
+    q = gen.normal_f16(r, (T, q_dim))
+    d_q = dev(q)
+    scratch = torch.full((H * T * 1024,), float("nan"), dtype=torch.float32, device="cuda")
+    outs = []
+    for variant in (0, 1):
+        kv.set_attention_variant(variant)
+        try:
+            out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+            kv.launch_turbo_gqa_prefill_attention(out, d_q, ck[0], cv[0], kn[0], vn[0], rot, scratch, T, T, H, Hk, D,
+                                                  q_dim, kv_dim, bits)
+            outs.append(host(out))
+        finally:
+            kv.set_attention_variant(0)
+        if variant == 0:
+            assert bool(torch.isnan(scratch).all()), "the prompt kernel keeps nothing in the scratch"
+    err = rel_err_rows(outs[0], outs[1])
+    assert err.max() <= 2 * TOL, f"kernel families: max rel err {err.max():.3e} at row {err.argmax() // H}"
+    h_ck, h_cv, h_kn, h_vn = host(ck[0]), host(cv[0]), host(kn[0]), host(vn[0])
+    for t in (0, 1, 31, 32, 63, 64, 1000, 4095, 4096, 6143, 8190, 8191):
+        want = np.zeros(q_dim, np.float16)
+        oracle.turbo_gqa_attention(q[t], h_ck, h_cv, h_kn, h_vn, rotation_fixture, want, t, T, H, Hk, D, bits)
+        for name, got in (("matrix-core", outs[0][t]), ("vector-ALU", outs[1][t])):
+            e = rel_err_rows(got, want).max()
+            assert e <= TOL, f"{name} kernel, row {t}: rel err {e:.3e}"
