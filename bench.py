@@ -166,6 +166,35 @@ def prefill_bench(args):
 
         def launch():
             kvcache.launch_gqa_prefill_attention(out, q, ck, cv, ws, T, T, H, Hk, D, H * D, Hk * D)
+    if args.prompt_step:
+        # the whole layer over the prompt: producers of q and k, T-token append, attention (prefill_chunked,
+        # engine.cpp:2097-2146), as one call (1) or as the reference's sequence of launchers (2)
+        k = torch.randn((T, Hk * D), generator=g, device="cuda", dtype=torch.float16)
+        v = torch.randn((T, Hk * D), generator=g, device="cuda", dtype=torch.float16)
+        qw = (1 + 0.1 * torch.randn(D, generator=g, device="cuda")).to(torch.float16)
+        kw = (1 + 0.1 * torch.randn(D, generator=g, device="cuda")).to(torch.float16)
+        ang = torch.arange(T, device="cuda", dtype=torch.float64)[:, None] * 1e6 ** (-2.0 * torch.arange(D // 2, device="cuda", dtype=torch.float64) / D)[None, :]
+        ct, st = torch.cos(ang).to(torch.float16), torch.sin(ang).to(torch.float16)
+        pos = torch.arange(T, device="cuda", dtype=torch.int32)
+        q0, k0 = q.clone(), k.clone()
+        attention_only = launch
+
+        def launch():
+            q.copy_(q0); k.copy_(k0)                     # the producers work in place (two copies: 50 MB at 8192 tokens)
+            if args.prompt_step == 1:
+                kvcache.tw_layer_prompt_step(out, q, k, v, pos, T, T, H, Hk, D, H * D, Hk * D, ck, cv, ws, kv_bits=kv_bits,
+                                             k_norms=kn if kv_bits else None, v_norms=vn if kv_bits else None,
+                                             rotation=rot if kv_bits else None, q_weight=qw, k_weight=kw, eps=1e-6,
+                                             cos_table=ct, sin_table=st, rope_dim=D)
+                return
+            kvcache.launch_qk_norm_batch(q, k, qw, kw, H, Hk, D, T, 1e-6, H * D, Hk * D)
+            kvcache.launch_rope_batch(q, k, ct, st, pos, T, T, H, Hk, D, H * D, Hk * D, D)
+            if kv_bits:
+                kvcache.launch_turbo_kv_quantize(ck, kn, k, rot, pos, T, T, Hk, D, Hk * D, kv_bits)
+                kvcache.launch_turbo_kv_quantize(cv, vn, v, rot, pos, T, T, Hk, D, Hk * D, kv_bits)
+            else:
+                ck.copy_(k); cv.copy_(v)
+            attention_only()
     for _ in range(max(args.warmup, 1)):
         launch()
     torch.cuda.synchronize()
@@ -183,7 +212,9 @@ def prefill_bench(args):
         "steps": args.steps, "warmup": max(args.warmup, 1), "ms_per_step": ms, "higher_is_better": True,
         "dtype": "f32 accumulate over f16" if not kv_bits else "f32 accumulate over u8 codes + f16 norms", "data": "synthetic",
         "config": {"workload": f"causal prefill attention, one sequence, {T} tokens, {H} heads over {Hk} KV heads",
-                   "kv_bits": kv_bits if kv_bits else 16, "variant": args.variant},
+                   "kv_bits": kv_bits if kv_bits else 16, "variant": args.variant,
+                   "timed": ["the attention launch", "tw_layer_prompt_step: producers + T-token append + attention (+ 2 copies restoring q and k)",
+                             "launch_qk_norm_batch, launch_rope_batch, 2 appends, the attention launch (+ 2 copies restoring q and k)"][args.prompt_step]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s", "frac": tflops / 2500.0,
                      "flops_per_launch": flop, "traffic": None},
     }))
@@ -212,6 +243,10 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device-to-device copy of this many MiB five times (reference for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--prompt-step", type=int, default=0, choices=[0, 1, 2],
+                    help="with --prefill: 0 time the attention launch alone, 1 the whole layer over the prompt through "
+                         "tw_layer_prompt_step (QK norm, RoPE, T-token append, attention), 2 the same as the reference's "
+                         "sequence of launchers")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="instead of the decode step, time causal prefill attention over a T-token prompt of one "
                          "sequence (one layer's launch, the workload's head counts, --kv-bits cache) and exit")

@@ -301,6 +301,15 @@ typedef struct tw_layer_step_args {
 } tw_layer_step_args;
 void tw_layer_attention_step(const tw_layer_step_args* args, hipStream_t s);
 
+/* The same for a prompt: steps 3-5b of a layer in prefill_chunked (engine.cpp:2097-2150: launch_qk_norm_batch,
+ * launch_rope_batch, cudaMemcpyAsync x2 or launch_turbo_kv_quantize x2, launch_*_prefill_attention,
+ * launch_sigmoid_gate_batch) in one call and at most four launches.  The struct is read with G = T, the number of
+ * prompt tokens: row t of q / k / v / out / gate is token t, positions is device int32[T] and holds 0 .. T-1 (what
+ * the engine puts there before prefill_chunked; the rotary table row and the cache row of token t are
+ * positions[t]), the cache pointers are sequence 0's, scratch is sized as for the prefill launchers.  q (and with
+ * the compressed cache k) come back normalised and rotated.  ctx_min / ctx_max are not used. */
+void tw_layer_prompt_step(const tw_layer_step_args* args, hipStream_t s);
+
 /* Paged cache.  A page holds TW_PAGE_TOKENS consecutive positions of one
  * sequence in the same row layout the contiguous cache uses, so
  *   row(g, p) = block_table[g*bt_stride + p/16]*16 + p%16

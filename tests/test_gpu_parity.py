@@ -1004,6 +1004,60 @@ def test_layer_attention_step_with_gate(kv, oracle, rotation_fixture, kv_bits, n
     assert_bytes_equal(host(d_q)[:, H * D:], gate_rows, "gate rows")
 
 
+@pytest.mark.parametrize("kv_bits,T,producers,gated", [(4, 333, True, True), (2, 200, True, False), (0, 150, True, True),
+                                                       (4, 97, False, False), (0, 70, False, True), (2, 40, False, True)])
+def test_layer_prompt_step(kv, oracle, rotation_fixture, kv_bits, T, producers, gated):
+    """A layer over a prompt in one call (producers of q and k, T-token append into sequence 0, causal
+    attention, sigmoid gate; prefill_chunked, engine.cpp:2097-2150) == the oracle's steps one by one: the
+    cache bit for bit, the output within the attention tolerance.  Gated rows: q_dim = 2*H*D, the gate in the
+    second half of the q rows."""
+    import torch
+    r = gen.rng(820 + kv_bits + T)
+    H, Hk, msl = 8, 4, T + 11
+    kv_dim = Hk * D
+    q_dim = 2 * H * D if gated else H * D
+    pos = np.arange(T, dtype=np.int32)
+    q = gen.normal_f16(r, (T, q_dim)); k = gen.kv_rows_with_outliers(r, (T, kv_dim), kv_dim)[0]; v = gen.normal_f16(r, (T, kv_dim))
+    qw = (1.0 + 0.2 * r.standard_normal(D)).astype(np.float16); kw = (1.0 + 0.2 * r.standard_normal(D)).astype(np.float16)
+    ct, st = rope_tables(msl, D)
+    kvp = kv_dim * kv_bits // 8 if kv_bits else kv_dim
+    ck = np.zeros((msl, kvp), np.uint8 if kv_bits else np.float16); cv = np.zeros_like(ck)
+    kn = np.zeros((msl, Hk), np.float16); vn = np.zeros_like(kn)
+    d_q, d_k, d_ck, d_cv, d_kn, d_vn = dev(q), dev(k), dev(ck), dev(cv), dev(kn), dev(vn)
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * max(T, 1024), dtype=torch.float32, device="cuda")
+    extra = {}
+    if producers:
+        extra = dict(q_weight=dev(qw), k_weight=dev(kw), eps=1e-6, cos_table=dev(ct), sin_table=dev(st), rope_dim=D)
+    if gated:
+        extra.update(gate=d_q, gate_stride=q_dim, gate_offset=H * D)
+    kv.tw_layer_prompt_step(out, d_q, d_k, dev(v), dev(pos), msl, T, H, Hk, D, q_dim, kv_dim, d_ck, d_cv, scratch,
+                            kv_bits=kv_bits, k_norms=d_kn if kv_bits else None, v_norms=d_vn if kv_bits else None,
+                            rotation=dev(rotation_fixture) if kv_bits else None, **extra)
+    gate_rows = q[:, H * D:].copy()
+    if producers:
+        oracle.qk_norm_batch(q, k, qw, kw, H, Hk, D, T, 1e-6, q_dim, kv_dim, False)
+        oracle.rope_batch(q, k, ct, st, pos, msl, T, H, Hk, D, q_dim, kv_dim, D)
+    want = np.zeros((T, q_dim), np.float16)
+    if kv_bits:
+        oracle.turbo_kv_quantize(ck, kn, k, rotation_fixture, pos, msl, T, Hk, D, kv_dim, kv_bits)
+        oracle.turbo_kv_quantize(cv, vn, v, rotation_fixture, pos, msl, T, Hk, D, kv_dim, kv_bits)
+        oracle.turbo_gqa_prefill_attention(want, q, ck, cv, kn, vn, rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, kv_bits)
+        assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+    else:
+        ck[:T] = k; cv[:T] = v                                    # engine.cpp:2115-2118
+        oracle.gqa_prefill_attention(want, q, ck, cv, T, msl, H, Hk, D, q_dim, kv_dim)
+    assert_bytes_equal(host(d_ck), ck, "K cache"); assert_bytes_equal(host(d_cv), cv, "V cache")
+    assert_bytes_equal(host(d_q)[:, :H * D], q[:, :H * D], "q after its producers")
+    attn = np.ascontiguousarray(want[:, :H * D])
+    if gated:
+        oracle.sigmoid_gate_batch(attn, np.ascontiguousarray(gate_rows), H * D, T)
+        assert_bytes_equal(host(d_q)[:, H * D:], gate_rows, "gate rows")
+    got = host(out)
+    assert rel_err(got[:, :H * D], attn) <= TOL
+    assert not got[:, H * D:].any()
+
+
 # ------------------------------------------------------------------ engine: append -> attention -> positions, eager and graph
 @pytest.mark.parametrize("kv_bits", [0, 4, 2])
 @pytest.mark.parametrize("use_graph", [False, True])

@@ -77,6 +77,7 @@ SIGNATURES = {
     "tw_qk_norm_rope_append_attention_batch": (None, [P, P, P, P, P, P, C.c_float, I, P, P, I, P, P, P, P,
                                                       I, I, I, I, I, I, I, P]),
     "tw_layer_attention_step": (None, [C.POINTER(LayerStepArgs), P]),
+    "tw_layer_prompt_step": (None, [C.POINTER(LayerStepArgs), P]),
     "tw_paged_kv_cache_write_batch": (None, [P, P, P, P, P, P, I, I, I, P]),
     "tw_paged_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_paged_gqa_attention_batch": (None, [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),

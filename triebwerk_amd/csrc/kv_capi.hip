@@ -851,6 +851,67 @@ void tw_layer_attention_step(const tw_layer_step_args* p, hipStream_t s) {
     t_ctx_min = t_ctx_max = 0;
 }
 
+// Steps 3-5b of a layer over a prompt (prefill_chunked, engine.cpp:2097-2150): rows are the prompt's tokens,
+// the cache rows are sequence 0's.
+void tw_layer_prompt_step(const tw_layer_step_args* p, hipStream_t s) {
+    const char* fn = "tw_layer_prompt_step";
+    if (!p) { set_error(1, "%s: NULL arguments", fn); return; }
+    if (p->kv_bits != 0 && !check_bits(fn, p->kv_bits)) return;
+    if (!check_shape(fn, p->num_heads, p->num_kv_heads, p->head_dim)) return;
+    if (p->kv_dim != p->num_kv_heads * p->head_dim) {
+        set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, p->kv_dim);
+        return;
+    }
+    if (p->cos_table && !check_rope_dim(fn, p->rope_dim)) return;
+    if ((p->q_weight == nullptr) != (p->k_weight == nullptr) || (p->cos_table == nullptr) != (p->sin_table == nullptr)) {
+        set_error(1, "%s: q_weight/k_weight and cos_table/sin_table come in pairs", fn);
+        return;
+    }
+    const int T = p->G;
+    if (T <= 0) return;
+    const bool producers = p->q_weight || p->cos_table;
+    ProducerArgs pr;
+    fill_producer(pr, p->q, p->k, T, p->num_heads, p->num_kv_heads, p->q_dim, p->kv_dim);
+    pr.norm = p->q_weight ? 1 : 0; pr.q_weight = H(p->q_weight); pr.k_weight = H(p->k_weight);
+    pr.eps = p->eps; pr.biased = p->biased ? 1 : 0;
+    pr.cos_table = H(p->cos_table); pr.sin_table = H(p->sin_table); pr.rope_dim = p->rope_dim; pr.positions = p->positions;
+    if (p->kv_bits == 0) {
+        tw_half* ck = (tw_half*)p->cache_k;
+        tw_half* cv = (tw_half*)p->cache_v;
+        if (producers) {               // q in place; K (transformed) and V straight to rows positions[t] of sequence 0
+            pr.v = reinterpret_cast<half_t*>(const_cast<tw_half*>(p->v));
+            pr.write_cache = 1;
+            pr.cache_k = reinterpret_cast<half_t*>(ck);
+            pr.cache_v = reinterpret_cast<half_t*>(cv);
+            pr.kv_dim = p->kv_dim;
+            pr.seq_stride_rows = 0;
+            launch_producer(pr, s);
+        } else {
+            launch_kv_write(reinterpret_cast<half_t*>(ck), reinterpret_cast<half_t*>(cv), H(p->k), H(p->v), p->positions,
+                            nullptr, 0, 0, T, p->kv_dim, s);
+        }
+        check_launch(fn);
+        launch_gqa_prefill_attention(p->out, p->q, ck, cv, p->scratch, T, p->max_seq_len, p->num_heads, p->num_kv_heads,
+                                     p->head_dim, p->q_dim, p->kv_dim, s);
+    } else {
+        if (producers) {               // q and k in place
+            launch_producer(pr, s);
+            check_launch(fn);
+        }
+        quantize_common(fn, (uint8_t*)p->cache_k, p->k_norms, p->k, (uint8_t*)p->cache_v, p->v_norms, p->v, 2, p->rotation,
+                        p->positions, nullptr, 0, p->max_seq_len, 1, T, p->num_kv_heads, p->head_dim, p->kv_dim,
+                        p->kv_bits, s);
+        launch_turbo_gqa_prefill_attention(p->out, p->q, (const uint8_t*)p->cache_k, (const uint8_t*)p->cache_v, p->k_norms,
+                                           p->v_norms, p->rotation, p->scratch, T, p->max_seq_len, p->num_heads,
+                                           p->num_kv_heads, p->head_dim, p->q_dim, p->kv_dim, p->kv_bits, s);
+    }
+    if (p->gate) {
+        launch_sigmoid_gate(reinterpret_cast<half_t*>(p->out), p->q_dim, H(p->gate), p->gate_stride,
+                            p->num_heads * p->head_dim, T, s);
+        check_launch(fn);
+    }
+}
+
 void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const uint8_t* ck_q,
                                         const uint8_t* cv_q, const tw_half* k_norms,
                                         const tw_half* v_norms, const tw_half* rotation, float* as,

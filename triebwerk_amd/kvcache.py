@@ -324,9 +324,11 @@ def launch_sigmoid_gate_batch(data, gate, dim, G, stream=None):
 def tw_layer_attention_step(out, q, k, v, positions, max_seq_len, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim,
                             cache_k, cache_v, scratch, kv_bits=0, k_norms=None, v_norms=None, rotation=None,
                             q_weight=None, k_weight=None, eps=1e-6, biased=False, cos_table=None, sin_table=None,
-                            rope_dim=0, gate=None, gate_stride=0, gate_offset=0, ctx_min=0, ctx_max=0, stream=None):
+                            rope_dim=0, gate=None, gate_stride=0, gate_offset=0, ctx_min=0, ctx_max=0, stream=None,
+                            prompt=False):
     """Steps 3-6 of a layer (producers, append, attention, gate) through tw_layer_attention_step.
-    `gate` may be the q tensor itself with gate_offset = num_heads*head_dim (gated q projection)."""
+    `gate` may be the q tensor itself with gate_offset = num_heads*head_dim (gated q projection).
+    prompt=True: the rows are the G = T tokens of a prompt of sequence 0 (tw_layer_prompt_step)."""
     lib = _lib.load()
     a = _lib.LayerStepArgs()
     a.out, a.q, a.k, a.v = _ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(k, "f16", "k"), _ptr(v, "f16", "v")
@@ -344,5 +346,11 @@ def tw_layer_attention_step(out, q, k, v, positions, max_seq_len, G, num_heads, 
     a.gate = (gp + 2 * gate_offset) if gp is not None else None
     a.gate_stride = gate_stride
     a.ctx_min, a.ctx_max = int(ctx_min), int(ctx_max)       # host knowledge of positions + 1; 0, 0 = none
-    lib.tw_layer_attention_step(_lib.C.byref(a), _stream(stream))
+    (lib.tw_layer_prompt_step if prompt else lib.tw_layer_attention_step)(_lib.C.byref(a), _stream(stream))
     _done(lib)
+
+
+def tw_layer_prompt_step(out, q, k, v, positions, max_seq_len, T, *args, **kwargs):
+    """Steps 3-5b of a layer over a prompt of T tokens (prefill_chunked, engine.cpp:2097-2150); arguments as
+    tw_layer_attention_step with T in the place of G, positions = 0 .. T-1, the caches of sequence 0."""
+    tw_layer_attention_step(out, q, k, v, positions, max_seq_len, T, *args, prompt=True, **kwargs)
