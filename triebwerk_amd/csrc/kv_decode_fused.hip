@@ -260,8 +260,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     uint32_t nreg = 0;
     // (Tiles are only requested after the rotations.  Asking for the first one up front, without the row this
     // workgroup is about to store, made launches 0.4 to 0.9 us slower at every context length, also with R
-    // arriving in 4 coalesced pieces per lane; pulling further tiles towards the caches during the prologue cost 2 us per tile: what the
-    // prologue waits for then queues behind them.)
+    // arriving in 4 coalesced pieces per lane, and no faster when only the waves without a rotation to do ask;
+    // pulling further tiles towards the caches during the prologue cost 2 us per tile: what the prologue waits
+    // for then queues behind them.)
 
     // ---- 1. rotations of the unit's vectors
     {
