@@ -382,3 +382,30 @@ def test_compressed_prefill_8192_tokens(kv, oracle, rotation_fixture, bits):
         for name, got in (("matrix-core", outs[0][t]), ("vector-ALU", outs[1][t])):
             e = rel_err_rows(got, want).max()
             assert e <= TOL, f"{name} kernel, row {t}: rel err {e:.3e}"
+
+
+@pytest.mark.parametrize("bits,T", [(4, 4100), (2, 8200)])
+def test_compressed_prefill_per_wave_kernel_long_prompt(kv, rotation_fixture, bits, T):
+    """The prompt kernel that expands tiles per wave (form 4) keeps the three-launch shape: query rotation,
+    scan with partials, merge + rotate-back.  At these lengths its two small kernels walk several tiles per
+    wave / workgroup (more than 2048 tiles of 16 vectors); its output must agree row by row with the
+    one-launch kernel, which the test above pins to the oracle."""
+    import torch
+    H, Hk = 16, 8
+    kv_dim, q_dim = Hk * D, H * D
+    r, rot, base_k, base_v, ck, cv, kn, vn = build_target_cache(kv, rotation_fixture, bits, 1, Hk, T, 1)
+    d_q = dev(gen.normal_f16(r, (T, q_dim)))
+    scratch = torch.zeros(H * T * 1024, dtype=torch.float32, device="cuda")
+    outs = []
+    for form in (0, 4):
+        kv.set_prefill_form(form)
+        try:
+            out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+            kv.launch_turbo_gqa_prefill_attention(out, d_q, ck[0], cv[0], kn[0], vn[0], rot, scratch, T, T, H, Hk, D,
+                                                  q_dim, kv_dim, bits)
+            outs.append(host(out))
+        finally:
+            kv.set_prefill_form(0)
+    assert outs[1].any()
+    err = rel_err_rows(outs[0], outs[1])
+    assert err.max() <= 2 * TOL, f"max rel err {err.max():.3e} at row {err.argmax() // H}"
