@@ -409,3 +409,26 @@ def test_compressed_prefill_per_wave_kernel_long_prompt(kv, rotation_fixture, bi
     assert outs[1].any()
     err = rel_err_rows(outs[0], outs[1])
     assert err.max() <= 2 * TOL, f"max rel err {err.max():.3e} at row {err.argmax() // H}"
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_prompt_step_8192_tokens_same_cache_and_output(kv, rotation_fixture, bits):
+    """tw_layer_prompt_step over 8192 tokens (K and V rows appended in one launch, 131072 vectors) leaves the
+    bytes that two launch_turbo_kv_quantize calls leave (pinned to the oracle above and in the small cases),
+    and the output of the prefill launcher on that cache."""
+    import torch
+    H, Hk, T = 16, 8, 8192
+    kv_dim, q_dim = Hk * D, H * D
+    r, rot, base_k, base_v, ck, cv, kn, vn = build_target_cache(kv, rotation_fixture, bits, 1, Hk, T, 1)
+    q = dev(gen.normal_f16(r, (T, q_dim)))
+    scratch = torch.zeros(H * T * 1024, dtype=torch.float32, device="cuda")
+    want = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    kv.launch_turbo_gqa_prefill_attention(want, q, ck[0], cv[0], kn[0], vn[0], rot, scratch, T, T, H, Hk, D, q_dim, kv_dim, bits)
+    ck2, cv2, kn2, vn2 = torch.zeros_like(ck[0]), torch.zeros_like(cv[0]), torch.zeros_like(kn[0]), torch.zeros_like(vn[0])
+    out = torch.zeros_like(want)
+    pos = dev(np.arange(T, dtype=np.int32))
+    kv.tw_layer_prompt_step(out, q, dev(base_k[0]), dev(base_v[0]), pos, T, T, H, Hk, D, q_dim, kv_dim, ck2, cv2, scratch,
+                            kv_bits=bits, k_norms=kn2, v_norms=vn2, rotation=rot)
+    for name, a, b in (("K codes", ck2, ck[0]), ("V codes", cv2, cv[0]), ("K norms", kn2, kn[0]), ("V norms", vn2, vn[0]),
+                       ("output", out, want)):
+        assert torch.equal(a, b), name
