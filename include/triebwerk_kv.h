@@ -220,6 +220,14 @@ void tw_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q, tw
                               const int* positions, int max_seq_len, int G, int num_kv_heads,
                               int head_dim, int kv_dim, int bits, hipStream_t s);
 
+/* The same for the T tokens of a prompt of one sequence (prefill_chunked's two launch_turbo_kv_quantize calls,
+ * engine.cpp:2121-2131, in one launch): row t of k_buf / v_buf goes to cache row positions[t] of the sequence
+ * whose arrays are passed.  Same layout and arithmetic as launch_turbo_kv_quantize. */
+void tw_turbo_kv_append_tokens(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q, tw_half* v_norms,
+                               const tw_half* k_buf, const tw_half* v_buf, const tw_half* rotation,
+                               const int* positions, int max_seq_len, int num_tokens, int num_kv_heads,
+                               int head_dim, int kv_dim, int bits, hipStream_t s);
+
 /* One decode step of one layer in a single call: append K and V at positions[g],
  * then attention over 0..positions[g] (forward_layer_batch steps 4-5,
  * engine.cpp:1979-2006).  Same results as tw_turbo_kv_append_batch followed by

@@ -1004,6 +1004,27 @@ def test_layer_attention_step_with_gate(kv, oracle, rotation_fixture, kv_bits, n
     assert_bytes_equal(host(d_q)[:, H * D:], gate_rows, "gate rows")
 
 
+@pytest.mark.parametrize("bits,T", [(4, 77), (2, 300)])
+def test_turbo_kv_append_tokens(kv, oracle, rotation_fixture, bits, T):
+    """K and V rows of a prompt in one launch == the oracle's two T-token appends, bit for bit; positions in
+    any order, rows that are not written stay as they are."""
+    r = gen.rng(810 + bits)
+    Hk, msl = 8, T + 20
+    kv_dim = Hk * D
+    kvp = kv_dim * bits // 8
+    pos = r.permutation(msl)[:T].astype(np.int32)
+    k = gen.kv_rows_with_outliers(r, (T, kv_dim), kv_dim)[0]; v = gen.normal_f16(r, (T, kv_dim))
+    ck = r.integers(0, 256, (msl, kvp), dtype=np.uint8); cv = r.integers(0, 256, (msl, kvp), dtype=np.uint8)
+    kn = gen.normal_f16(r, (msl, Hk)); vn = gen.normal_f16(r, (msl, Hk))
+    d_ck, d_cv, d_kn, d_vn = dev(ck), dev(cv), dev(kn), dev(vn)
+    kv.tw_turbo_kv_append_tokens(d_ck, d_kn, d_cv, d_vn, dev(k), dev(v), dev(rotation_fixture), dev(pos), msl, T, Hk, D,
+                                 kv_dim, bits)
+    oracle.turbo_kv_quantize(ck, kn, k, rotation_fixture, pos, msl, T, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize(cv, vn, v, rotation_fixture, pos, msl, T, Hk, D, kv_dim, bits)
+    assert_bytes_equal(host(d_ck), ck, "K codes"); assert_bytes_equal(host(d_cv), cv, "V codes")
+    assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+
+
 @pytest.mark.parametrize("kv_bits,T,producers,gated", [(4, 333, True, True), (2, 200, True, False), (0, 150, True, True),
                                                        (4, 97, False, False), (0, 70, False, True), (2, 40, False, True)])
 def test_layer_prompt_step(kv, oracle, rotation_fixture, kv_bits, T, producers, gated):

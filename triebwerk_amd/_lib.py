@@ -70,6 +70,7 @@ SIGNATURES = {
     "tw_kv_broadcast_rows": (I, [P, P, P, I, I, I, I, P]),
     "tw_attention_workspace_floats": (SZ, [I, I, I]),
     "tw_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
+    "tw_turbo_kv_append_tokens": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_append_attention_batch": (None, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P]),
     "tw_turbo_append_attention_batch": (None, [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
     "tw_qk_norm_rope_turbo_append_attention_batch": (None, [P, P, P, P, P, P, C.c_float, I, P, P, I, P, P, P, P, P, P, P,

@@ -409,6 +409,15 @@ void tw_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q, tw
                     kv_dim, bits, s);
 }
 
+void tw_turbo_kv_append_tokens(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q, tw_half* v_norms,
+                               const tw_half* k_buf, const tw_half* v_buf, const tw_half* rotation,
+                               const int* positions, int max_seq_len, int num_tokens, int num_kv_heads,
+                               int head_dim, int kv_dim, int bits, hipStream_t s) {
+    quantize_common("tw_turbo_kv_append_tokens", ck_q, k_norms, k_buf, cv_q, v_norms, v_buf, 2,
+                    rotation, positions, nullptr, 0, max_seq_len, 1, num_tokens, num_kv_heads, head_dim,
+                    kv_dim, bits, s);
+}
+
 void tw_paged_turbo_kv_append_batch(uint8_t* ck_q, tw_half* k_norms, uint8_t* cv_q,
                                     tw_half* v_norms, const tw_half* k_buf, const tw_half* v_buf,
                                     const tw_half* rotation, const int* positions,

@@ -148,6 +148,18 @@ def tw_turbo_kv_append_batch(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotatio
     _done(lib)
 
 
+def tw_turbo_kv_append_tokens(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotation, positions,
+                              max_seq_len, num_tokens, num_kv_heads, head_dim, kv_dim, bits, stream=None):
+    """K and V rows of a prompt's tokens into one sequence's cache, one launch (engine.cpp:2121-2131)."""
+    lib = _lib.load()
+    lib.tw_turbo_kv_append_tokens(_ptr(ck_q, "u8", "ck_q"), _ptr(k_norms, "f16", "k_norms"),
+                                  _ptr(cv_q, "u8", "cv_q"), _ptr(v_norms, "f16", "v_norms"),
+                                  _ptr(k_buf, "f16", "k_buf"), _ptr(v_buf, "f16", "v_buf"),
+                                  _ptr(rotation, "f16", "rotation"), _ptr(positions, "i32", "positions"),
+                                  max_seq_len, num_tokens, num_kv_heads, head_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
 def tw_turbo_append_attention_batch(out, q, k_buf, v_buf, ck_q, cv_q, k_norms, v_norms, rotation, scratch,
                                     pos, msl, G, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits,
                                     stream=None):
