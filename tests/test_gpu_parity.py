@@ -583,7 +583,8 @@ def test_turbo_prefill_attention_long(kv, oracle, rotation_fixture, bits, H, Hk,
 
 
 @pytest.mark.parametrize("form", [1, 2, 3, 4])
-@pytest.mark.parametrize("bits,H,Hk,T", [(4, 16, 8, 300), (2, 8, 8, 129), (4, 16, 4, 97), (2, 16, 8, 31)])
+@pytest.mark.parametrize("bits,H,Hk,T", [(4, 16, 8, 300), (2, 8, 8, 129), (4, 16, 4, 97), (2, 16, 8, 31), (4, 8, 4, 1),
+                                         (2, 4, 4, 7), (4, 4, 1, 16), (2, 8, 4, 33)])
 def test_turbo_prefill_every_form(kv, oracle, rotation_fixture, bits, H, Hk, T, form):
     """Compressed prefill: the three forms of the kernel that expands a tile once per workgroup and (form 4)
     the kernel that expands per wave, each against the oracle."""
