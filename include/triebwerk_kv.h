@@ -413,6 +413,13 @@ int tw_engine_set_producers(tw_engine* e, int mode, const tw_half* q_norm, const
 int tw_engine_layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k,
                          const tw_half* v, tw_half* out, hipStream_t s);
 
+/* The path of `layer` over a prompt of T tokens for sequence `seq` of the batch (prefill_chunked, engine.cpp:2097-2150,
+ * which does it for sequence 0): the producers the engine was given, the T-token append into that sequence's cache
+ * rows, causal attention.  q/out: (T, num_heads*head_dim); k/v: (T, kv_dim); token_positions: device int32[T] holding
+ * 0 .. T-1.  The positions of the batch are the caller's to set afterwards (tw_engine_set_positions). */
+int tw_engine_prompt_layer(tw_engine* e, int layer, int seq, const tw_half* q, const tw_half* k, const tw_half* v,
+                           tw_half* out, const int* token_positions, int T, hipStream_t s);
+
 /* All layers, then positions += 1.  q/out: (L, G, q_dim); k/v: (L, G, kv_dim).
  * With use_graph != 0 the step is captured once into a hipGraph and replayed
  * (engine.cpp:2369-2412, 2480); the capture is dropped when the arena, G or

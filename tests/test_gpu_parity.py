@@ -1344,6 +1344,66 @@ def test_engine_prefix_broadcast(oracle, kv_bits, Hk, src, dst):
                     assert np.array_equal(now[g], was[g]), (l, g)
 
 
+@pytest.mark.parametrize("kv_bits,mode", [(4, 1), (2, 2), (0, 1), (4, 0)])
+def test_engine_prompt_layer_then_broadcast(oracle, rotation_fixture, kv_bits, mode):
+    """The engine's prompt call for one sequence of the batch (producers fused, as the reference's two launches,
+    or none), then the prefix broadcast: that sequence's cache rows and the output equal the oracle's steps, the
+    destinations hold the same rows, everything else keeps its bytes."""
+    import torch
+    from triebwerk_amd import Engine
+    L, H, Hk, G, msl, T, seq = 2, 8, 4, 4, 96, 50, 2
+    kv_dim, q_dim = Hk * D, H * D
+    r = gen.rng(880 + kv_bits + mode)
+    eng = Engine(max_seq_len=msl, kv_bits=kv_bits)
+    eng.set_shape(L, H, Hk, D)
+    eng.alloc_batch(G, msl)
+    qw = (1.0 + 0.2 * r.standard_normal((L, D))).astype(np.float16); kw = (1.0 + 0.2 * r.standard_normal((L, D))).astype(np.float16)
+    ct, st = rope_tables(msl, D)
+    if mode:
+        eng.set_producers(mode, dev(qw), dev(kw), 1e-6, False, dev(ct), dev(st), D)
+    pos = np.arange(T, dtype=np.int32)
+    layer = 1
+    marks = []
+    for arr in eng.cache(layer):
+        if arr is not None:
+            raw = arr.view(torch.uint8)
+            raw.fill_(0x5A)
+            marks.append(raw)
+    q = gen.normal_f16(r, (T, q_dim)); k = gen.kv_rows_with_outliers(r, (T, kv_dim), kv_dim)[0]; v = gen.normal_f16(r, (T, kv_dim))
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    eng.prompt_layer(layer, seq, dev(q), dev(k), dev(v), out, dev(pos))
+    if mode:
+        oracle.qk_norm_batch(q, k, qw[layer], kw[layer], H, Hk, D, T, 1e-6, q_dim, kv_dim, False)
+        oracle.rope_batch(q, k, ct, st, pos, msl, T, H, Hk, D, q_dim, kv_dim, D)
+    want = np.zeros((T, q_dim), np.float16)
+    if kv_bits:
+        kvp = kv_dim * kv_bits // 8
+        ck = np.full((msl, kvp), 0x5A, np.uint8); cv = ck.copy()
+        kn = np.full((msl, Hk), 0x5A5A, np.uint16).view(np.float16); vn = kn.copy()
+        oracle.turbo_kv_quantize(ck, kn, k, rotation_fixture, pos, msl, T, Hk, D, kv_dim, kv_bits)
+        oracle.turbo_kv_quantize(cv, vn, v, rotation_fixture, pos, msl, T, Hk, D, kv_dim, kv_bits)
+        oracle.turbo_gqa_prefill_attention(want, q, ck, cv, kn, vn, rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, kv_bits)
+        expect = [ck, cv, kn.view(np.uint8).reshape(msl, -1), vn.view(np.uint8).reshape(msl, -1)]
+    else:
+        ck = np.full((msl, kv_dim), 0x5A5A, np.uint16).view(np.float16); cv = ck.copy()
+        ck[:T] = k; cv[:T] = v
+        oracle.gqa_prefill_attention(want, q, ck, cv, T, msl, H, Hk, D, q_dim, kv_dim)
+        expect = [ck.view(np.uint8).reshape(msl, -1), cv.view(np.uint8).reshape(msl, -1)]
+    assert rel_err(host(out), want) <= TOL
+    for raw, exp in zip(marks, expect):
+        now = host(raw).reshape(G, msl, -1)
+        assert np.array_equal(now[seq], exp)
+        for g in range(G):
+            if g != seq:
+                assert (now[g] == 0x5A).all()
+    eng.broadcast_prefix(seq, 0, G, T)
+    for raw, exp in zip(marks, expect):
+        now = host(raw).reshape(G, msl, -1)
+        for g in range(G):
+            assert np.array_equal(now[g, :T], exp[:T]), g
+            assert g == seq or (now[g, T:] == 0x5A).all()
+
+
 def test_plain_read_bandwidth_probe(kv):
     """The calibration kernel the benchmark quotes: plausible on a large buffer, an error on a bad one."""
     import ctypes as C

@@ -108,6 +108,7 @@ SIGNATURES = {
     "tw_engine_output": (I, [P, I, C.POINTER(C.POINTER(I)), C.POINTER(I)]),
     "tw_engine_host_position": (I, [P, I]),
     "tw_engine_layer_step": (I, [P, I, P, P, P, P, P]),
+    "tw_engine_prompt_layer": (I, [P, I, I, P, P, P, P, P, I, P]),
     "tw_engine_decode_step": (I, [P, P, P, P, P, I, P]),
     "tw_engine_broadcast_prefix": (I, [P, I, I, I, I, P]),
 }

@@ -430,6 +430,54 @@ int tw_engine_layer_step(tw_engine* e, int layer, const tw_half* q, const tw_hal
     return tw_kv_last_error();
 }
 
+int tw_engine_prompt_layer(tw_engine* e, int layer, int seq, const tw_half* q, const tw_half* k, const tw_half* v,
+                           tw_half* out, const int* token_positions, int T, hipStream_t s) {
+    if (!e->arena || layer < 0 || layer >= e->shape.num_layers || seq < 0 || seq >= e->G || T < 0 || T > e->batch_msl ||
+        !token_positions)
+        return -1;
+    if (T == 0) return 0;
+    s = pick(e, s);
+    tw_kv_clear_error();
+    const tw_model_shape& m = e->shape;
+    tw_half* qm = const_cast<tw_half*>(q);      // with producers q and k are the caller's scratch rows
+    tw_half* km = const_cast<tw_half*>(k);
+    const tw_half* qw = e->q_norm ? e->q_norm + (size_t)layer * m.head_dim : nullptr;
+    const tw_half* kw = e->k_norm ? e->k_norm + (size_t)layer * m.head_dim : nullptr;
+    if (e->producers == 2) {                    // the reference's sequence of launches (engine.cpp:2103-2108)
+        if (qw) launch_qk_norm_batch(qm, km, qw, kw, m.num_heads, m.num_kv_heads, m.head_dim, T, e->norm_eps,
+                                     e->q_dim(), e->kv_dim(), s, e->norm_biased != 0);
+        if (e->rope_cos) launch_rope_batch(qm, km, e->rope_cos, e->rope_sin, token_positions, e->batch_msl, T,
+                                           m.num_heads, m.num_kv_heads, m.head_dim, e->q_dim(), e->kv_dim(),
+                                           e->rope_dim, s);
+    }
+    tw_layer_step_args p;
+    memset(&p, 0, sizeof(p));
+    p.out = out; p.q = qm; p.k = km; p.v = v;
+    p.G = T; p.num_heads = m.num_heads; p.num_kv_heads = m.num_kv_heads; p.head_dim = m.head_dim;
+    p.q_dim = e->q_dim(); p.kv_dim = e->kv_dim();
+    p.positions = token_positions; p.max_seq_len = e->batch_msl;
+    if (e->producers == 1) {
+        p.q_weight = qw; p.k_weight = kw; p.eps = e->norm_eps; p.biased = e->norm_biased;
+        p.cos_table = e->rope_cos; p.sin_table = e->rope_sin; p.rope_dim = e->rope_dim;
+    }
+    p.kv_bits = e->kv_bits;
+    const size_t msl = (size_t)e->batch_msl;
+    const size_t row = e->kv_bits == 0 ? (size_t)e->kv_dim() * 2 : e->kv_dim_packed();
+    const size_t nrow = (size_t)m.num_kv_heads * 2;
+    p.cache_k = (char*)e->cache[layer][0] + seq * msl * row;
+    p.cache_v = (char*)e->cache[layer][1] + seq * msl * row;
+    if (e->kv_bits != 0) {
+        p.k_norms = (tw_half*)((char*)e->cache[layer][2] + seq * msl * nrow);
+        p.v_norms = (tw_half*)((char*)e->cache[layer][3] + seq * msl * nrow);
+    }
+    p.rotation = e->d_rotation;
+    // the batch's attention scratch holds G * num_heads * max_seq_len floats (engine.cpp:1371); the prefill
+    // launchers count on T floats per (token, head) and do without a workspace when there is none
+    p.scratch = ((size_t)T * T <= (size_t)e->G * msl) ? e->attn_scores : nullptr;
+    tw_layer_prompt_step(&p, s);
+    return tw_kv_last_error();
+}
+
 int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v,
                           tw_half* out, int use_graph, hipStream_t s) {
     if (!e->arena) return -1;

@@ -124,6 +124,17 @@ class Engine:
             _lib.check(self._lib)
             raise RuntimeError(f"layer_step failed ({rc})")
 
+    def prompt_layer(self, layer, seq, q, k, v, out, token_positions, stream=None) -> None:
+        """The path of one layer over a prompt (rows of q/k/v/out = its tokens, token_positions = 0 .. T-1) for
+        sequence `seq`: producers, T-token append, causal attention (prefill_chunked, engine.cpp:2097-2150)."""
+        rc = self._lib.tw_engine_prompt_layer(self._h, layer, seq, _ptr(q, "f16", "q"), _ptr(k, "f16", "k"),
+                                              _ptr(v, "f16", "v"), _ptr(out, "f16", "out"),
+                                              _ptr(token_positions, "i32", "token_positions"), int(q.shape[0]),
+                                              _stream(stream))
+        if rc != 0:
+            _lib.check(self._lib)
+            raise RuntimeError(f"prompt_layer failed ({rc})")
+
     def decode_step(self, q, k, v, out, use_graph: bool = False, stream=None) -> None:
         """Append + attention for every layer, then positions += 1.
         q/out: (L, G, H*D); k/v: (L, G, Hk*D)."""
