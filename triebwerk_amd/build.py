@@ -81,10 +81,20 @@ def build_library(verbose: bool = False) -> Path:
 
     def compile_one(src: str) -> str:
         obj = objdir / (Path(src).stem + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src, []), "-c", str(CSRC / src), "-o", str(obj)]
+        base = [hipcc, *HIPCC_FLAGS]
+        tail = ["-c", str(CSRC / src), "-o", str(obj)]
+        extra = PER_FILE_FLAGS.get(src, [])
+        cmd = [*base, *extra, *tail]
         if verbose:
             print(" ".join(cmd), flush=True)
-        _run(cmd)
+        try:
+            _run(cmd)
+        except RuntimeError:
+            if not extra:
+                raise
+            # a compiler that does not know the scheduler option: the same code with its default scheduler
+            print(f"{src}: retrying without {' '.join(extra)}", file=sys.stderr, flush=True)
+            _run([*base, *tail])
         return str(obj)
 
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
