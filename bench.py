@@ -220,6 +220,121 @@ def prefill_bench(args):
     }))
 
 
+def paged_bench(args):
+    """The decode step over a paged cache: 16-token pages in one pool per layer, a per-sequence block table in
+    random page order (shared by the layers), every layer = paged append of K and V + paged decode attention, then
+    positions += 1; the step is captured in a graph and replayed.  Same metric and byte count as the contiguous
+    run of the same workload; the roofline object is the context-scanning kernel's."""
+    import torch
+    from triebwerk_amd import _lib, kvcache
+    w = dict(WORKLOADS[args.workload])
+    kv_bits = w["kv_bits"] if args.kv_bits is None else args.kv_bits
+    if kv_bits == 0:
+        sys.exit("bench.py: --paged measures the compressed caches (--kv-bits 4 or 2)")
+    for key, val in (("ctx", args.ctx), ("G", args.batch), ("L", args.layers)):
+        if val is not None:
+            w[key] = val
+    L, H, Hk, G, D = w["L"], w["H"], w["Hk"], w["G"], 128
+    K, W = args.steps, args.warmup
+    kv_dim, q_dim, kvp = Hk * D, H * D, Hk * D * kv_bits // 8
+    total_steps = W + K + K + 2
+    msl = (w["ctx"] + total_steps + 255) // 256 * 256
+    pages_per_seq, n_pages = msl // 16, G * msl // 16
+    lib = _lib.load()
+    torch.cuda.set_device(0)
+    kvcache.set_attention_variant(args.variant)
+    kvcache.set_num_splits(args.nsplit)
+
+    rng = np.random.Generator(np.random.Philox(3))            # the same lengths as the contiguous run
+    if w["ragged"]:
+        ctx0 = rng.integers(w["ragged"][0], w["ragged"][1] + 1, size=G).astype(np.int64)
+    else:
+        ctx0 = np.full(G, w["ctx"], np.int64)
+    start_pos = np.maximum(ctx0 - 1 - W, 0).astype(np.int32)
+    bt = np.random.Generator(np.random.Philox(4)).permutation(n_pages).astype(np.int32).reshape(G, pages_per_seq)
+    g = torch.Generator(device="cuda"); g.manual_seed(1)
+    pools = []
+    for _ in range(L):
+        pools.append((torch.randint(0, 256, (n_pages, 16, kvp), generator=g, device="cuda", dtype=torch.uint8),
+                      torch.randint(0, 256, (n_pages, 16, kvp), generator=g, device="cuda", dtype=torch.uint8),
+                      (11.3 + 0.7 * torch.randn((n_pages, 16, Hk), generator=g, device="cuda")).to(torch.float16),
+                      (11.3 + 0.7 * torch.randn((n_pages, 16, Hk), generator=g, device="cuda")).to(torch.float16)))
+    q = torch.randn((L, G, q_dim), generator=g, device="cuda", dtype=torch.float16)
+    k = torch.randn((L, G, kv_dim), generator=g, device="cuda", dtype=torch.float16)
+    v = torch.randn((L, G, kv_dim), generator=g, device="cuda", dtype=torch.float16)
+    out = torch.zeros((L, G, q_dim), device="cuda", dtype=torch.float16)
+    rot = kvcache.make_rotation().cuda()
+    ws = torch.zeros(kvcache.attention_workspace_floats(G, H, msl), dtype=torch.float32, device="cuda")
+    pos = torch.from_numpy(start_pos).cuda()
+    d_bt = torch.from_numpy(bt).cuda()
+    stream = torch.cuda.Stream()
+
+    def layers():
+        for l in range(L):
+            ck, cv, kn, vn = pools[l]
+            kvcache.tw_paged_turbo_kv_append_batch(ck, kn, cv, vn, k[l], v[l], rot, pos, d_bt, pages_per_seq, G, Hk, D,
+                                                   kv_dim, kv_bits)
+            kvcache.tw_paged_turbo_gqa_attention_batch(out[l], q[l], ck, cv, kn, vn, rot, ws, pos, d_bt, pages_per_seq,
+                                                       msl, G, H, Hk, D, q_dim, kv_dim, kv_bits)
+        pos.add_(1)
+
+    use_graph = not args.no_graph
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        layers()                                             # warm-up step 1, eager
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                layers()
+        step = graph.replay if use_graph else layers
+        for _ in range(W - 1):
+            step()
+    torch.cuda.synchronize()
+    pos_now = start_pos.astype(np.int64) + max(W, 1)
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        for _ in range(K):
+            step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    n_tokens_timed = int(sum(int((pos_now + i + 1).sum()) for i in range(K)))
+    pos_now = pos_now + K
+    assert np.array_equal(pos.cpu().numpy().astype(np.int64), pos_now), "positions drifted"
+    assert torch.isfinite(out.float()).all(), "non-finite attention output"
+    step_bytes = algorithmic_bytes(n_tokens_timed, G * K, L, H, Hk, kv_bits, with_append=True) / K
+    step_gbs = step_bytes / (elapsed / K) * 1e-9
+
+    Kp = max(1, min(K, 4096 // L))
+    lib.tw_kv_profile_attention(1)
+    with torch.cuda.stream(stream):
+        for _ in range(Kp):
+            layers()
+    torch.cuda.synchronize()
+    total_ms, launches = C.c_double(0), C.c_int(0)
+    rc = lib.tw_kv_profile_read(C.byref(total_ms), C.byref(launches))
+    lib.tw_kv_profile_attention(0)
+    assert rc == 0 and launches.value == Kp * L, (rc, launches.value)
+    n_tokens_prof = int(sum(int((pos_now + i + 1).sum()) for i in range(Kp)))
+    kern_ms = total_ms.value / launches.value
+    launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=False) / (Kp * L)
+    achieved = launch_bytes / (kern_ms * 1e-3) * 1e-9
+    print(json.dumps({
+        "metric": "decode-attn tokens/s", "value": G * K / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 accumulate over u8 codes + f16 norms", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['desc']}, paged cache: 16-token pages, block table in random page order",
+                   "kv_bits": kv_bits, "layers": L, "num_heads": H, "num_kv_heads": Hk, "head_dim": D, "batch": G,
+                   "pages": n_pages, "context_first_timed_step": [int(ctx0.min()), int(ctx0.max())],
+                   "tokens_attended_per_step": n_tokens_timed / K, "hipgraph": use_graph,
+                   "step": "paged append K,V + paged decode attention for every layer, positions += 1"},
+        "step_algorithmic_GB": step_bytes * 1e-9, "step_achieved_GBps": step_gbs,
+        "step_frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "paged decode attention (context scan), one launch per layer",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "launch_ms": kern_ms, "launch_algorithmic_MB": launch_bytes * 1e-6, "traffic": None},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -240,6 +355,11 @@ def main():
     ap.add_argument("--ctx", type=int, default=None, help="override the workload's context length")
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--layers", type=int, default=None, help="override the workload's layer count")
+    ap.add_argument("--paged", action="store_true",
+                    help="the same step over a paged cache (16-token pages, block table in random page order) through "
+                         "the tw_paged_* entry points; compressed caches only")
+    ap.add_argument("--max-seq-len", type=int, default=None,
+                    help="the engine's max_seq_len (rows per sequence in every cache array); default: context + steps, rounded up to 256")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run a plain device-to-device copy of this many MiB five times (reference for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -268,6 +388,9 @@ def main():
         print("bench.py: this build runs on one GPU; sharding is by sequence or KV head with no exchange "
               "inside the path, and is not implemented. Use --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    if args.paged:
+        paged_bench(args)
+        return
 
     import torch
     from triebwerk_amd import Engine, _lib, kvcache
@@ -286,6 +409,11 @@ def main():
     kv_dim, q_dim = Hk * D, H * D
     total_steps = W + K + K + 2          # warm-up, graph-timed, kernel-timed (eager), slack
     msl = (w["ctx"] + total_steps + 255) // 256 * 256   # the engine's max_seq_len: context + room for the steps, rounded up
+    if args.max_seq_len is not None:
+        if args.max_seq_len < w["ctx"] + total_steps:
+            sys.exit(f"bench.py: --max-seq-len {args.max_seq_len} leaves no room for context {w['ctx']} + {total_steps} steps")
+        msl = args.max_seq_len
+        w["desc"] += f" [max_seq_len={msl}]"
 
     lib = _lib.load()
     torch.cuda.set_device(0)

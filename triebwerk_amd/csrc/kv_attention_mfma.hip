@@ -201,9 +201,15 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     // Buffer descriptors: base = first cache row of the tile (contiguous cache) or of the
     // 16-token page (paged cache), extent = the rows that exist, so lanes past the end
     // of the sequence read zeros instead of foreign memory.  All scalar.
-    auto page_row = [&](int ts) -> long long {   // paged: past the end re-read the last page (masked)
-        return (long long)uniform(bt[min(ts, t1 - 1) >> 4]) * kPageTokens;
+    // Paged: the two block-table entries of a tile are fetched one tile ahead by a vector load
+    // (even lanes: first page, odd lanes: second) that is issued before the loads of the tile in
+    // between, so it has returned, in order, by the time that tile's codes are waited for, and the
+    // wait for it holds up no load in flight.  Past the end the last page is re-read (masked).
+    auto fetch_pages = [&](int ts) -> int { return bt[min(ts + 16 * (lane & 1), t1 - 1) >> 4]; };
+    auto page_row = [&](int pages, int sub) -> long long {
+        return (long long)__builtin_amdgcn_readlane(pages, sub) * kPageTokens;
     };
+    int pages_next = 0;                          // entries of the tile whose loads are issued next in the loop
     auto load_k = [&](__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t (&dst)[KW]) {
         if constexpr (BITS == 4) {
             uint32x4_t q = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
@@ -213,22 +219,22 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
             dst[0] = q[0]; dst[1] = q[1];
         }
     };
-    auto issue_k = [&](uint32_t (&kreg)[2][KW], int tile) {
+    auto issue_k = [&](uint32_t (&kreg)[2][KW], int tile, int pages) {
         if (PAGED) {
 #pragma unroll
             for (int sub = 0; sub < 2; sub++)
-                load_k(make_rsrc(kseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp), koff, kreg[sub]);
+                load_k(make_rsrc(kseq + page_row(pages, sub) * kvp, kPageTokens * (int)kvp), koff, kreg[sub]);
         } else {
             __amdgpu_buffer_rsrc_t r = make_rsrc(kseq + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
             load_k(r, koff, kreg[0]);
             load_k(r, koff + sub_bytes, kreg[1]);
         }
     };
-    auto issue_v = [&](uint32_t (&vreg)[2][VW], int tile) {
+    auto issue_v = [&](uint32_t (&vreg)[2][VW], int tile, int pages) {
         if (PAGED) {
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
-                __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + page_row(tile + 16 * sub) * kvp, kPageTokens * (int)kvp);
+                __amdgpu_buffer_rsrc_t r = make_rsrc(vseq + page_row(pages, sub) * kvp, kPageTokens * (int)kvp);
 #pragma unroll
                 for (int i = 0; i < VW; i++) vreg[sub][i] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff[i], 0, 0);
             }
@@ -252,12 +258,11 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
         uint32_t w = dw == 0 ? q[0] : dw == 1 ? q[1] : dw == 2 ? q[2] : q[3];
         return (h & 1) ? (w >> 16) : (w & 0xffffu);
     };
-    auto issue_n = [&](int tile) -> uint32_t {
+    auto issue_n = [&](int tile, int pages) -> uint32_t {
         const bool wide = (nrow & 15u) == 0;
         const uint32_t hgrp = (uint32_t)(h >> 3) * 16u;          // 16-byte group of this head inside a row
         if (PAGED) {
-            long long r0 = page_row(tile), r1 = page_row(tile + 16);
-            const long long rr = my_sub ? r1 : r0;
+            const long long rr = my_sub ? page_row(pages, 1) : page_row(pages, 0);
             if (wide) {
                 uint32x4_t kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
                 if (useful) {
@@ -297,12 +302,18 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     uint32_t vring[DEPTH][2][VW];
     uint32_t nring[DEPTH];
     auto issue_first = [&]() {
+        int pg[DEPTH + 1];
+        if (PAGED) {
+#pragma unroll
+            for (int d = 0; d <= DEPTH; d++) pg[d] = fetch_pages(t0 + 32 * d);
+            pages_next = pg[DEPTH];
+        }
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
             if (d == 0 || t0 + 32 * d < t1) {
-                issue_k(kring[d], t0 + 32 * d);
-                nring[d] = issue_n(t0 + 32 * d);
-                issue_v(vring[d], t0 + 32 * d);
+                issue_k(kring[d], t0 + 32 * d, PAGED ? pg[d] : 0);
+                nring[d] = issue_n(t0 + 32 * d, PAGED ? pg[d] : 0);
+                issue_v(vring[d], t0 + 32 * d, PAGED ? pg[d] : 0);
             }
         }
     };
@@ -440,6 +451,8 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
             const int tile = t0 + 32 * it;
             const int next_tile = tile + 32 * DEPTH;
             const bool more = it + DEPTH < ntiles;
+            const int pages = pages_next;
+            if (PAGED && more) pages_next = fetch_pages(next_tile + 32);
 
             // ---- scores S[head][token] for both sub-tiles
             float4_t s[2];
@@ -469,11 +482,11 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
 #pragma unroll
                 for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[sub], 0, 0, 0);
             }
-            if (more) issue_k(kreg, next_tile);
+            if (more) issue_k(kreg, next_tile, pages);
 
             // ---- online softmax (base 2): this lane owns token ln of sub-tile my_sub
             const float kn = h2f_bits(nreg & 0xffffu), vn = h2f_bits(nreg >> 16);
-            if (more) nreg = issue_n(next_tile);
+            if (more) nreg = issue_n(next_tile, pages);
             const bool valid = useful && (tile + 16 * my_sub + ln < t1);
             float raw[R], x[R];
             bool raise = false;
@@ -529,7 +542,7 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
                         xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
                     }
                 }
-                if (more) issue_v(vreg, next_tile);
+                if (more) issue_v(vreg, next_tile, pages);
 #pragma unroll
                 for (int jp = 0; jp < 4; jp++) {         // two dims (even, odd) per step: 8 look-ups, 2 MFMAs
                     const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
@@ -557,7 +570,7 @@ attention_mfma_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
                     ie[sub] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
                     io[sub] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
                 }
-                if (more) issue_v(vreg, next_tile);
+                if (more) issue_v(vreg, next_tile, pages);
 #pragma unroll
                 for (int q = 0; q < 4; q++) {            // dims (2q, 2q+1): 4 look-ups, 2 MFMAs
                     const uint32_t x0 = (q & 1) ? io[0] : ie[0], x1 = (q & 1) ? io[1] : ie[1];

@@ -125,11 +125,14 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
 
     // Global -> registers: this lane's share of the tile at `tile`.  Rows past the end of the
     // sequence are cut by the descriptors' extents and read as zeros.
-    auto load_tile = [&](int tile, uint4& kr, uint4& vr, uint4& nr) {
+    // Paged: the two block-table entries of a tile (even lanes: first page, odd lanes: second) are
+    // fetched a tile ahead of its loads, so that no load waits for its page number.
+    auto fetch_pages = [&](int tile) -> int { return bt[min(tile + 16 * (lane & 1), t1 - 1) >> 4]; };
+    auto load_tile = [&](int tile, int pages, uint4& kr, uint4& vr, uint4& nr) {
         long long row;
         int rows;
-        if (PAGED) {          // a page is one 16-token sub-tile; past the end re-read the last page (masked)
-            row = (long long)uniform(bt[min(tile + 16 * (wv >> 2), t1 - 1) >> 4]) * kPageTokens;
+        if (PAGED) {          // a page is one 16-token sub-tile; past the end the last page is re-read (masked)
+            row = (long long)__builtin_amdgcn_readlane(pages, wv >> 2) * kPageTokens;
             rows = kPageTokens;
         } else {
             row = seq_row0 + tile;
@@ -144,7 +147,8 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
         if (wv < 2 && lane < 32) {                           // wave 0: the 32 K-norm rows, wave 1: the V-norm rows
             const char* nbase = reinterpret_cast<const char*>(wv ? a.v_norms : a.k_norms);
             if (PAGED) {      // pages are whole: a plain load, one page per half of the tile
-                const long long prow = (long long)bt[min(tile + (lane & 16), t1 - 1) >> 4] * kPageTokens + (lane & 15);
+                const int p0 = __builtin_amdgcn_readlane(pages, 0), p1 = __builtin_amdgcn_readlane(pages, 1);
+                const long long prow = (long long)((lane & 16) ? p1 : p0) * kPageTokens + (lane & 15);
                 nr = *reinterpret_cast<const uint4*>(nbase + prow * 16);
             } else {
                 __amdgpu_buffer_rsrc_t rn = make_rsrc(nbase + (seq_row0 + tile) * 16, max(min(n - tile, 32), 0) * 16);
@@ -236,8 +240,14 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
         const bool have = advance();
         const int ntiles = have ? (t1 - t0 + 31) >> 5 : 0;
         uint4 ra[3] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+        int pages_next = 0;                                  // entries of the tile after the one being loaded
         if (have) {
-            load_tile(t0, ra[0], ra[1], ra[2]);
+            int pages = 0;
+            if (PAGED) {
+                pages = fetch_pages(t0);
+                pages_next = fetch_pages(t0 + 32);
+            }
+            load_tile(t0, pages, ra[0], ra[1], ra[2]);
             stash(0, ra[0], ra[1], ra[2]);
         }
         if (wv == 0 && lane == 0) nt_s[grp] = ntiles;
@@ -381,7 +391,11 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
         // tile that arrived into the other buffer, and meet the other waves.  (Two tiles of loads in
         // flight were measured: no faster.)
         for (int it = 0; it < round_tiles; it++) {
-            if (it + 1 < ntiles) load_tile(t0 + 32 * (it + 1), ra[0], ra[1], ra[2]);
+            if (it + 1 < ntiles) {
+                const int pages = pages_next;
+                if (PAGED && it + 2 < ntiles) pages_next = fetch_pages(t0 + 32 * (it + 2));
+                load_tile(t0 + 32 * (it + 1), pages, ra[0], ra[1], ra[2]);
+            }
             if (it < ntiles) compute(it & 1, t0 + 32 * it);
             if (it + 1 < ntiles) stash((it & 1) ^ 1, ra[0], ra[1], ra[2]);
             __syncthreads();
