@@ -352,6 +352,23 @@ void tw_paged_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const ui
                                         int num_kv_heads, int head_dim, int q_dim, int kv_dim,
                                         int bits, hipStream_t s);
 
+/* No counterpart in the reference.  launch_turbo_gqa_attention_batch for callers that cannot allocate and have
+ * no scratch to hand over (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * the same arguments without `as`, same kernels and results; the split workspace is a device array inside the
+ * library, TW_NOALLOC_SCRATCH_BYTES per GPU, held from the first call on that GPU until the process ends.  The
+ * call allocates and frees nothing (no hipMalloc / hipFree / event or stream creation); its first call on a GPU
+ * looks the array's address up once and should not happen under stream capture.
+ * Limit: G * num_heads <= TW_NOALLOC_MAX_HEAD_VECTORS, else nothing is launched and an error is returned.
+ * All calls on one GPU share that GPU's array, which keeps the last call's contents (nothing in it needs to
+ * start at zero: a call reads only what it wrote itself): calls that overlap on one GPU race -- run them on one
+ * stream, or order them.  Returns 0, or non-zero with the message in tw_kv_last_error_string(). */
+#define TW_NOALLOC_SCRATCH_BYTES (32u << 20)
+#define TW_NOALLOC_MAX_HEAD_VECTORS 16384
+int tw_turbo_gqa_attention_batch_noalloc(tw_half* out, const tw_half* q, const uint8_t* ck_q, const uint8_t* cv_q,
+                                         const tw_half* k_norms, const tw_half* v_norms, const tw_half* rotation,
+                                         const int* pos, int msl, int G, int num_heads, int num_kv_heads,
+                                         int head_dim, int q_dim, int kv_dim, int bits, hipStream_t s);
+
 /* Host: the rotation matrix of engine.cpp:366-392 (mt19937(42), N(0,1),
  * modified Gram-Schmidt over rows, fp16).  out: head_dim*head_dim halves, HOST. */
 void tw_make_rotation_host(tw_half* out_host, int head_dim, unsigned seed);

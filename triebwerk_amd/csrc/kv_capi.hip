@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <random>
 #include <vector>
 
@@ -158,8 +159,8 @@ void attach_profiler(hipStream_t s) {
     if (prof) { t_scan_start = g_prof.start[g_prof.used]; t_scan_stop = g_prof.stop[g_prof.used]; g_prof.used++; }
 }
 
-void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done = false) {
-    attach_profiler(s);
+void run_attention(AttnArgs& a, hipStream_t s, const char* fn, bool query_done = false, bool may_profile = true) {
+    if (may_profile) attach_profiler(s);   // creates events on first use: not for the entry point that allocates nothing
     if (a.bits == 0 && g_variant.load() != 1 && prefill_f16_mfma_usable(a)) {   // fp16 prefill: one MFMA kernel, no splits
         launch_prefill_f16_mfma(a, s, g_prefill_form.load());
         t_scan_start = t_scan_stop = nullptr;
@@ -940,6 +941,73 @@ void launch_turbo_gqa_prefill_attention(tw_half* out, const tw_half* q, const ui
     a.pos_mode = kPosIota; a.seq_stride_rows = 0;
     plan_splits(a, T, T);
     run_attention(a, s, "launch_turbo_gqa_prefill_attention");
+}
+
+// ---------------------------------------------------------------- attention without any allocation
+}  // extern "C"
+
+// The split workspace of launch_turbo_gqa_attention_batch as a device array of the library itself, for callers
+// that can neither allocate nor hand over scratch memory.  In host code the array's name only stands for the
+// symbol: its address on a device comes from hipGetSymbolAddress with that device current (every device has its
+// own copy), is looked up once per device and is what the kernels get.
+static __device__ __align__(256) float scratch[TW_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+
+namespace {
+constexpr int kNoallocMaxDevices = 64;
+float* g_scratch_ptr[kNoallocMaxDevices];   // per device, nullptr = not looked up yet
+std::mutex g_scratch_mutex;
+
+float* static_scratch_on_current_device(const char* fn) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kNoallocMaxDevices) {
+        set_error(e != hipSuccess ? (int)e : 1, "%s: no usable current device (%d)", fn, dev);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_error(e != hipSuccess ? (int)e : 1, "%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" {
+
+int tw_turbo_gqa_attention_batch_noalloc(tw_half* out, const tw_half* q, const uint8_t* ck_q, const uint8_t* cv_q,
+                                         const tw_half* k_norms, const tw_half* v_norms, const tw_half* rotation,
+                                         const int* pos, int msl, int G, int num_heads, int num_kv_heads, int head_dim,
+                                         int q_dim, int kv_dim, int bits, hipStream_t s) {
+    const char* fn = "tw_turbo_gqa_attention_batch_noalloc";
+    if (!check_shape(fn, num_heads, num_kv_heads, head_dim) || !check_bits(fn, bits)) return 1;
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, kv_dim);
+        return 1;
+    }
+    if (G <= 0 || msl <= 0) { set_error(1, "%s: G=%d, msl=%d", fn, G, msl); return 1; }
+    if ((long long)G * num_heads > TW_NOALLOC_MAX_HEAD_VECTORS) {
+        set_error(1, "%s: G*num_heads=%lld exceeds the %d (sequence, head) pairs the library's %d MiB of scratch serve",
+                  fn, (long long)G * num_heads, TW_NOALLOC_MAX_HEAD_VECTORS, (int)(TW_NOALLOC_SCRATCH_BYTES >> 20));
+        return 1;
+    }
+    float* ws = static_scratch_on_current_device(fn);
+    if (!ws) return 2;
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads, num_kv_heads, bits, ws);
+    a.pos_mode = kPosArray; a.positions = pos; a.seq_stride_rows = msl;
+    // the room per (sequence, head) the reference-signature launcher has (msl floats) when the array gives that much:
+    // then both make the same plan and the same bits
+    const long long room = (long long)(TW_NOALLOC_SCRATCH_BYTES / sizeof(float)) / ((long long)G * num_heads);
+    plan_splits(a, msl, room < msl ? room : msl);
+    const int before = g_err;
+    run_attention(a, s, fn, /*query_done=*/false, /*may_profile=*/false);
+    return (before == 0 && g_err != 0) ? 3 : 0;
 }
 
 void tw_paged_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half* ck,

@@ -118,6 +118,22 @@ def launch_turbo_gqa_attention_batch(out, q, ck_q, cv_q, k_norms, v_norms, rotat
     _done(lib)
 
 
+def tw_turbo_gqa_attention_batch_noalloc(out, q, ck_q, cv_q, k_norms, v_norms, rotation, pos, msl, G, num_heads,
+                                         num_kv_heads, head_dim, q_dim, kv_dim, bits, stream=None):
+    """launch_turbo_gqa_attention_batch without the scratch argument: the library's own device array is the
+    workspace and the call allocates nothing."""
+    lib = _lib.load()
+    rc = lib.tw_turbo_gqa_attention_batch_noalloc(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"),
+                                                  _ptr(ck_q, "u8", "ck_q"), _ptr(cv_q, "u8", "cv_q"),
+                                                  _ptr(k_norms, "f16", "k_norms"), _ptr(v_norms, "f16", "v_norms"),
+                                                  _ptr(rotation, "f16", "rotation"), _ptr(pos, "i32", "pos"), msl, G,
+                                                  num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits,
+                                                  _stream(stream))
+    _done(lib)
+    if rc != 0:
+        raise RuntimeError(f"tw_turbo_gqa_attention_batch_noalloc returned {rc}")
+
+
 def launch_turbo_gqa_prefill_attention(out, q, ck_q, cv_q, k_norms, v_norms, rotation, scratch, T,
                                        msl, num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits,
                                        stream=None):
