@@ -49,9 +49,37 @@ BYTES_HEAD = {0: 256, 4: 66, 2: 34}  # per (token, kv head): fp16 row | codes + 
 # HBM bytes per launch (read + write) of the context-scanning kernel, from rocprofv3 --pmc FETCH_SIZE
 # and WRITE_SIZE on this file's own run, each counter scaled by what `--copy-calibration` reads for a
 # copy of known size (2.0 and 1.0); summary and commands in profiles/scan_target_hbm_traffic_pmc.txt.
-# Keyed by (workload, kv_bits, kernel that ran); a measurement of the kernels as committed with that file, not live.
+# Keyed by (workload, kv_bits, kernel that ran).  Counters are not read in this run: the figures belong to
+# the kernel sources whose digest is recorded with them (`python bench.py --csrc-digest` prints the current
+# one) and are only reported while the sources are still those; otherwise `traffic` is null.
+MEASURED_TRAFFIC_CSRC_DIGEST = "unset"
 MEASURED_TRAFFIC_BYTES = {("target", 4, "one-launch"): 556.6e6, ("target", 4, "scan"): 560.8e6,
                           ("target", 2, "scan"): 292.2e6, ("target", 0, "scan"): 2151.8e6}
+TRAFFIC_SOURCE = "profiles/scan_target_hbm_traffic_pmc.txt"
+
+
+def csrc_digest() -> str:
+    """Digest of the kernel sources (triebwerk_amd/csrc), file names and contents in sorted order."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in sorted((ROOT / "triebwerk_amd" / "csrc").iterdir()):
+        if f.suffix in (".hip", ".hpp"):
+            h.update(f.name.encode()); h.update(b"\0"); h.update(f.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload: str, kv_bits: int, one_launch: bool):
+    """(bytes or None, where the figure comes from)."""
+    if csrc_digest() != MEASURED_TRAFFIC_CSRC_DIGEST:
+        return None, f"none: kernel sources changed since {TRAFFIC_SOURCE} was measured"
+    val = MEASURED_TRAFFIC_BYTES.get((workload, kv_bits, "one-launch" if one_launch else "scan"))
+    return val, (f"{TRAFFIC_SOURCE} (rocprofv3 --pmc, not read in this run; kernel sources {MEASURED_TRAFFIC_CSRC_DIGEST})"
+                 if val is not None else "none: not measured for this workload")
+
+
+DTYPE = {0: "f16 cache, f32 accumulate (vector ALU)",
+         4: "u8 codes (4 bit) + f16 norms -> f16-operand MFMA (centroids as f16, q and p as f16 hi+lo pairs), f32 accumulate",
+         2: "u8 codes (2 bit) + f16 norms -> f16-operand MFMA (centroids as f16, q and p as f16 hi+lo pairs), f32 accumulate"}
 
 
 def algorithmic_bytes(n_tokens_total: int, G: int, L: int, H: int, Hk: int, kv_bits: int, with_append: bool) -> int:
@@ -210,7 +238,7 @@ def prefill_bench(args):
     print(json.dumps({
         "metric": "prefill-attn prompt tokens/s (one layer)", "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": max(args.warmup, 1), "ms_per_step": ms, "higher_is_better": True,
-        "dtype": "f32 accumulate over f16" if not kv_bits else "f32 accumulate over u8 codes + f16 norms", "data": "synthetic",
+        "dtype": "f16-operand MFMA, f32 accumulate" if not kv_bits else DTYPE[kv_bits], "data": "synthetic",
         "config": {"workload": f"causal prefill attention, one sequence, {T} tokens, {H} heads over {Hk} KV heads",
                    "kv_bits": kv_bits if kv_bits else 16, "variant": args.variant,
                    "timed": ["the attention launch", "tw_layer_prompt_step: producers + T-token append + attention (+ 2 copies restoring q and k)",
@@ -321,7 +349,7 @@ def paged_bench(args):
     print(json.dumps({
         "metric": "decode-attn tokens/s", "value": G * K / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": K,
         "warmup": W, "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32 accumulate over u8 codes + f16 norms", "data": "synthetic",
+        "vs_baseline": None, "dtype": DTYPE[kv_bits], "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}, paged cache: 16-token pages, block table in random page order",
                    "kv_bits": kv_bits, "layers": L, "num_heads": H, "num_kv_heads": Hk, "head_dim": D, "batch": G,
                    "pages": n_pages, "context_first_timed_step": [int(ctx0.min()), int(ctx0.max())],
@@ -355,6 +383,12 @@ def main():
     ap.add_argument("--ctx", type=int, default=None, help="override the workload's context length")
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--layers", type=int, default=None, help="override the workload's layer count")
+    ap.add_argument("--launchers", default="engine", choices=["engine", "reference"],
+                    help="engine: one tw_layer_attention_step per layer (default); reference: only the launchers the "
+                         "reference's forward_layer_batch calls (two appends + attention per layer), captured in a graph")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="default run: skip the other two cache widths (per_kv_bits)")
+    ap.add_argument("--csrc-digest", action="store_true", help="print the digest of the kernel sources and exit")
     ap.add_argument("--paged", action="store_true",
                     help="the same step over a paged cache (16-token pages, block table in random page order) through "
                          "the tw_paged_* entry points; compressed caches only")
@@ -371,6 +405,9 @@ def main():
                     help="instead of the decode step, time causal prefill attention over a T-token prompt of one "
                          "sequence (one layer's launch, the workload's head counts, --kv-bits cache) and exit")
     args = ap.parse_args()
+    if args.csrc_digest:
+        print(csrc_digest())
+        return
     if args.prefill:
         prefill_bench(args)
         return
@@ -392,11 +429,34 @@ def main():
         paged_bench(args)
         return
 
-    import torch
-    from triebwerk_amd import Engine, _lib, kvcache
+    headline_bits = WORKLOADS[args.workload]["kv_bits"] if args.kv_bits is None else args.kv_bits
+    result = decode_bench(args, headline_bits, with_probe=True)
+    # The metric is quoted at kv_bits = 16 / 4 / 2: the default run measures the other two widths of the same
+    # workload as well (same shapes and steps; no CPU leg, no read probe) and reports them beside the headline.
+    default_run = (args.workload == "target" and args.kv_bits is None and args.ctx is None and args.batch is None and
+                   args.layers is None and args.producers == "none" and args.launchers == "engine" and
+                   not args.headline_only)
+    if default_run:
+        per = {str(headline_bits if headline_bits else 16): compact(result)}
+        for bits in (2, 0):
+            if bits != headline_bits:
+                per[str(bits if bits else 16)] = compact(decode_bench(args, bits, with_probe=False))
+        result["per_kv_bits"] = {k: per[k] for k in ("16", "4", "2") if k in per}
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(workload_of(args), headline_bits)
+    print(json.dumps(result))
 
+
+def compact(r):
+    """The figures of one cache width for the per_kv_bits table."""
+    return {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "step_achieved_GBps": r["step_achieved_GBps"],
+            "step_frac_of_hbm_peak": r["step_frac_of_hbm_peak"], "dtype": r["dtype"], "launches_per_layer": r["config"]["launches_per_layer"],
+            "roofline": {k: r["roofline"][k] for k in ("kernel", "achieved", "frac", "launch_ms", "launch_ms_timed", "launch_algorithmic_MB",
+                                                       "traffic", "traffic_source")}}
+
+
+def workload_of(args):
     w = dict(WORKLOADS[args.workload])
-    kv_bits = w["kv_bits"] if args.kv_bits is None else args.kv_bits
     overridden = []
     for key, val in (("ctx", args.ctx), ("G", args.batch), ("L", args.layers)):
         if val is not None:
@@ -404,6 +464,17 @@ def main():
             overridden.append(f"{key}={val}")
     if overridden:
         w["desc"] += " [override " + ",".join(overridden) + "]"
+    w["overridden"] = bool(overridden)
+    return w
+
+
+def decode_bench(args, kv_bits, with_probe):
+    """W warm-up steps, K timed steps (one hipGraph replay each), then the dominant kernel's launches timed
+    one by one, for one cache width.  Returns the result dictionary (without the CPU leg)."""
+    import torch
+    from triebwerk_amd import Engine, _lib, kvcache
+
+    w = workload_of(args)
     L, H, Hk, G, D = w["L"], w["H"], w["Hk"], w["G"], 128
     K, W = args.steps, args.warmup
     kv_dim, q_dim = Hk * D, H * D
@@ -483,20 +554,65 @@ def main():
         rope_cos, rope_sin = torch.cos(ang).to(torch.float16).contiguous(), torch.sin(ang).to(torch.float16).contiguous()
         eng.set_producers(1 if args.producers == "fused" else 2, q_norm, k_norm, 1e-6, False, rope_cos, rope_sin, D)
 
-    def step():
-        eng.decode_step(q, k, v, out, use_graph=use_graph, stream=stream)
+    if args.launchers == "reference":
+        # forward_layer_batch's own calls and nothing else (engine.cpp:1979-2006, 2394): what an engine whose
+        # source is left as it is gets from this library
+        if args.producers != "none":
+            sys.exit("bench.py: --launchers reference runs the append and attention launchers only")
+        caches = [eng.cache(l) for l in range(L)]
+        rot = eng.rotation()
+        pos = eng.positions()
+        scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+
+        def layers():
+            for l in range(L):
+                ck, cv, kn, vn = caches[l]
+                if kv_bits == 0:
+                    kvcache.launch_kv_cache_write_batch(ck, cv, k[l], v[l], pos, msl, G, kv_dim)
+                    kvcache.launch_gqa_attention_batch(out[l], q[l], ck, cv, scratch, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+                else:
+                    kvcache.launch_turbo_kv_quantize_batch(ck, kn, k[l], rot, pos, msl, G, Hk, D, kv_dim, kv_bits)
+                    kvcache.launch_turbo_kv_quantize_batch(cv, vn, v[l], rot, pos, msl, G, Hk, D, kv_dim, kv_bits)
+                    kvcache.launch_turbo_gqa_attention_batch(out[l], q[l], ck, cv, kn, vn, rot, scratch, pos, msl, G, H, Hk, D,
+                                                             q_dim, kv_dim, kv_bits)
+            kvcache.launch_increment_positions(pos, G)
+
+        eager_step = layers
+        with torch.cuda.stream(stream):
+            layers()                                         # first warm-up step, eager (loads the kernels)
+            if use_graph:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=stream):
+                    layers()
+                graph.replay()                               # the captured step was recorded, not run
+        torch.cuda.synchronize()
+        step = graph.replay if use_graph else layers
+        warm_done = 2 if use_graph else 1
+    else:
+        def step():
+            eng.decode_step(q, k, v, out, use_graph=use_graph, stream=stream)
+
+        def eager_step():
+            eng.decode_step(q, k, v, out, use_graph=False, stream=stream)
+        warm_done = 0
 
     with torch.cuda.stream(stream):
-        for _ in range(W):
+        for _ in range(max(W - warm_done, 0)):
             step()
     torch.cuda.synchronize()
-    pos_now = start_pos.astype(np.int64) + W
+    W_run = max(W, warm_done)
+    pos_now = start_pos.astype(np.int64) + W_run
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    fused_before = lib.tw_kv_decode_fused_launches()
     t0 = time.perf_counter()
     with torch.cuda.stream(stream):
+        e0.record(stream)
         for _ in range(K):
             step()
+        e1.record(stream)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    events_ms = e0.elapsed_time(e1)      # the same K steps as seen by events on the launch stream
     n_tokens_timed = int(sum(int((pos_now + i + 1).sum()) for i in range(K)))   # attended tokens, all steps
     pos_now = pos_now + K
     assert np.array_equal(eng.positions().cpu().numpy().astype(np.int64), pos_now), "positions drifted"
@@ -515,59 +631,86 @@ def main():
     lib.tw_kv_profile_attention(1)
     with torch.cuda.stream(stream):
         for _ in range(Kp):
-            eng.decode_step(q, k, v, out, use_graph=False, stream=stream)
+            eager_step()
     torch.cuda.synchronize()
     total_ms, launches = C.c_double(0), C.c_int(0)
     rc = lib.tw_kv_profile_read(C.byref(total_ms), C.byref(launches))
     lib.tw_kv_profile_attention(0)
     assert rc == 0 and launches.value == Kp * L, (rc, launches.value)
     n_tokens_prof = int(sum(int((pos_now + i + 1).sum()) for i in range(Kp)))
-    kern_ms = total_ms.value / launches.value
+    eager_kern_ms = total_ms.value / launches.value
     # which kernel those launches were: the whole layer step in one launch (append included), or the scan of the
     # three-kernel path
     one_launch = lib.tw_kv_decode_fused_launches() - fused_before == Kp * L
     launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=one_launch) / (Kp * L)
+    if one_launch and use_graph:
+        # The layer step is this one kernel, so the timed region itself is K * L launches of it (plus K one-block
+        # position increments): its average duration there, the launches `value` is made of, is the events' time
+        # over the region divided by the launches.  (Launched one by one with events attached the same kernel
+        # reads 1-2 % longer: a replayed graph overlaps one kernel's drain with the next one's start.)
+        kern_ms = events_ms / (K * L)
+        launch_bytes = algorithmic_bytes(n_tokens_timed, G * K, L, H, Hk, kv_bits, with_append=True) / (K * L)
+        timed = (f"HIP events on the launch stream around the {K} graph-replayed steps of the timed region / ({K} x {L}) launches; "
+                 "includes 1/L of a one-block positions += 1 kernel per launch")
+    else:
+        kern_ms = eager_kern_ms
+        timed = (f"a pair of HIP events attached to each of {Kp * L} eager launches of the kernel on its stream, in steps that "
+                 "continue the timed decode")
     achieved = launch_bytes / (kern_ms * 1e-3) * 1e-9
+    if args.launchers == "reference":
+        launches_per_layer = 3 if kv_bits == 0 else 5     # write + scan + merge | 2 appends + query rotation + scan + merge
+    else:
+        launches_per_layer = 1 if one_launch else (2 if kv_bits == 0 else 3)
 
-    # ---- what a plain contiguous read kernel reaches on this GPU: over 4 GiB, and over exactly the
-    # scan's bytes per launch on memory not touched since (launch overheads included, as for the scan)
-    probe = torch.empty(int(4 << 30), dtype=torch.uint8, device="cuda")
-    probe.fill_(1)
-    torch.cuda.synchronize()
-    lib.tw_kv_measure_read_bandwidth.restype = C.c_double
-    read_big = lib.tw_kv_measure_read_bandwidth(C.c_void_p(probe.data_ptr()), C.c_size_t(probe.numel()), 3,
-                                                C.c_void_p(stream.cuda_stream))
-    nb = int(launch_bytes) // 16 * 16
-    same, reps = 0.0, 0
-    for off in range(0, probe.numel() - nb + 1, max(nb, 1) + (1 << 20)):
-        same += lib.tw_kv_measure_read_bandwidth(C.c_void_p(probe.data_ptr() + off // 16 * 16), C.c_size_t(nb), 1,
-                                                 C.c_void_p(stream.cuda_stream))
-        reps += 1
-        if reps == 6:
-            break
-    read_same = same / max(reps, 1)
-    del probe
+    read_big = read_same = None
+    if with_probe:
+        # ---- what a plain contiguous read kernel reaches on this GPU: over 4 GiB, and over exactly the
+        # scan's bytes per launch on memory not touched since (launch overheads included, as for the scan)
+        probe = torch.empty(int(4 << 30), dtype=torch.uint8, device="cuda")
+        probe.fill_(1)
+        torch.cuda.synchronize()
+        lib.tw_kv_measure_read_bandwidth.restype = C.c_double
+        read_big = lib.tw_kv_measure_read_bandwidth(C.c_void_p(probe.data_ptr()), C.c_size_t(probe.numel()), 3,
+                                                    C.c_void_p(stream.cuda_stream))
+        nb = int(launch_bytes) // 16 * 16
+        same, reps = 0.0, 0
+        for off in range(0, probe.numel() - nb + 1, max(nb, 1) + (1 << 20)):
+            same += lib.tw_kv_measure_read_bandwidth(C.c_void_p(probe.data_ptr() + off // 16 * 16), C.c_size_t(nb), 1,
+                                                     C.c_void_p(stream.cuda_stream))
+            reps += 1
+            if reps == 6:
+                break
+        read_same = same / max(reps, 1)
+        del probe
 
+    traffic, traffic_source = (measured_traffic(args.workload, kv_bits, one_launch)
+                               if not w["overridden"] and args.producers == "none" and args.launchers == "engine"
+                               else (None, "none: not measured for this variation of the workload"))
     result = {
         "metric": "decode-attn tokens/s",
         "value": tokens_per_s,
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": K,
-        "warmup": W,
+        "warmup": W_run,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 accumulate over u8 codes + f16 norms" if kv_bits else "f32 accumulate over f16",
+        "dtype": DTYPE[kv_bits],
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: {w['desc']}" + (f" [kv_bits={kv_bits}]" if kv_bits != w["kv_bits"] else ""),
+            "workload": f"{args.workload}: {w['desc']}" + (f" [kv_bits={kv_bits}]" if kv_bits != WORKLOADS[args.workload]["kv_bits"] else ""),
             "kv_bits": kv_bits if kv_bits else 16,
             "layers": L, "num_heads": H, "num_kv_heads": Hk, "head_dim": D, "batch": G,
             "context_first_timed_step": [int(ctx0.min()), int(ctx0.max())],
             "tokens_attended_per_step": n_tokens_timed / K,
             "hipgraph": use_graph,
+            "launchers": ("tw_layer_attention_step per layer (engine object)" if args.launchers == "engine" else
+                          "the reference's own launchers only: " +
+                          ("launch_kv_cache_write_batch + launch_gqa_attention_batch" if kv_bits == 0 else
+                           "launch_turbo_kv_quantize_batch x2 + launch_turbo_gqa_attention_batch") + " per layer, launch_increment_positions"),
+            "launches_per_layer": launches_per_layer,
             "step": ("append K,V + decode attention for every layer, positions += 1" if args.producers == "none" else
                      f"QK RMSNorm + RoPE ({args.producers}) + append K,V + decode attention for every layer, positions += 1"),
             **({"shared_prefix_tokens": w["prefix"][0], "prefix_append_and_broadcast_ms": prefix_ms} if w.get("prefix") else {}),
@@ -584,16 +727,20 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "launch_ms": kern_ms,
+            "launch_ms_timed": timed,
+            "launch_ms_eager_events": eager_kern_ms,
             "launch_algorithmic_MB": launch_bytes * 1e-6,
             "plain_read_GBps_4GiB": read_big,
             "plain_read_GBps_same_bytes_per_launch": read_same,
-            "traffic": (MEASURED_TRAFFIC_BYTES.get((args.workload, kv_bits, "one-launch" if one_launch else "scan"))
-                        if not overridden and args.producers == "none" else None),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
         },
     }
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(w, kv_bits)
-    print(json.dumps(result))
+    if args.producers != "none":
+        eng.set_producers(0)
+    del eng, q, k, v, out
+    torch.cuda.empty_cache()
+    return result
 
 
 if __name__ == "__main__":

@@ -397,13 +397,19 @@ int tw_engine_set_shape(tw_engine* e, const tw_model_shape* shape);
 
 /* alloc_batch, engine.cpp:1338-1560: one arena for G sequences of max_seq_len
  * rows, carved with 256-byte alignment in the reference's order (keys, values,
- * key norms, value norms per layer).  Returns 0 on success. */
+ * key norms, value norms per layer).  Returns 0 on success.  A call with the G and max_seq_len the engine
+ * already has changes nothing; any other carves the caches anew and zeroes them -- inside the memory already
+ * held when that is big enough -- so the steps below always work on exactly G rows (the reference keeps a
+ * larger batch and its strides, engine.cpp:1339). */
 int tw_engine_alloc_batch(tw_engine* e, int G, int max_seq_len);
 /* set_arena, engine.cpp:1609-1620: carve out of caller-owned device memory. */
 int tw_engine_set_arena(tw_engine* e, void* device_ptr, size_t bytes);
 size_t tw_engine_arena_bytes_needed(const tw_engine* e, int G, int max_seq_len);
 
-/* reset(), engine.cpp:893-916 / 2262-2283: zero every cache, positions to 0. */
+/* reset(), engine.cpp:893-916 / 2262-2283: zero every cache, positions to 0.
+ * Stream order: reset, set_positions, alloc_batch, set_arena and sleep first wait for the stream the latest
+ * step, prompt layer or prefix broadcast was issued on; reset returns when its own work is done.  Work that the
+ * caller put on other streams is the caller's to order. */
 int tw_engine_reset(tw_engine* e);
 
 /* Device pointers into the arena (for tests and for callers that keep using
@@ -411,6 +417,10 @@ int tw_engine_reset(tw_engine* e);
 void* tw_engine_cache_ptr(tw_engine* e, int layer, int which);
 int* tw_engine_positions(tw_engine* e);          /* device int32[G] */
 const tw_half* tw_engine_rotation(tw_engine* e); /* device, NULL when kv_bits==0 */
+/* Host positions (each in [0, max_seq_len)) to the device array, engine.cpp:2364.  The engine keeps their range
+ * on the host and advances it with every decode step: it picks the kernels from it, and refuses a step (-8,
+ * nothing launched, cache and positions untouched) once a sequence has used its last row.  A caller that writes
+ * the device array itself must keep positions[g] < max_seq_len on its own. */
 int tw_engine_set_positions(tw_engine* e, const int* host_positions, int G);
 
 /* Make the producers of q and k part of every step (forward_layer_batch step 3,
@@ -440,7 +450,9 @@ int tw_engine_prompt_layer(tw_engine* e, int layer, int seq, const tw_half* q, c
 /* All layers, then positions += 1.  q/out: (L, G, q_dim); k/v: (L, G, kv_dim).
  * With use_graph != 0 the step is captured once into a hipGraph and replayed
  * (engine.cpp:2369-2412, 2480); the capture is dropped when the arena, G or
- * the buffers change. */
+ * the buffers change, and made again when the context lengths the host knows of have moved to where the other
+ * choice of kernels (tw_kv_decode_step_plan) applies.  -8: a sequence has no row left (see
+ * tw_engine_set_positions). */
 int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v,
                           tw_half* out, int use_graph, hipStream_t s);
 
@@ -451,8 +463,9 @@ int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end
 
 /* sleep() / wake(), engine.cpp:922-1022: sleep hands the cache memory back (frees an arena the engine
  * allocated, forgets one the caller owns), drops the captured step and the generation bookkeeping;
- * wake has nothing to restore for the batch path -- tw_engine_alloc_batch (or tw_engine_set_arena +
- * tw_engine_alloc_batch) re-creates it on the next use, zeroed. */
+ * wake is intentionally empty: the reference's wake re-allocates the single-sequence caches it freed in sleep
+ * (engine.cpp:985-1022), state this engine object does not own, and the batch state is re-created, zeroed, by the
+ * next tw_engine_alloc_batch (or tw_engine_set_arena + tw_engine_alloc_batch), as in the reference. */
 int tw_engine_sleep(tw_engine* e);
 int tw_engine_wake(tw_engine* e);
 int tw_engine_is_allocated(const tw_engine* e);

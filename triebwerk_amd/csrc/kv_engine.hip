@@ -62,6 +62,17 @@ struct tw_engine {
     hipGraphExec_t graph_exec = nullptr;
     const void* graph_key[4] = {};
     int graph_G = 0;
+    int graph_plan = 0;               // tw_kv_decode_step_plan's answer the captured launches were chosen under
+
+    // The stream of the latest step: reset, set_positions and everything that lets go of the arena wait for it
+    // first (a caller's stream has no implicit order with the engine's own stream or with the null stream).
+    hipStream_t last_stream = nullptr;
+    bool steps_in_flight = false;
+    void note_step(hipStream_t s) { last_stream = s; steps_in_flight = true; }
+    void wait_for_steps() {
+        if (steps_in_flight) (void)hipStreamSynchronize(last_stream);
+        steps_in_flight = false;
+    }
 
     // generation bookkeeping (generate_batch, engine.cpp:2350, 2496-2534)
     int* d_token_history = nullptr;   // (max_new_tokens, G) device
@@ -95,6 +106,7 @@ struct tw_engine {
         graph_G = 0;
     }
     void drop_arena() {
+        wait_for_steps();
         drop_graph();  // the capture holds arena addresses, engine.cpp:1440-1442
         drop_generation();
         if (arena && arena_owned) hipFree(arena);
@@ -158,6 +170,18 @@ int carve(tw_engine* e, int G, int msl) {
 }
 
 hipStream_t pick(tw_engine* e, hipStream_t s) { return s ? s : e->stream; }
+
+// A step appends at positions[g]: once the furthest sequence the host knows of has used its last row there is no
+// row left, and the append would land in the next sequence's rows (or past the array).
+bool cache_full(const tw_engine* e) { return e->pos_known && e->pos_max >= e->batch_msl; }
+
+// What tw_layer_attention_step will choose for the compressed cache from the host's view of the positions
+// (one launch per layer or three); the captured graph holds the launches of one such choice.
+int step_plan(const tw_engine* e) {
+    if (e->kv_bits == 0) return 0;
+    return tw_kv_decode_step_plan(e->G, e->shape.num_heads, e->shape.num_kv_heads, e->kv_bits, e->batch_msl,
+                                  e->pos_known ? e->pos_min + 1 : 0, e->pos_known ? e->pos_max + 1 : 0);
+}
 
 // forward_layer_batch steps 4-5 (with producers: 3-5), engine.cpp:1972-2006.
 void layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, const tw_half* v,
@@ -244,10 +268,13 @@ size_t tw_engine_arena_bytes_needed(const tw_engine* e, int G, int max_seq_len) 
 int tw_engine_alloc_batch(tw_engine* e, int G, int max_seq_len) {
     if (G < 1 || max_seq_len < 1) return -1;
     if (!e->stream && hipStreamCreate(&e->stream) != hipSuccess) return -3;
-    // engine.cpp:1339: keep a batch that is already large enough.
-    if (e->arena && e->G >= G && e->batch_msl >= max_seq_len) return 0;
+    // engine.cpp:1339 keeps a batch that is already large enough and goes on striding with its G and max_seq_len.
+    // Here the steps take their row counts and strides from the batch as allocated, so only an identical batch
+    // is kept as it is; a different one is carved anew (and zeroed), inside the memory already held when that
+    // is big enough.
+    if (e->arena && e->G == G && e->batch_msl == max_seq_len) return 0;
     size_t need = arena_need(e, G, max_seq_len);
-    if (!(e->arena && !e->arena_owned && e->arena_cap >= need)) {
+    if (!(e->arena && e->arena_cap >= need)) {
         e->drop_arena();
         void* p = nullptr;
         if (hipMalloc(&p, need) != hipSuccess) return -2;
@@ -255,7 +282,9 @@ int tw_engine_alloc_batch(tw_engine* e, int G, int max_seq_len) {
         e->arena_cap = need;
         e->arena_owned = true;
     } else {
+        e->wait_for_steps();
         e->drop_graph();
+        e->drop_generation();
     }
     int rc = carve(e, G, max_seq_len);
     if (rc != 0) return rc;
@@ -273,6 +302,7 @@ int tw_engine_set_arena(tw_engine* e, void* device_ptr, size_t bytes) {
 
 int tw_engine_reset(tw_engine* e) {
     if (!e->arena || e->G == 0) return 0;
+    e->wait_for_steps();
     hipStream_t s = e->stream;
     const size_t rows = (size_t)e->G * e->batch_msl;
     for (int i = 0; i < e->shape.num_layers; i++) {
@@ -303,6 +333,7 @@ int tw_engine_set_positions(tw_engine* e, const int* host_positions, int G) {
     if (!e->d_positions || G > e->G) return -1;
     for (int g = 0; g < G; g++)
         if (host_positions[g] < 0 || host_positions[g] >= e->batch_msl) return -2;
+    e->wait_for_steps();
     // engine.cpp:2364
     if (hipMemcpy(e->d_positions, host_positions, (size_t)G * sizeof(int), hipMemcpyHostToDevice) != hipSuccess) return -3;
     e->pos_known = G == e->G && G > 0;
@@ -425,8 +456,11 @@ int tw_engine_host_position(const tw_engine* e, int g) {
 int tw_engine_layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k,
                          const tw_half* v, tw_half* out, hipStream_t s) {
     if (!e->arena || layer < 0 || layer >= e->shape.num_layers) return -1;
+    if (cache_full(e)) return -8;
     tw_kv_clear_error();
-    layer_step(e, layer, q, k, v, out, pick(e, s));
+    s = pick(e, s);
+    e->note_step(s);
+    layer_step(e, layer, q, k, v, out, s);
     return tw_kv_last_error();
 }
 
@@ -437,6 +471,7 @@ int tw_engine_prompt_layer(tw_engine* e, int layer, int seq, const tw_half* q, c
         return -1;
     if (T == 0) return 0;
     s = pick(e, s);
+    e->note_step(s);
     tw_kv_clear_error();
     const tw_model_shape& m = e->shape;
     tw_half* qm = const_cast<tw_half*>(q);      // with producers q and k are the caller's scratch rows
@@ -481,7 +516,9 @@ int tw_engine_prompt_layer(tw_engine* e, int layer, int seq, const tw_half* q, c
 int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v,
                           tw_half* out, int use_graph, hipStream_t s) {
     if (!e->arena) return -1;
+    if (cache_full(e)) return -8;          // before any launch or replay: cache and positions stay as they are
     s = pick(e, s);
+    e->note_step(s);
     tw_kv_clear_error();
     if (!use_graph) {
         all_layers(e, q, k, v, out, s);
@@ -489,7 +526,10 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
         return tw_kv_last_error();
     }
     const void* key[4] = {q, k, v, out};
-    if (!e->graph_exec || e->graph_G != e->G || memcmp(key, e->graph_key, sizeof(key)) != 0) {
+    // The launches in a captured step were chosen from the context lengths at capture; when the lengths have
+    // grown (or spread) to where the other kernels are the better choice, the step is captured again.
+    const int plan = step_plan(e);
+    if (!e->graph_exec || e->graph_G != e->G || e->graph_plan != plan || memcmp(key, e->graph_key, sizeof(key)) != 0) {
         e->drop_graph();
         // Capture records the launches without running them, so unlike the
         // reference (engine.cpp:2414-2444) nothing has to be re-prefilled.
@@ -509,6 +549,7 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
         }
         e->graph = g;
         e->graph_G = e->G;
+        e->graph_plan = plan;
         memcpy(e->graph_key, key, sizeof(key));
     }
     if (hipGraphLaunch(e->graph_exec, s) != hipSuccess) return -7;
@@ -520,6 +561,7 @@ int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end
     if (!e->arena || src < 0 || src >= e->G || dst_begin < 0 || dst_end > e->G || T < 0 || T > e->batch_msl)
         return -1;
     s = pick(e, s);
+    e->note_step(s);
     const size_t msl = (size_t)e->batch_msl;
     for (int l = 0; l < e->shape.num_layers; l++) {
         void* bases[4];

@@ -57,12 +57,16 @@ class Engine:
         """Carve the caches for G sequences out of one torch-owned arena
         (the reference's set_arena + alloc_batch, engine.cpp:1609-1620, 1338)."""
         need = self._lib.tw_engine_arena_bytes_needed(self._h, G, max_seq_len)
-        arena = torch.empty(need + 256, dtype=torch.uint8, device=device)
-        base = (arena.data_ptr() + 255) & ~255
-        rc = self._lib.tw_engine_set_arena(self._h, base, need)
-        if rc != 0:
-            raise RuntimeError(f"set_arena failed ({rc})")
-        self._arena = arena
+        if self._arena is None or self._arena.numel() < need + 256:
+            arena = torch.empty(need + 256, dtype=torch.uint8, device=device)
+            base = (arena.data_ptr() + 255) & ~255
+            # set_arena waits for the stream of the latest step before it lets go of the old memory,
+            # which torch frees when the last reference below goes
+            rc = self._lib.tw_engine_set_arena(self._h, base, arena.numel() - (base - arena.data_ptr()))
+            if rc != 0:
+                raise RuntimeError(f"set_arena failed ({rc})")
+            self._arena = arena
+        # a batch that fits the memory already held is carved anew inside it (and zeroed)
         rc = self._lib.tw_engine_alloc_batch(self._h, G, max_seq_len)
         if rc != 0:
             raise RuntimeError(f"alloc_batch failed ({rc})")
@@ -117,7 +121,16 @@ class Engine:
             raise ValueError(f"set_producers failed ({rc})")
         self._producers = (q_norm, k_norm, rope_cos, rope_sin)
 
+    def _check_rows(self, q, k, v, out, lead) -> None:
+        """The C side takes the row counts from the batch as allocated: the buffers must have exactly that shape."""
+        L, H, Hk, D = self._shape
+        want_q, want_kv = (*lead, self._G, H * D), (*lead, self._G, Hk * D)
+        for name, t, want in (("q", q, want_q), ("out", out, want_q), ("k", k, want_kv), ("v", v, want_kv)):
+            if tuple(t.shape) != want:
+                raise ValueError(f"{name}: shape {tuple(t.shape)}, the allocated batch needs {want}")
+
     def layer_step(self, layer, q, k, v, out, stream=None) -> None:
+        self._check_rows(q, k, v, out, ())
         rc = self._lib.tw_engine_layer_step(self._h, layer, _ptr(q, "f16", "q"), _ptr(k, "f16", "k"),
                                             _ptr(v, "f16", "v"), _ptr(out, "f16", "out"), _stream(stream))
         if rc != 0:
@@ -138,6 +151,7 @@ class Engine:
     def decode_step(self, q, k, v, out, use_graph: bool = False, stream=None) -> None:
         """Append + attention for every layer, then positions += 1.
         q/out: (L, G, H*D); k/v: (L, G, Hk*D)."""
+        self._check_rows(q, k, v, out, (self._shape[0],))
         rc = self._lib.tw_engine_decode_step(self._h, _ptr(q, "f16", "q"), _ptr(k, "f16", "k"),
                                              _ptr(v, "f16", "v"), _ptr(out, "f16", "out"),
                                              1 if use_graph else 0, _stream(stream))
