@@ -372,7 +372,7 @@ def main():
     ap.add_argument("--kv-bits", type=int, default=None, choices=[0, 2, 4])
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 vector-ALU kernel, 2 MFMA kernel")
     ap.add_argument("--nsplit", type=int, default=0)
-    ap.add_argument("--one-launch", type=int, default=None, choices=[0, 1, 2],
+    ap.add_argument("--one-launch", type=int, default=None, choices=[0, 1, 2, 3],
                     help="decode step of a compressed layer as one kernel: 0 by max_seq_len, 1 whenever possible, 2 never "
                          "(default: what the engine picks from the spread of the context lengths)")
     ap.add_argument("--no-graph", action="store_true")

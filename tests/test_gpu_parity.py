@@ -476,14 +476,16 @@ def test_decode_step_in_one_launch(kv, oracle, rotation_fixture, bits, H, Hk, le
     assert rel_err(host(out), want) <= TOL
 
 
+@pytest.mark.parametrize("mode", [1, 3])
 @pytest.mark.parametrize("bits", [4, 2])
 @pytest.mark.parametrize("G,H,Hk,producers", [(64, 16, 8, False), (128, 16, 8, True), (256, 16, 8, False), (264, 32, 8, True),
                                               (520, 8, 8, False), (130, 8, 2, True)])
-def test_decode_step_in_one_launch_every_head_grouping(kv, oracle, rotation_fixture, bits, G, H, Hk, producers):
+def test_decode_step_in_one_launch_every_head_grouping(kv, oracle, rotation_fixture, bits, G, H, Hk, producers, mode):
     """The one-launch step with 2, 4 and 8 KV heads per workgroup (batches of 64, 128 and 256 and more sequences on a
     256-CU GPU; 8 heads make units of more than 16 vectors, two rotation tiles), batch sizes that are and are not
     multiples of 8 (the workgroup numbering differs), with and without the producers: cache bytes and outputs
-    against the oracle."""
+    against the oracle.  Mode 1 takes the 4-bit kernel whose waves scan two KV heads each where the shape admits
+    it, mode 3 keeps one head per wave."""
     import torch
     r = gen.rng(950 + bits + G)
     msl = 96
@@ -499,7 +501,7 @@ def test_decode_step_in_one_launch_every_head_grouping(kv, oracle, rotation_fixt
     out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
     scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
     launches = kv._lib.load().tw_kv_decode_fused_launches()
-    kv.set_decode_fused(1)
+    kv.set_decode_fused(mode)
     try:
         if producers:
             kv.tw_qk_norm_rope_turbo_append_attention_batch(
@@ -521,6 +523,46 @@ def test_decode_step_in_one_launch_every_head_grouping(kv, oracle, rotation_fixt
     assert_bytes_equal(host(d_ck), ck, "K codes"); assert_bytes_equal(host(d_cv), cv, "V codes")
     assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
     assert rel_err(host(out), want) <= TOL
+
+
+@pytest.mark.parametrize("mode", [1, 3])
+@pytest.mark.parametrize("G,H,Hk,msl", [(64, 16, 8, 2048), (64, 8, 8, 1100), (64, 32, 8, 1100), (128, 16, 8, 700), (256, 16, 8, 400),
+                                        (128, 8, 4, 520)])
+def test_decode_step_two_heads_per_wave_long_contexts(kv, oracle, rotation_fixture, G, H, Hk, msl, mode):
+    """The 4-bit one-launch step at batch sizes where a workgroup owns 2, 4 or 8 KV heads (mode 1: its waves scan
+    two heads each, every load a whole cache line; mode 3: one head per wave), over contexts that hit every tile and
+    part edge up to max_seq_len - 1, query groups of 1, 2 and 4: appended rows bit for bit, outputs within tolerance."""
+    import torch
+    bits = 4
+    r = gen.rng(990 + G + H + Hk)
+    kv_dim, q_dim = Hk * D, H * D
+    edges = [0, 1, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 767, 1023,
+             1024, 1025, 1500, 2046, 2047]
+    lens = [e for e in edges if e < msl] + [msl - 1, msl - 2]
+    lens = (lens + [int(x) for x in r.integers(0, msl - 1, size=G)])[:G]
+    ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, G, Hk, msl, lens, bits)
+    pos = np.array(lens, np.int32)
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    d_ck, d_cv, d_kn, d_vn = dev(ck), dev(cv), dev(kn), dev(vn)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    launches = kv._lib.load().tw_kv_decode_fused_launches()
+    kv.set_decode_fused(mode)
+    try:
+        kv.tw_turbo_append_attention_batch(out, dev(q), dev(k), dev(v), d_ck, d_cv, d_kn, d_vn, dev(rotation_fixture),
+                                           scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    finally:
+        kv.set_decode_fused(0)
+    assert kv._lib.load().tw_kv_decode_fused_launches() == launches + 1
+    oracle.turbo_kv_quantize_batch(ck, kn, k, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    oracle.turbo_kv_quantize_batch(cv, vn, v, rotation_fixture, pos, msl, G, Hk, D, kv_dim, bits)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    assert_bytes_equal(host(d_ck), ck, "K codes"); assert_bytes_equal(host(d_cv), cv, "V codes")
+    assert_bytes_equal(host(d_kn), kn, "K norms"); assert_bytes_equal(host(d_vn), vn, "V norms")
+    got = host(out)
+    worst = [(rel_err(got[g], want[g]), g, lens[g]) for g in range(G)]
+    assert max(worst)[0] <= TOL, f"worst (error, sequence, context): {sorted(worst)[-3:]}"
 
 
 @pytest.mark.parametrize("bits", [4, 2])

@@ -140,8 +140,8 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
         }
         __amdgpu_buffer_rsrc_t rk = make_rsrc(reinterpret_cast<const char*>(a.k) + row * kRowBytes, rows * kRowBytes);
         __amdgpu_buffer_rsrc_t rv = make_rsrc(reinterpret_cast<const char*>(a.v) + row * kRowBytes, rows * kRowBytes);
-        uint32x4_t k4 = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)goff, 0, 0);
-        uint32x4_t v4 = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)goff, 0, 0);
+        uint32x4_t k4 = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)goff, 0, kStreamCodes);
+        uint32x4_t v4 = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)goff, 0, kStreamCodes);
         kr = uint4{k4[0], k4[1], k4[2], k4[3]};
         vr = uint4{v4[0], v4[1], v4[2], v4[3]};
         if (wv < 2 && lane < 32) {                           // wave 0: the 32 K-norm rows, wave 1: the V-norm rows
@@ -152,7 +152,7 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
                 nr = *reinterpret_cast<const uint4*>(nbase + prow * 16);
             } else {
                 __amdgpu_buffer_rsrc_t rn = make_rsrc(nbase + (seq_row0 + tile) * 16, max(min(n - tile, 32), 0) * 16);
-                uint32x4_t n4 = __builtin_amdgcn_raw_buffer_load_b128(rn, lane * 16, 0, 0);
+                uint32x4_t n4 = __builtin_amdgcn_raw_buffer_load_b128(rn, lane * 16, 0, kStreamCodes);
                 nr = uint4{n4[0], n4[1], n4[2], n4[3]};
             }
         }

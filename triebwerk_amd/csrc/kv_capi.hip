@@ -19,7 +19,7 @@ using namespace twkv;
 
 namespace twkv {
 static std::atomic<long long> g_fused_launches{0};   // one-launch decode steps issued so far (tw_kv_decode_fused_launches)
-static std::atomic<int> g_decode_fused{0};   // tw_kv_set_decode_fused: 0 by context bound, 1 whenever possible, 2 never
+static std::atomic<int> g_decode_fused{0};   // tw_kv_set_decode_fused: 0 by context bound, 1 whenever possible, 2 never, 3 as 1 with one head per wave
 static std::atomic<int> g_prefill_form{0};   // test hook, see prefill_form()
 int prefill_form() { return g_prefill_form.load(); }
 thread_local hipEvent_t t_scan_start = nullptr;
@@ -586,10 +586,10 @@ static bool try_decode_fused(const AttnArgs& a, const FusedArgs& f, int msl, hip
     const int mode = g_decode_fused.load();
     if (mode == 2 || g_variant.load() == 1) return false;
     if (!decode_fused_usable(a, f)) return false;
-    if (mode == 0 && !tw_kv_decode_step_plan(a.G, a.num_heads, a.num_kv_heads, a.bits, msl, t_ctx_min, t_ctx_max)) return false;
+    if (mode != 1 && mode != 3 && !tw_kv_decode_step_plan(a.G, a.num_heads, a.num_kv_heads, a.bits, msl, t_ctx_min, t_ctx_max)) return false;
     attach_profiler(s);
     g_fused_launches.fetch_add(1);
-    launch_decode_fused(a, f, s);
+    launch_decode_fused(a, f, s, /*allow_pairs=*/mode != 3);
     t_scan_start = t_scan_stop = nullptr;
     check_launch(fn);
     return true;

@@ -38,10 +38,10 @@ namespace twkv {
 namespace {
 
 constexpr int kFusedWaves = 16;
-#ifndef TW_FUSED_SHARE
-#define TW_FUSED_SHARE 33
-#endif
-constexpr unsigned kFusedShare = TW_FUSED_SHARE;  // 64ths of a sequence's tiles that go to the lower eight waves
+constexpr int kPairWaves = 8;                  // waves of a workgroup whose waves scan two KV heads each
+constexpr unsigned kFusedShare = 33;           // 64ths of a sequence's tiles that go to the lower eight waves
+constexpr int kTilesAhead = 1;                 // tiles of loads a wave of that kernel keeps in flight
+constexpr unsigned kPairTileShare = 32;        // the same with eight waves in all: two per SIMD, no upper slots
 constexpr int kFusedMaxQ = 32;                 // query heads of a unit: HKW * R <= 8 * 4
 constexpr int kRowFloats = kHeadDim + 4;       // LDS row of a vector: conflict-free 16-byte accesses
 constexpr int kStageStride = 2 * kHeadDim + 16;   // bytes per staged fp16 vector
@@ -49,15 +49,17 @@ static_assert(8 * (2 + 4) * kStageStride <= kFusedMaxQ * kRowFloats * 4, "staged
 
 }  // namespace
 
-template <int R, int BITS, bool PROD>
-__global__ void __launch_bounds__(kFusedWaves * kWave)
+template <int R, int BITS, bool PROD, bool PAIR>
+__global__ void __launch_bounds__((PAIR ? kPairWaves : kFusedWaves) * kWave)
 decode_fused_kernel(AttnArgs a, FusedArgs f) {
+    static_assert(!PAIR || BITS == 4, "two heads per wave: a 128-byte cache line is two 4-bit heads");
+    constexpr int NW = PAIR ? kPairWaves : kFusedWaves;        // waves of the workgroup
     constexpr int KW = BITS, VW = BITS;
     constexpr uint32_t kHeadBytes = BITS * 16;
     constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
     // the scan's probabilities and partials; before the scan the same space holds R as 8 operand tiles
-    constexpr int kPBytes = kFusedWaves * 16 * 32 * 2, kPartBytes = kFusedWaves * R * kRowFloats * 4;
+    constexpr int kPBytes = NW * 16 * 32 * 2, kPartBytes = kFusedWaves * R * kRowFloats * 4;   // 16 (part, head) partials either way
     constexpr int kRotBytes = 8 * kOperandTileDwords * 4;
     __shared__ __attribute__((aligned(16))) char scan_s[kPBytes + kPartBytes > kRotBytes ? kPBytes + kPartBytes : kRotBytes];
     half_t (*p_s)[16][32] = reinterpret_cast<half_t (*)[16][32]>(scan_s);
@@ -73,7 +75,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const int Hk = a.num_kv_heads;
     const int HKW = f.hkw;
     const int nhg = Hk / HKW;
-    const int SPLIT = kFusedWaves / HKW;
+    const int SPLIT = kFusedWaves / HKW;               // parts of the context per head (PAIR: 8 waves, 2 heads each)
 
     // ---- unit of this workgroup.  Workgroups are dealt to the 8 XCDs in turn; the units of one sequence
     // go to one XCD so that the norm rows they all read (16 bytes per token for 8 heads) come out of one L2.
@@ -126,8 +128,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
 
     const int pos = uniform(a.positions[g]);
     const int n = pos + 1;
-    const int hk_local = wave % HKW, part = wave / HKW;
-    const int h = hg * HKW + hk_local;                 // KV head of this wave
+    // PAIR: wave = part * (HKW / 2) + pair; hk_local is the first head of the pair
+    const int hk_local = PAIR ? 2 * (wave % (HKW >> 1)) : wave % HKW, part = PAIR ? wave / (HKW >> 1) : wave / HKW;
+    const int h = hg * HKW + hk_local;                 // (first) KV head of this wave
 
     // producers' operands: the two weight vectors and the table rows of this sequence's position, 16 bytes per thread
     const bool normed = PROD && f.q_weight != nullptr, roped = PROD && f.cos_table != nullptr;
@@ -152,7 +155,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     // the tiles); what is left goes round the lower waves' parts.
     const int ntile = (n + 31) >> 5;
     const int halfparts = SPLIT >> 1;                      // SPLIT is 2, 4, 8 or 16
-    const int lower = min(ntile, (int)((ntile * kFusedShare + 63u) / 64u));
+    const int lower = min(ntile, (int)((ntile * (PAIR ? kPairTileShare : kFusedShare) + 63u) / 64u));
     const int rounds = (ntile - lower) / halfparts;
     const int tail0 = rounds * SPLIT;                      // tail tiles tail0 + part + j * halfparts, lower parts only
     const int left = ntile - tail0 - part;
@@ -271,7 +274,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         // the centroid table while the loads are under way: entry e fills 256 bytes with replicas.  The centroids
         // come out of a register by wave shuffle (lane c holds centroid c): indexing the constant array with a
         // per-lane index is a dependent memory load per look-up, several microseconds for this loop.
-        for (int i = tid * 4; i < kTableWords; i += kFusedWaves * kWave * 4) {
+        for (int i = tid * 4; i < kTableWords; i += NW * kWave * 4) {
             const int e = i >> 6;
             if constexpr (BITS == 4) {
                 half2_t p = {(half_t)__shfl(cent_lane, e & 15, 64), (half_t)__shfl(cent_lane, e >> 4, 64)};
@@ -298,7 +301,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             // optional producers on the staged K and query vectors, one vector per wave: per-head RMSNorm
             // (kernels.cu:880-923), then rotary embedding (927-961), each rounded to fp16 as the reference's
             // in-place kernels leave it; V vectors stay as they are
-            for (int v = wave; v < nvec; v += kFusedWaves) {
+            for (int v = wave; v < nvec; v += NW) {
                 int kind, head;
                 (void)unit_vector(v, kind, head);
                 if (kind == 1) continue;                           // uniform over the wave
@@ -319,7 +322,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             lds_barrier();
         }
 
-        for (int vt = wave >> 3; vt * 16 < nvec; vt += 2) {       // uniform over the wave
+        for (int vt = wave >> 3; vt * 16 < nvec; vt += NW / 8) {  // uniform over the wave
             const int vi = vt * 16 + i16;
             const int vc = vi < nvec ? vi : nvec - 1;              // clamp reads, mask stores
             int kind, head;
@@ -368,181 +371,6 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     __syncthreads();        // table, q_rot and the new cache row are in place; R has been read
     // the wave's slice of the probabilities starts at zero (no other wave touches it)
     *reinterpret_cast<uint4*>(&p_s[wave][0][0] + 8 * lane) = uint4{0u, 0u, 0u, 0u};
-    {
-        int l2 = lane;
-        asm volatile("" : "+v"(l2));
-        derive_lane(l2);
-    }
-
-    // ---- 2. scan of this wave's part
-    float4_t o[8];
-#pragma unroll
-    for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float m_run[R], l_run[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
-
-    if (ntiles > 0) {
-        issue_k(kreg, first_tile);
-        nreg = issue_n(first_tile);
-        issue_v(vreg, first_tile);
-        // A operand of the score MFMAs: q_rot[head][32kg + 8j + i], row m = fp16 value of head m, row m + 8
-        // its rounding remainder; the 2-bit table returns the codes of a byte in the order 0,2,1,3
-        half8_t aq[4];
-        {
-            const int hq = ln & 7;
-            const bool lo_part = (ln & 8) != 0;
-            const float* qr = &qrot_s[hk_local * R + (hq < R ? hq : 0)][32 * kg];
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
-                float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
-                float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const int src = BITS == 4 ? i : ((i & 4) | ((i & 1) << 1) | ((i & 2) >> 1));
-                    float x = (hq < R) ? v[src] : 0.0f;
-                    half_t hi = (half_t)x;
-                    half_t lo = (half_t)(x - (float)hi);
-                    aq[j][i] = lo_part ? lo : hi;
-                }
-            }
-        }
-
-        for (int it = 0; it < ntiles; it++) {
-            const int tile = tile_at(it);
-            const int next_tile = tile_at(it + 1);
-            const bool more = it + 1 < ntiles;
-
-            // ---- scores S[head][token] for both sub-tiles
-            float4_t s[2];
-#pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
-                uint32_t kw[KW];
-#pragma unroll
-                for (int i = 0; i < KW; i++) kw[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(ksrc, (int)kreg[sub][i]);
-                union { uint32_t u[4]; half8_t h; } kv[4];
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    if constexpr (BITS == 4) {
-                        const uint32_t w = kw[j];
-                        kv[j].u[0] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0400u));
-                        kv[j].u[1] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0500u));
-                        kv[j].u[2] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0600u));
-                        kv[j].u[3] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0700u));
-                    } else {
-                        const uint32_t w = kw[j >> 1];
-                        const uint32_t sel = (j & 1) ? 0x0c0c0600u : 0x0c0c0400u;
-                        uint2 l0 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel));
-                        uint2 l1 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel + 0x100u));
-                        kv[j].u[0] = l0.x; kv[j].u[1] = l0.y; kv[j].u[2] = l1.x; kv[j].u[3] = l1.y;
-                    }
-                }
-                s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[sub], 0, 0, 0);
-            }
-            if (more) issue_k(kreg, next_tile);
-
-            // ---- online softmax (base 2): this lane owns token ln of sub-tile my_sub
-            const float kn = h2f_bits(nreg & 0xffffu), vn = h2f_bits(nreg >> 16);
-            if (more) nreg = issue_n(next_tile);
-            const bool valid = useful && (tile + 16 * my_sub + ln < n);
-            float raw[R], x[R];
-            bool raise = false;
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                uint32x2_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(s[0][r]), __float_as_uint(s[1][r]), false, false);
-                raw[r] = (__uint_as_float(sw[0]) + __uint_as_float(sw[1])) * kn;    // kernels.cu:1707
-                x[r] = valid ? raw[r] - m_run[r] : kNegBig;
-                raise = raise || (x[r] > kRaise);
-            }
-            if (__any(raise)) {
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    float m_new = fmaxf(m_run[r], wave_max(valid ? raw[r] : kNegBig));
-                    float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_new);
-                    m_run[r] = m_new;
-                    l_run[r] *= alpha;
-                    x[r] = valid ? raw[r] - m_new : kNegBig;
-#pragma unroll
-                    for (int j = 0; j < 8; j++) o[j][r] *= alpha;
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                float p = __builtin_amdgcn_exp2f(x[r]);
-                l_run[r] += p;
-                float pf = p * vn;                                      // (s * vn) * centroid, kernels.cu:1765
-                half_t hi = (half_t)pf;
-                half_t lo = (half_t)(pf - (float)hi);
-                if (useful) {
-                    p_w[r * 32] = hi;
-                    p_w[(r + 8) * 32] = lo;
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            union { uint4 q; half8_t h; } pa;
-            pa.q = *p_r;
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-
-            // ---- O[head][dim 8ln + j] += P[head][token] V[token][dim]
-            if constexpr (BITS == 4) {
-                uint32_t xe[4], xo[4];
-#pragma unroll
-                for (int sub = 0; sub < 2; sub++) {
-#pragma unroll
-                    for (int pr = 0; pr < 2; pr++) {
-                        uint32_t wa = vreg[sub][2 * pr], wb = vreg[sub][2 * pr + 1];
-                        xe[2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
-                        xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
-                    }
-                }
-                if (more) issue_v(vreg, next_tile);
-#pragma unroll
-                for (int jp = 0; jp < 4; jp++) {
-                    const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
-                    union { uint32_t u[4]; half8_t h; } be, bo;
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        be.u[q4] = lut32(__builtin_amdgcn_perm(xe[q4], lane_rep, sel));
-                        bo.u[q4] = lut32(__builtin_amdgcn_perm(xo[q4], lane_rep, sel));
-                    }
-                    o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * jp], 0, 0, 0);
-                    o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * jp + 1], 0, 0, 0);
-                }
-            } else {
-                uint32_t ie[2], io[2];
-#pragma unroll
-                for (int sub = 0; sub < 2; sub++) {
-                    const uint32_t keep = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_keep);
-                    const uint32_t send = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_send);
-                    const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xf, 0xf, false);  // lane ^ 1
-                    const uint32_t wa = odd ? recv : keep, wb = odd ? keep : recv;
-                    ie[sub] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
-                    io[sub] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
-                }
-                if (more) issue_v(vreg, next_tile);
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const uint32_t x0 = (q & 1) ? io[0] : ie[0], x1 = (q & 1) ? io[1] : ie[1];
-                    const uint32_t sel = 0x0c0c0400u + ((uint32_t)(q >> 1) << 8);
-                    uint2 l00 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel));
-                    uint2 l01 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel + 0x200u));
-                    uint2 l10 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel));
-                    uint2 l11 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel + 0x200u));
-                    union { uint32_t u[4]; half8_t h; } be, bo;
-                    be.u[0] = l00.x; be.u[1] = l01.x; be.u[2] = l10.x; be.u[3] = l11.x;
-                    bo.u[0] = l00.y; bo.u[1] = l01.y; bo.u[2] = l10.y; bo.u[3] = l11.y;
-                    o[2 * q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * q], 0, 0, 0);
-                    o[2 * q + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * q + 1], 0, 0, 0);
-                }
-            }
-        }
-    }
-
     // ---- 3. the parts meet in LDS.  B operand of the rotate-back first (its loads run under the merge, and stay
     // hidden there: R brought in coalesced and passed through LDS instead was 0.25 us slower per launch):
     // R[32kk + s][16*dblk + i16], s = 0..31
@@ -550,26 +378,477 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const int dblk = wave & 7;
     const bool back = (wave >> 3) * 16 < nv;
     uint16_t rb[32];
+    auto load_rb = [&]() {
     if (back) {
         const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.rotation) + (32 * kg) * kHeadDim + 16 * dblk + ln;
 #pragma unroll
         for (int s = 0; s < 32; s++) rb[s] = rp[s * kHeadDim];
     }
+    };
+    if constexpr (PAIR) {
+        // ---- 2 (PAIR). scan of this wave's part, two KV heads per wave.  A 128-byte line of a cache row is two
+        // 4-bit heads: with a head per wave two waves fetch every line, each for its half.  Here a wave takes both
+        // halves, so every load instruction covers whole lines that no other instruction touches, and the loads
+        // carry the non-temporal hint (see kStreamCodes): the same bytes arrive ~11 % faster.  The two heads share
+        // the MFMAs: score columns 0-7 are 8 tokens of the first head, columns 8-15 the same tokens of the second;
+        // P.V columns 0-7 are dims of the first head, 8-15 of the second; the A operands carry the query heads
+        // (probabilities) of both KV heads in rows hd * R + r (+ 8: rounding remainders).  A product of a row with
+        // a column of the other head is computed and never used.
+        int l2 = lane;
+        asm volatile("" : "+v"(l2));
+        const int pn = l2 & 15, pkg = l2 >> 4;
+        const int hd = pn >> 3;                                   // head of the pair this lane's columns belong to
+        const int pw = hk_local >> 1;
+        const uint32_t lane_rep = (uint32_t)l2 * 4u;
+        const uint32_t kvp = (uint32_t)Hk * kHeadBytes;
+        const uint32_t nrow = (uint32_t)Hk * 2u;
+        // K: instruction c of a tile covers tokens 8c .. 8c+7, lane l the 16-byte piece l % 8 of token l / 8
+        const uint32_t koff = (uint32_t)(l2 >> 3) * kvp + 16u * (uint32_t)(l2 & 7);
+        // operand order: lane (pn, pkg) takes token pn % 8, head pn / 8, dims 32 pkg .. +31 = piece 4 hd + pkg
+        const int ksrc = 4 * (8 * (pn & 7) + 4 * hd + pkg);
+        // V: lane (pn, pkg) loads 8 bytes (16 dims: head pn / 8, dims 16 (pn % 8) ..) of tokens 4 pkg + i (+ 16)
+        const uint32_t voff = (uint32_t)(4 * pkg) * kvp + 8u * (uint32_t)pn;
+        // softmax: a lane owns the scores of tokens tok0 and tok0 + 16 of its head
+        const bool useful = R == 4 ? ((pkg & 1) == hd) : ((pkg & 1) == 0);
+        const int tok0 = 8 * (pkg >> 1) + (pn & 7);
+        const uint32_t noff = (uint32_t)tok0 * nrow;
+        half_t* p_w = &p_s[wave][hd * R][8 * (tok0 >> 2) + (tok0 & 3)];     // row + r (+ 8), token tok0 + 16: + 4
+        const uint4* p_r = reinterpret_cast<const uint4*>(&p_s[wave][pn][8 * pkg]);
+        constexpr float kRaise = 5.0f;
+        const char* tab_lane = reinterpret_cast<const char*>(tab_s);
+        auto lut32 = [&](uint32_t addr) -> uint32_t { return *reinterpret_cast<const uint32_t*>(tab_lane + addr); };
+
+        const long long seq_row0 = (long long)g * a.seq_stride_rows;
+        const char* kpair = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes;
+        const char* vpair = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes;
+        const char* knpair = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
+        const char* vnpair = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
+        // (loads of a tile index past the wave's last one are given an empty extent: they return zeros without touching memory)
+        auto tile_rows = [&](int i, int tile) -> int { return i < ntiles ? max(min(n - tile, 32), 0) : 0; };
+        auto issue_k = [&](uint32x4_t (&kr)[4], int i) {
+            const int tile = tile_at(i);
+            __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (seq_row0 + tile) * kvp, tile_rows(i, tile) * (int)kvp);
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        l_run[r] = wave_sum(l_run[r]);
+            for (int c = 0; c < 4; c++) kr[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kStreamCodes);
+        };
+        auto issue_v = [&](uint32x2_t (&vr)[2][4], int i) {
+            const int tile = tile_at(i);
+            __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (seq_row0 + tile) * kvp, tile_rows(i, tile) * (int)kvp);
 #pragma unroll
-        for (int j = 0; j < 8; j++) o[j][r] += __shfl_xor(o[j][r], 32, 64);   // row r + row r+8 (lo part of P)
-    }
-    if (kg == 0) {
+            for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    vr[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kStreamCodes);
+            }
+        };
+        // norms of the pair (two fp16) for the lane's two tokens: [token][K | V]
+        auto issue_n = [&](uint32_t (&nr)[2][2], int i) {
+            const int tile = tile_at(i);
+            const int rows = tile_rows(i, tile);
+            __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
+            __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
+            if (useful) {
+                nr[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
+                nr[1][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)(noff + 16u * nrow), 0, kStreamNorms);
+                nr[0][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
+                nr[1][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)(noff + 16u * nrow), 0, kStreamNorms);
+            }
+        };
+        auto head_max = [&](float v) -> float {                   // over the lanes of this lane's head
+            v = fmaxf(v, __shfl_xor(v, 1, 64)); v = fmaxf(v, __shfl_xor(v, 2, 64)); v = fmaxf(v, __shfl_xor(v, 4, 64));
+            v = fmaxf(v, __shfl_xor(v, 16, 64)); v = fmaxf(v, __shfl_xor(v, 32, 64));
+            return v;
+        };
+        auto head_sum = [&](float v) -> float {
+            v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64);
+            v += __shfl_xor(v, 16, 64); v += __shfl_xor(v, 32, 64);
+            return v;
+        };
+
+        float4_t o[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        float m_run[R], l_run[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
+
+        if (ntiles > 0) {
+            // kTilesAhead register sets, used in turn (two tiles in flight measured 2 % slower than one: the wave is
+            // not waiting for memory)
+            uint32x4_t kreg[kTilesAhead][4];
+            uint32x2_t vreg[kTilesAhead][2][4];
+            uint32_t nreg[kTilesAhead][2][2] = {};
+#pragma unroll
+            for (int d = 0; d < kTilesAhead; d++) {
+                issue_k(kreg[d], d);
+                issue_n(nreg[d], d);
+                issue_v(vreg[d], d);
+            }
+            // A operand of the score MFMAs: row m < 8: query head m % R of KV head m / R of the pair (fp16 value),
+            // row m + 8 its rounding remainder; q_rot[..][32 pkg + 8 j + i]
+            half8_t aq[4];
+            {
+                const int m = pn & 7;
+                const bool lo_part = (pn & 8) != 0;
+                const bool live = m < 2 * R;
+                const float* qr = &qrot_s[(hk_local + (live ? m / R : 0)) * R + (live ? m % R : 0)][32 * pkg];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
+                    float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
+                    float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        float x = live ? v[i] : 0.0f;
+                        half_t hi = (half_t)x;
+                        half_t lo = (half_t)(x - (float)hi);
+                        aq[j][i] = lo_part ? lo : hi;
+                    }
+                }
+            }
+
+            auto scan_tile = [&](int it, uint32x4_t (&kreg)[4], uint32x2_t (&vreg)[2][4], uint32_t (&nreg)[2][2]) {
+                const int tile = tile_at(it);
+                const int ahead = it + kTilesAhead;              // the tile this register set is asked for next
+
+                // ---- scores: set c = tokens 8c .. 8c+7 of both heads
+                float4_t s[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    union { uint32_t u[4]; half8_t h; } kv[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint32_t w = (uint32_t)__builtin_amdgcn_ds_bpermute(ksrc, (int)kreg[c][j]);
+                        kv[j].u[0] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0400u));
+                        kv[j].u[1] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0500u));
+                        kv[j].u[2] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0600u));
+                        kv[j].u[3] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0700u));
+                    }
+                    s[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) s[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[c], 0, 0, 0);
+                }
+                issue_k(kreg, ahead);
+
+                // ---- online softmax (base 2): this lane owns tokens tok0 and tok0 + 16 of head hd
+                float kn[2], vn[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    kn[t] = h2f_bits(hd ? (nreg[t][0] >> 16) : (nreg[t][0] & 0xffffu));
+                    vn[t] = h2f_bits(hd ? (nreg[t][1] >> 16) : (nreg[t][1] & 0xffffu));
+                }
+                issue_n(nreg, ahead);
+                const bool valid[2] = {useful && (tile + tok0 < n), useful && (tile + tok0 + 16 < n)};
+                float raw[2][R], x[2][R];
+                bool raise = false;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    // the row of (hd, r): hd * R + r; rows 0-3 sit in lane group 0 (R = 4: the second head's in group 1),
+                    // their remainders 32 lanes further on
+                    float v[4];
+#pragma unroll
+                    for (int c = 0; c < 4; c++) v[c] = R == 4 ? s[c][r] : (hd ? s[c][R + r] : s[c][r]);
+                    uint32x2_t s01 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[1]), false, false);
+                    uint32x2_t s23 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[2]), __float_as_uint(v[3]), false, false);
+                    raw[0][r] = (__uint_as_float(s01[0]) + __uint_as_float(s01[1])) * kn[0];    // kernels.cu:1707
+                    raw[1][r] = (__uint_as_float(s23[0]) + __uint_as_float(s23[1])) * kn[1];
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        x[t][r] = valid[t] ? raw[t][r] - m_run[r] : kNegBig;
+                        raise = raise || (x[t][r] > kRaise);
+                    }
+                }
+                if (__any(raise)) {
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const float mine = fmaxf(valid[0] ? raw[0][r] : kNegBig, valid[1] ? raw[1][r] : kNegBig);
+                        const float m_new = fmaxf(m_run[r], head_max(mine));
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                        m_run[r] = m_new;
+                        l_run[r] *= alpha;
+#pragma unroll
+                        for (int t = 0; t < 2; t++) x[t][r] = valid[t] ? raw[t][r] - m_new : kNegBig;
+                        // accumulator register i of a lane is row 4 pkg + i: query head i % R (of either KV head)
+#pragma unroll
+                        for (int j = 0; j < 16; j++) {
+#pragma unroll
+                            for (int i = r; i < 4; i += R) o[j][i] *= alpha;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const float pe = __builtin_amdgcn_exp2f(x[t][r]);
+                        l_run[r] += pe;
+                        const float pf = pe * vn[t];                            // (s * vn) * centroid, kernels.cu:1765
+                        const half_t hi = (half_t)pf;
+                        const half_t lo = (half_t)(pf - (float)hi);
+                        if (useful) {
+                            p_w[r * 32 + 4 * t] = hi;
+                            p_w[(r + 8) * 32 + 4 * t] = lo;
+                        }
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                union { uint4 q; half8_t h; } pa;
+                pa.q = *p_r;
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+
+                // ---- O[row][dim 16 (pn % 8) + j of head pn / 8] += P[row][token] V[token][dim]
+                uint32_t xe[2][4], xo[2][4];
+#pragma unroll
+                for (int dw = 0; dw < 2; dw++) {
+#pragma unroll
+                    for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                        for (int pr = 0; pr < 2; pr++) {
+                            const uint32_t wa = vreg[sub][2 * pr][dw], wb = vreg[sub][2 * pr + 1][dw];
+                            xe[dw][2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                            xo[dw][2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                        }
+                    }
+                }
+                issue_v(vreg, ahead);
+#pragma unroll
+                for (int dw = 0; dw < 2; dw++) {
+#pragma unroll
+                    for (int jp = 0; jp < 4; jp++) {
+                        const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
+                        union { uint32_t u[4]; half8_t h; } be, bo;
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; q4++) {
+                            be.u[q4] = lut32(__builtin_amdgcn_perm(xe[dw][q4], lane_rep, sel));
+                            bo.u[q4] = lut32(__builtin_amdgcn_perm(xo[dw][q4], lane_rep, sel));
+                        }
+                        o[8 * dw + 2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[8 * dw + 2 * jp], 0, 0, 0);
+                        o[8 * dw + 2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[8 * dw + 2 * jp + 1], 0, 0, 0);
+                    }
+                }
+            };
+            for (int it = 0; it < ntiles; it += kTilesAhead) {
+#pragma unroll
+                for (int d = 0; d < kTilesAhead; d++) {
+                    if (it + d < ntiles) scan_tile(it + d, kreg[d], vreg[d], nreg[d]);
+                }
+            }
+        }
+        load_rb();
+        // the wave's partials: rows hd * R + r of the columns of head hd, value + remainder rows added
+        const int khi = R == 4 ? hd : 0;                          // lane group that holds the rows of head hd
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            float* pr = &part_s[wave][r][0];
-            float4 lo4 = {o[0][r] * (1.0f / kAlpha), o[1][r] * (1.0f / kAlpha), o[2][r] * (1.0f / kAlpha), o[3][r] * (1.0f / kAlpha)};
-            float4 hi4 = {o[4][r] * (1.0f / kAlpha), o[5][r] * (1.0f / kAlpha), o[6][r] * (1.0f / kAlpha), o[7][r] * (1.0f / kAlpha)};
-            *reinterpret_cast<float4*>(pr + 8 * ln) = lo4;
-            *reinterpret_cast<float4*>(pr + 8 * ln + 4) = hi4;
-            if (ln == 0) { pr[kHeadDim] = m_run[r]; pr[kHeadDim + 1] = l_run[r]; }
+            l_run[r] = head_sum(l_run[r]);
+            float ov[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                float v = R == 4 ? o[j][r] : (hd ? o[j][R + r] : o[j][r]);
+                ov[j] = (v + __shfl_xor(v, 32, 64)) * (1.0f / kAlpha);
+            }
+            if (pkg == khi) {
+                float* pr = &part_s[part * HKW + hk_local + hd][r][0];
+#pragma unroll
+                for (int j4 = 0; j4 < 4; j4++)
+                    *reinterpret_cast<float4*>(pr + 16 * (pn & 7) + 4 * j4) = float4{ov[4 * j4], ov[4 * j4 + 1], ov[4 * j4 + 2], ov[4 * j4 + 3]};
+                if ((pn & 7) == 0) { pr[kHeadDim] = m_run[r]; pr[kHeadDim + 1] = l_run[r]; }
+            }
+        }
+    } else {
+        {
+            int l2 = lane;
+            asm volatile("" : "+v"(l2));
+            derive_lane(l2);
+        }
+
+        // ---- 2. scan of this wave's part
+        float4_t o[8];
+    #pragma unroll
+        for (int j = 0; j < 8; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        float m_run[R], l_run[R];
+    #pragma unroll
+        for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
+
+        if (ntiles > 0) {
+            issue_k(kreg, first_tile);
+            nreg = issue_n(first_tile);
+            issue_v(vreg, first_tile);
+            // A operand of the score MFMAs: q_rot[head][32kg + 8j + i], row m = fp16 value of head m, row m + 8
+            // its rounding remainder; the 2-bit table returns the codes of a byte in the order 0,2,1,3
+            half8_t aq[4];
+            {
+                const int hq = ln & 7;
+                const bool lo_part = (ln & 8) != 0;
+                const float* qr = &qrot_s[hk_local * R + (hq < R ? hq : 0)][32 * kg];
+    #pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
+                    float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
+                    float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+    #pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const int src = BITS == 4 ? i : ((i & 4) | ((i & 1) << 1) | ((i & 2) >> 1));
+                        float x = (hq < R) ? v[src] : 0.0f;
+                        half_t hi = (half_t)x;
+                        half_t lo = (half_t)(x - (float)hi);
+                        aq[j][i] = lo_part ? lo : hi;
+                    }
+                }
+            }
+
+            for (int it = 0; it < ntiles; it++) {
+                const int tile = tile_at(it);
+                const int next_tile = tile_at(it + 1);
+                const bool more = it + 1 < ntiles;
+
+                // ---- scores S[head][token] for both sub-tiles
+                float4_t s[2];
+    #pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+                    uint32_t kw[KW];
+    #pragma unroll
+                    for (int i = 0; i < KW; i++) kw[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(ksrc, (int)kreg[sub][i]);
+                    union { uint32_t u[4]; half8_t h; } kv[4];
+    #pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if constexpr (BITS == 4) {
+                            const uint32_t w = kw[j];
+                            kv[j].u[0] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0400u));
+                            kv[j].u[1] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0500u));
+                            kv[j].u[2] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0600u));
+                            kv[j].u[3] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0700u));
+                        } else {
+                            const uint32_t w = kw[j >> 1];
+                            const uint32_t sel = (j & 1) ? 0x0c0c0600u : 0x0c0c0400u;
+                            uint2 l0 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel));
+                            uint2 l1 = lut64(__builtin_amdgcn_perm(w, lane_rep, sel + 0x100u));
+                            kv[j].u[0] = l0.x; kv[j].u[1] = l0.y; kv[j].u[2] = l1.x; kv[j].u[3] = l1.y;
+                        }
+                    }
+                    s[sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+                    for (int j = 0; j < 4; j++) s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[sub], 0, 0, 0);
+                }
+                if (more) issue_k(kreg, next_tile);
+
+                // ---- online softmax (base 2): this lane owns token ln of sub-tile my_sub
+                const float kn = h2f_bits(nreg & 0xffffu), vn = h2f_bits(nreg >> 16);
+                if (more) nreg = issue_n(next_tile);
+                const bool valid = useful && (tile + 16 * my_sub + ln < n);
+                float raw[R], x[R];
+                bool raise = false;
+    #pragma unroll
+                for (int r = 0; r < R; r++) {
+                    uint32x2_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(s[0][r]), __float_as_uint(s[1][r]), false, false);
+                    raw[r] = (__uint_as_float(sw[0]) + __uint_as_float(sw[1])) * kn;    // kernels.cu:1707
+                    x[r] = valid ? raw[r] - m_run[r] : kNegBig;
+                    raise = raise || (x[r] > kRaise);
+                }
+                if (__any(raise)) {
+    #pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        float m_new = fmaxf(m_run[r], wave_max(valid ? raw[r] : kNegBig));
+                        float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                        m_run[r] = m_new;
+                        l_run[r] *= alpha;
+                        x[r] = valid ? raw[r] - m_new : kNegBig;
+    #pragma unroll
+                        for (int j = 0; j < 8; j++) o[j][r] *= alpha;
+                    }
+                }
+    #pragma unroll
+                for (int r = 0; r < R; r++) {
+                    float p = __builtin_amdgcn_exp2f(x[r]);
+                    l_run[r] += p;
+                    float pf = p * vn;                                      // (s * vn) * centroid, kernels.cu:1765
+                    half_t hi = (half_t)pf;
+                    half_t lo = (half_t)(pf - (float)hi);
+                    if (useful) {
+                        p_w[r * 32] = hi;
+                        p_w[(r + 8) * 32] = lo;
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                union { uint4 q; half8_t h; } pa;
+                pa.q = *p_r;
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+
+                // ---- O[head][dim 8ln + j] += P[head][token] V[token][dim]
+                if constexpr (BITS == 4) {
+                    uint32_t xe[4], xo[4];
+    #pragma unroll
+                    for (int sub = 0; sub < 2; sub++) {
+    #pragma unroll
+                        for (int pr = 0; pr < 2; pr++) {
+                            uint32_t wa = vreg[sub][2 * pr], wb = vreg[sub][2 * pr + 1];
+                            xe[2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                            xo[2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                        }
+                    }
+                    if (more) issue_v(vreg, next_tile);
+    #pragma unroll
+                    for (int jp = 0; jp < 4; jp++) {
+                        const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
+                        union { uint32_t u[4]; half8_t h; } be, bo;
+    #pragma unroll
+                        for (int q4 = 0; q4 < 4; q4++) {
+                            be.u[q4] = lut32(__builtin_amdgcn_perm(xe[q4], lane_rep, sel));
+                            bo.u[q4] = lut32(__builtin_amdgcn_perm(xo[q4], lane_rep, sel));
+                        }
+                        o[2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * jp], 0, 0, 0);
+                        o[2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * jp + 1], 0, 0, 0);
+                    }
+                } else {
+                    uint32_t ie[2], io[2];
+    #pragma unroll
+                    for (int sub = 0; sub < 2; sub++) {
+                        const uint32_t keep = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_keep);
+                        const uint32_t send = __builtin_amdgcn_perm(vreg[sub][1], vreg[sub][0], sel_send);
+                        const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xf, 0xf, false);  // lane ^ 1
+                        const uint32_t wa = odd ? recv : keep, wb = odd ? keep : recv;
+                        ie[sub] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                        io[sub] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+                    }
+                    if (more) issue_v(vreg, next_tile);
+    #pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const uint32_t x0 = (q & 1) ? io[0] : ie[0], x1 = (q & 1) ? io[1] : ie[1];
+                        const uint32_t sel = 0x0c0c0400u + ((uint32_t)(q >> 1) << 8);
+                        uint2 l00 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel));
+                        uint2 l01 = lut64(__builtin_amdgcn_perm(x0, lane_rep, sel + 0x200u));
+                        uint2 l10 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel));
+                        uint2 l11 = lut64(__builtin_amdgcn_perm(x1, lane_rep, sel + 0x200u));
+                        union { uint32_t u[4]; half8_t h; } be, bo;
+                        be.u[0] = l00.x; be.u[1] = l01.x; be.u[2] = l10.x; be.u[3] = l11.x;
+                        bo.u[0] = l00.y; bo.u[1] = l01.y; bo.u[2] = l10.y; bo.u[3] = l11.y;
+                        o[2 * q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * q], 0, 0, 0);
+                        o[2 * q + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * q + 1], 0, 0, 0);
+                    }
+                }
+            }
+        }
+
+    load_rb();
+    #pragma unroll
+        for (int r = 0; r < R; r++) {
+            l_run[r] = wave_sum(l_run[r]);
+    #pragma unroll
+            for (int j = 0; j < 8; j++) o[j][r] += __shfl_xor(o[j][r], 32, 64);   // row r + row r+8 (lo part of P)
+        }
+        if (kg == 0) {
+    #pragma unroll
+            for (int r = 0; r < R; r++) {
+                float* pr = &part_s[wave][r][0];
+                float4 lo4 = {o[0][r] * (1.0f / kAlpha), o[1][r] * (1.0f / kAlpha), o[2][r] * (1.0f / kAlpha), o[3][r] * (1.0f / kAlpha)};
+                float4 hi4 = {o[4][r] * (1.0f / kAlpha), o[5][r] * (1.0f / kAlpha), o[6][r] * (1.0f / kAlpha), o[7][r] * (1.0f / kAlpha)};
+                *reinterpret_cast<float4*>(pr + 8 * ln) = lo4;
+                *reinterpret_cast<float4*>(pr + 8 * ln + 4) = hi4;
+                if (ln == 0) { pr[kHeadDim] = m_run[r]; pr[kHeadDim + 1] = l_run[r]; }
+            }
         }
     }
     lds_barrier();                 // the loads of R above stay in flight
@@ -601,7 +880,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     lds_barrier();
 
     // ---- out[vector][d] = sum_k o[vector][k] R[k][d]; lane group kk owns k in [32kk, 32kk+32)
-    for (int vt = wave >> 3; vt * 16 < nv; vt += 2) {
+    for (int vt = wave >> 3; vt * 16 < nv; vt += NW / 8) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
         const float* orow = &o_s[vt * 16 + ln][32 * kg];
 #pragma unroll
@@ -657,18 +936,28 @@ bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
     return true;
 }
 
-void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s) {
+// Two KV heads per wave (PAIR) when the cache is 4 bit and the workgroup's heads come in pairs: eight waves, every
+// cache line fetched by one instruction.  The workgroup then has 512 threads: its HKW * (2 + R) vectors must fit
+// the 32 staging slots and its HKW * R outputs the 16 merge slots.
+bool decode_fused_pairs(const AttnArgs& a, int hkw) {
+    const int R = a.num_heads / a.num_kv_heads;
+    return a.bits == 4 && (hkw & 1) == 0 && hkw * (2 + R) <= 32 && hkw * R <= 16;
+}
+
+void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s, bool allow_pairs) {
     FusedArgs f = f_in;
     f.hkw = decode_fused_heads_per_workgroup(a.G, a.num_kv_heads);
     f.q_scale = attention_mfma_q_scale(a.bits);
     const int R = a.num_heads / a.num_kv_heads;
-    const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw))), b3(kFusedWaves * kWave);
+    const bool pair = allow_pairs && decode_fused_pairs(a, f.hkw);
+    const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw))), b3((pair ? kPairWaves : kFusedWaves) * kWave);
     const bool prod = f.q_weight != nullptr || f.cos_table != nullptr;
-#define TW_FUSED(RR, BB) \
-    do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true>, g3, b3, s, a, f); \
-         else launch_scan_kernel(decode_fused_kernel<RR, BB, false>, g3, b3, s, a, f); } while (0)
-#define TW_FUSED_R(BB) do { if (R == 1) TW_FUSED(1, BB); else if (R == 2) TW_FUSED(2, BB); else TW_FUSED(4, BB); } while (0)
-    if (a.bits == 4) TW_FUSED_R(4); else TW_FUSED_R(2);
+#define TW_FUSED(RR, BB, PP) \
+    do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true, PP>, g3, b3, s, a, f); \
+         else launch_scan_kernel(decode_fused_kernel<RR, BB, false, PP>, g3, b3, s, a, f); } while (0)
+#define TW_FUSED_R(BB, PP) do { if (R == 1) TW_FUSED(1, BB, PP); else if (R == 2) TW_FUSED(2, BB, PP); else TW_FUSED(4, BB, PP); } while (0)
+    if (a.bits == 4) { if (pair) TW_FUSED_R(4, true); else TW_FUSED_R(4, false); }
+    else TW_FUSED_R(2, false);
 #undef TW_FUSED_R
 #undef TW_FUSED
 }

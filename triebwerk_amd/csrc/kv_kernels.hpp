@@ -196,7 +196,8 @@ struct FusedArgs {
 };
 bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f);
 int decode_fused_heads_per_workgroup(int G, int num_kv_heads);   // 8, 4, 2 or 1; a workgroup has 16 waves
-void launch_decode_fused(const AttnArgs& a, const FusedArgs& f, hipStream_t s);
+// allow_pairs: the 4-bit kernel whose waves scan two KV heads each, where the shape admits it (false: one head per wave)
+void launch_decode_fused(const AttnArgs& a, const FusedArgs& f, hipStream_t s, bool allow_pairs);
 // causal prefill with blocks of query tokens per wave (kv_prefill_mfma.hip); same workspace and merge
 bool prefill_mfma_usable(const AttnArgs& a);
 void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s);

@@ -123,6 +123,8 @@ class Engine:
 
     def _check_rows(self, q, k, v, out, lead) -> None:
         """The C side takes the row counts from the batch as allocated: the buffers must have exactly that shape."""
+        if self._G == 0:
+            return                      # nothing allocated: the call itself reports that
         L, H, Hk, D = self._shape
         want_q, want_kv = (*lead, self._G, H * D), (*lead, self._G, Hk * D)
         for name, t, want in (("q", q, want_q), ("out", out, want_q), ("k", k, want_kv), ("v", v, want_kv)):

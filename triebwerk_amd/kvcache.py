@@ -261,7 +261,8 @@ def set_prefill_form(form: int) -> None:
 
 
 def set_decode_fused(mode: int) -> None:
-    """0: one-launch decode step when max_seq_len <= 2048, 1: whenever the shape allows it, 2: never."""
+    """tw_kv_set_decode_fused: 0 the library's own choice, 1 one launch whenever the shape allows it, 2 never,
+    3 as 1 but with one KV head per wave also where the 4-bit kernel would give a wave two."""
     _lib.load().tw_kv_set_decode_fused(int(mode))
 
 
