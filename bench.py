@@ -333,14 +333,14 @@ def paged_bench(args):
     step_gbs = step_bytes / (elapsed / K) * 1e-9
 
     Kp = max(1, min(K, 4096 // L))
-    lib.tw_kv_profile_attention(1)
+    lib.tw_kv_debug_profile_attention(1)
     with torch.cuda.stream(stream):
         for _ in range(Kp):
             layers()
     torch.cuda.synchronize()
     total_ms, launches = C.c_double(0), C.c_int(0)
-    rc = lib.tw_kv_profile_read(C.byref(total_ms), C.byref(launches))
-    lib.tw_kv_profile_attention(0)
+    rc = lib.tw_kv_debug_profile_read(C.byref(total_ms), C.byref(launches))
+    lib.tw_kv_debug_profile_attention(0)
     assert rc == 0 and launches.value == Kp * L, (rc, launches.value)
     n_tokens_prof = int(sum(int((pos_now + i + 1).sum()) for i in range(Kp)))
     kern_ms = total_ms.value / launches.value
@@ -628,14 +628,14 @@ def decode_bench(args, kv_bits, with_probe):
     # steps that continue the same decode; the library holds 4096 event pairs
     Kp = max(1, min(K, 4096 // L))
     fused_before = lib.tw_kv_decode_fused_launches()
-    lib.tw_kv_profile_attention(1)
+    lib.tw_kv_debug_profile_attention(1)
     with torch.cuda.stream(stream):
         for _ in range(Kp):
             eager_step()
     torch.cuda.synchronize()
     total_ms, launches = C.c_double(0), C.c_int(0)
-    rc = lib.tw_kv_profile_read(C.byref(total_ms), C.byref(launches))
-    lib.tw_kv_profile_attention(0)
+    rc = lib.tw_kv_debug_profile_read(C.byref(total_ms), C.byref(launches))
+    lib.tw_kv_debug_profile_attention(0)
     assert rc == 0 and launches.value == Kp * L, (rc, launches.value)
     n_tokens_prof = int(sum(int((pos_now + i + 1).sum()) for i in range(Kp)))
     eager_kern_ms = total_ms.value / launches.value

@@ -155,27 +155,33 @@ void tw_kv_clear_error(void);
 /* Library version / build info, for the loader to print. */
 const char* tw_kv_build_info(void);
 
-/* Compressed-attention kernel choice for the launchers above and below.
- * 0 = automatic, 1 = fp32 vector-ALU kernel, 2 = MFMA kernel (kv_bits 4 and 2).
- * Process-wide; meant for tests and benchmarks. */
-void tw_kv_set_attention_variant(int variant);
-int tw_kv_get_attention_variant(void);
+/* ---- Test and benchmark hooks (tw_kv_debug_*).  They force a kernel family, a split count or a kernel form so
+ * that every path can be checked against the oracle and timed; production callers leave them alone.  All of them
+ * are process-wide switches read at every launch and not synchronised with launches on other threads: set them
+ * while no other thread is inside the library. */
 
-/* Split count override for decode attention (0 = automatic). */
-void tw_kv_set_num_splits(int nsplit);
-/* Test hook: force a form of the matrix-core prefill kernels (0 = choose from the prompt length,
- * 1 = one 16-row query block per wave, 2 = the same with mirrored block pairs, 3 = two query blocks
- * per wave with mirrored pairs, 4 = compressed cache only: the kernel that expands tiles per wave). */
-void tw_kv_set_prefill_form(int form);
+/* Compressed-attention kernel family: 0 = automatic, 1 = fp32 vector-ALU kernels, 2 = MFMA kernels. */
+void tw_kv_debug_set_attention_variant(int variant);
+int tw_kv_debug_get_attention_variant(void);
+/* Split count of decode attention (0 = automatic). */
+void tw_kv_debug_set_num_splits(int nsplit);
+/* Form of the matrix-core prefill kernels: 0 = chosen from the prompt length, 1 = one 16-row query block per wave,
+ * 2 = the same with mirrored block pairs, 3 = two query blocks per wave with mirrored pairs, 4 = compressed cache
+ * only: the kernel that expands tiles per wave. */
+void tw_kv_debug_set_prefill_form(int form);
+/* tw_turbo_append_attention_batch and the calls built on it can run a layer's decode step as ONE kernel (append,
+ * query rotation, scan, merge, rotate-back; a workgroup owns a sequence's heads) instead of three.  0 (default):
+ * what tw_kv_decode_step_plan says; 1: one kernel whenever the shape allows it (contiguous compressed cache, GQA
+ * group 1, 2 or 4); 2: never; 3: as 1, with one KV head per wave also where the 4-bit kernel would give a wave two. */
+void tw_kv_debug_set_decode_fused(int mode);
+/* Timing of the context-scanning attention kernel alone, with HIP events attached to that kernel's launches on
+ * their stream.  Enable, run eager launches (not under stream capture; at most 4096 are kept), then read the
+ * summed duration and the launch count.  Reading waits for the recorded launches and resets the counter. */
+void tw_kv_debug_profile_attention(int enable);
+int tw_kv_debug_profile_read(double* total_ms, int* launches);
 
-/* tw_turbo_append_attention_batch and the calls built on it can run a layer's decode step as ONE kernel
- * (append, query rotation, scan, merge, rotate-back; a workgroup owns a sequence's heads) instead of three.
- * 0 (default): when the contexts are short (by max_seq_len, or by tw_layer_step_args::ctx_max), where launches
- * dominate, and when ctx_min / ctx_max say the lengths are alike and the batch fills the GPU -- one sequence is one
- * workgroup's work however long it is; 1: whenever the shape allows it (contiguous compressed cache, GQA group 1, 2
- * or 4); 2: never.  Process-wide. */
-void tw_kv_set_decode_fused(int mode);
-/* The choice mode 0 makes, as a pure function of what the host knows (1 = one launch, 0 = three): G sequences,
+/* One launch or three for a layer's decode step over the compressed cache, as a pure function of what the host
+ * knows (1 = one launch, 0 = three): G sequences,
  * cache width `bits`, max_seq_len, and the range of positions + 1 (ctx_max = 0: unknown).  One launch when every
  * wave gets at most 8 tiles of 32 tokens, or when the lengths are within 1/8 of each other, the batch gives at
  * least half the CUs a workgroup and the launch stays under ~1M tokens (256k at 2 bit with 8 KV heads).
@@ -184,14 +190,6 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
 /* Layer steps that took the one-launch kernel since the library was loaded (launches issued or recorded into a
  * graph under capture): lets a benchmark say which kernel its figures belong to. */
 long long tw_kv_decode_fused_launches(void);
-
-/* Timing of the context-scanning attention kernel alone, with HIP events
- * recorded on the launch stream around that kernel (not around the merge).
- * Enable, run eager launches (not under stream capture; at most 4096 are
- * kept), then read the summed duration and the launch count.  Reading waits
- * for the recorded launches and resets the counter.  Not thread-safe. */
-void tw_kv_profile_attention(int enable);
-int tw_kv_profile_read(double* total_ms, int* launches);
 
 /* No counterpart in the reference.  Rate (GB/s) at which this GPU streams `bytes` of device
  * memory through a plain contiguous 16-byte-per-lane read kernel, averaged over `iters`
@@ -243,7 +241,7 @@ void tw_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_ha
 /* The same for the fp16 cache: what engine.cpp:1979-2003 does with launch_kv_cache_write_batch and
  * launch_gqa_attention_batch, as one launch (plus the merge of the context chunks when there are several): the
  * attention kernel takes the new token's K and V rows from k_buf / v_buf and stores them into the cache itself.
- * Same cache bytes and outputs as the two calls.  (tw_kv_set_decode_fused(2) keeps the two launches.) */
+ * Same cache bytes and outputs as the two calls.  (tw_kv_debug_set_decode_fused(2) keeps the two launches.) */
 void tw_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf, const tw_half* v_buf,
                                tw_half* ck, tw_half* cv, float* as, const int* pos, int msl, int G,
                                int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim,
@@ -305,7 +303,7 @@ typedef struct tw_layer_step_args {
     const tw_half* gate;       /* row g at gate + g*gate_stride, laid out like a row of out; NULL = none */
     long long gate_stride;
     int ctx_min, ctx_max;      /* what the host knows of min and max over g of positions[g] + 1; 0, 0 = nothing.
-                                * Only steers the choice between kernels (tw_kv_set_decode_fused), never results. */
+                                * Only steers the choice between kernels (tw_kv_debug_set_decode_fused), never results. */
 } tw_layer_step_args;
 void tw_layer_attention_step(const tw_layer_step_args* args, hipStream_t s);
 

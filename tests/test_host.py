@@ -124,3 +124,87 @@ def test_decode_step_plan_is_the_documented_rule():
     assert plan(64, 64, 8, 4, 1024, 0, 0) == 0                # GQA group 8
     assert plan(64, 16, 8, 3, 1024, 0, 0) == 0
     assert plan(0, 16, 8, 4, 1024, 0, 0) == 0
+
+
+def header_prototypes():
+    """name -> (return kind, [parameter kinds]) for every function the header declares; a kind is 'ptr', 'int',
+    'uint', 'llong', 'size', 'float', 'double', 'bool', 'void' or 'cstr'."""
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    text = re.sub(r"^\s*#.*$", "", text, flags=re.M)
+    text = re.sub(r"typedef\s+struct\s+\w+\s*\{.*?\}\s*\w+\s*;", "", text, flags=re.S)   # struct bodies hold no prototypes
+
+    def kind(decl: str) -> str:
+        decl = decl.strip()
+        if "*" in decl:
+            return "cstr" if re.match(r"const\s+char\s*\*", decl) else "ptr"
+        base = re.sub(r"\b(const|struct)\b", "", decl).split()
+        if len(base) > 1 and re.match(r"^[A-Za-z_]\w*$", base[-1]) and base[-1] not in ("int", "long", "char", "unsigned"):
+            base = base[:-1]                                       # drop the parameter's name
+        t = " ".join(base)
+        return {"int": "int", "unsigned": "uint", "unsigned int": "uint", "long long": "llong", "size_t": "size",
+                "float": "float", "double": "double", "bool": "bool", "void": "void", "hipStream_t": "ptr"}[t]
+
+    protos = {}
+    for m in re.finditer(r"([A-Za-z_][\w\s\*]*?)\b((?:launch|tw)_[a-z0-9_]+)\s*\(([^()]*)\)\s*;", text):
+        ret, name, params = m.group(1), m.group(2), m.group(3).strip()
+        plist = [] if params in ("", "void") else [kind(p) for p in params.split(",")]
+        protos[name] = (kind(ret + " x") if "*" not in ret else kind(ret), plist)
+    return protos
+
+
+def test_ctypes_table_matches_the_header_prototypes():
+    """Parameter count and kind (pointer / int / float / ...) of every prototype in the header against the ctypes
+    table the Python mirror binds, return types included: a parameter added, dropped or retyped on one side fails."""
+    from triebwerk_amd import _lib
+    C = ctypes
+    kinds = {C.c_void_p: "ptr", C.c_int: "int", C.c_uint: "uint", C.c_longlong: "llong", C.c_size_t: "size",
+             C.c_float: "float", C.c_double: "double", C.c_bool: "bool", C.c_char_p: "cstr", None: "void"}
+
+    def ckind(t):
+        if t in kinds:
+            return kinds[t]
+        assert issubclass(t, C._Pointer), t          # POINTER(struct) / POINTER(c_int) / POINTER(POINTER(c_int))
+        return "ptr"
+    protos = header_prototypes()
+    assert sorted(protos) == sorted(_lib.SIGNATURES)
+    for name, (restype, argtypes) in _lib.SIGNATURES.items():
+        want_ret, want_args = protos[name]
+        got_ret = ckind(restype)
+        # size_t and unsigned long long share a ctypes type on this platform; pointers returned as void*
+        assert got_ret == want_ret or {got_ret, want_ret} <= {"ptr", "cstr"} or (got_ret, want_ret) == ("size", "size"), \
+            f"{name}: returns {want_ret} in the header, {got_ret} in the table"
+        got_args = [ckind(t) for t in argtypes]
+        assert got_args == want_args, f"{name}: header {want_args}, table {got_args}"
+    # the struct the layer-step calls take: same number of fields as the header's
+    body = re.search(r"typedef\s+struct\s+tw_layer_step_args\s*\{(.*?)\}\s*tw_layer_step_args\s*;", HEADER.read_text(), flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    nfields = sum(len(stmt.split(",")) for stmt in body.split(";") if stmt.strip())
+    assert nfields == len(_lib.LayerStepArgs._fields_)
+
+
+def test_pybind_module_by_the_reference_name(capfd):
+    """engine_py.cpp:18-26, 44-45 and triebwerk/engine.py:23: `jetson_engine.Engine(1024, kv_bits)`, `.kv_bits()`,
+    `.reset()`.  The module is built beside the library; no GPU work happens before a batch is allocated."""
+    import importlib
+    import sys
+    from triebwerk_amd import build
+    path = build.pybind_module_path()
+    assert path.exists(), f"{path} is not built (python -m triebwerk_amd.build)"
+    sys.path.insert(0, str(path.parent))
+    try:
+        je = importlib.import_module("jetson_engine")
+    finally:
+        sys.path.pop(0)
+    e = je.Engine()
+    assert e.kv_bits() == 0 and e.max_seq_len() == 1024
+    assert je.Engine(1024, 4).kv_bits() == 4
+    assert je.Engine(max_seq_len=512, kv_bits=2).kv_bits() == 2
+    capfd.readouterr()
+    assert je.Engine(1024, kv_bits=5).kv_bits() == 0
+    assert "kv_bits=5 not supported" in capfd.readouterr().err
+    e.reset()                                   # nothing allocated yet: a no-op, as before any load in the reference
+    assert not e.is_allocated()
+    with pytest.raises(RuntimeError):
+        e.decode_step(0, 0, 0, 0)               # no arena: the C call's error becomes RuntimeError
+    with pytest.raises(RuntimeError):
+        e.set_shape(2, 16, 8, 64)               # head_dim must be 128

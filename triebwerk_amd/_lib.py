@@ -8,10 +8,7 @@ from __future__ import annotations
 import ctypes as C
 from pathlib import Path
 
-import os
-
-# TRIEBWERK_KV_LIB selects another build of the same library (e.g. an experiment).
-LIB_PATH = Path(os.environ.get("TRIEBWERK_KV_LIB") or Path(__file__).resolve().parent / "lib" / "libtriebwerk_kv.so")
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriebwerk_kv.so"
 
 P = C.c_void_p
 I = C.c_int
@@ -57,15 +54,15 @@ SIGNATURES = {
     "tw_kv_last_error_string": (C.c_char_p, []),
     "tw_kv_clear_error": (None, []),
     "tw_kv_build_info": (C.c_char_p, []),
-    "tw_kv_set_attention_variant": (None, [I]),
-    "tw_kv_get_attention_variant": (I, []),
-    "tw_kv_set_num_splits": (None, [I]),
-    "tw_kv_set_prefill_form": (None, [I]),
-    "tw_kv_set_decode_fused": (None, [I]),
+    "tw_kv_debug_set_attention_variant": (None, [I]),
+    "tw_kv_debug_get_attention_variant": (I, []),
+    "tw_kv_debug_set_num_splits": (None, [I]),
+    "tw_kv_debug_set_prefill_form": (None, [I]),
+    "tw_kv_debug_set_decode_fused": (None, [I]),
     "tw_kv_decode_fused_launches": (LL, []),
     "tw_kv_decode_step_plan": (I, [I, I, I, I, I, I, I]),
-    "tw_kv_profile_attention": (None, [I]),
-    "tw_kv_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
+    "tw_kv_debug_profile_attention": (None, [I]),
+    "tw_kv_debug_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_kv_measure_read_bandwidth": (C.c_double, [P, C.c_size_t, I, P]),
     "tw_kv_broadcast_rows": (I, [P, P, P, I, I, I, I, P]),
     "tw_attention_workspace_floats": (SZ, [I, I, I]),

@@ -106,6 +106,27 @@ def build_library(verbose: bool = False) -> Path:
     return LIB
 
 
+def pybind_module_path() -> Path:
+    import sysconfig
+    return LIBDIR / ("jetson_engine" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_pybind(verbose: bool = False) -> Path:
+    """Compile the pybind11 module `jetson_engine` (host code, g++) next to the library it links against."""
+    import sysconfig
+
+    import pybind11
+    out = pybind_module_path()
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
+           "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"],
+           str(CSRC / "jetson_engine_py.cpp"), "-o", str(out),
+           "-L", str(LIBDIR), "-ltriebwerk_kv", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    _run(cmd)
+    return out
+
+
 def build_oracle(verbose: bool = False) -> Path:
     """Compile the CPU oracle (test infrastructure) with its own Makefile."""
     cmd = ["make", "-C", str(ORACLE_DIR), "-B"]
@@ -117,4 +138,5 @@ def build_oracle(verbose: bool = False) -> Path:
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_pybind(verbose=True))
     print(build_oracle(verbose=True))

@@ -85,12 +85,7 @@ constexpr int kMaxGroup = 4;          // query heads per KV head handled by this
 // Tiles of loads in flight per wave.  Deeper is only safe while nothing spills: a spilled
 // register is reloaded through the same in-order memory counter as the prefetched tiles,
 // so every reload waits for all of them.
-#ifndef TW_DEPTH4
-#define TW_DEPTH4 1
-#endif
-#ifndef TW_DEPTH2
-#define TW_DEPTH2 1
-#endif
+constexpr int kDepth4 = 1, kDepth2 = 1;
 
 }  // namespace
 
@@ -711,7 +706,7 @@ bool launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     }
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3(grid), b3(ngroups * waves * kWave);
-#define TW_LAUNCH(P, RR, BB) launch_scan_kernel(attention_mfma_kernel<P, RR, BB, (BB == 4 ? TW_DEPTH4 : TW_DEPTH2)>, g3, b3, s, a, items, hgroups, waves)
+#define TW_LAUNCH(P, RR, BB) launch_scan_kernel(attention_mfma_kernel<P, RR, BB, (BB == 4 ? kDepth4 : kDepth2)>, g3, b3, s, a, items, hgroups, waves)
 #define TW_LAUNCH_R(P, BB) \
     do { if (R == 1) TW_LAUNCH(P, 1, BB); else if (R == 2) TW_LAUNCH(P, 2, BB); else TW_LAUNCH(P, 4, BB); } while (0)
     if (a.block_table) {

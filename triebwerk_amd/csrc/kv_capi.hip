@@ -19,7 +19,7 @@ using namespace twkv;
 
 namespace twkv {
 static std::atomic<long long> g_fused_launches{0};   // one-launch decode steps issued so far (tw_kv_decode_fused_launches)
-static std::atomic<int> g_decode_fused{0};   // tw_kv_set_decode_fused: 0 by context bound, 1 whenever possible, 2 never, 3 as 1 with one head per wave
+static std::atomic<int> g_decode_fused{0};   // tw_kv_debug_set_decode_fused: 0 by context bound, 1 whenever possible, 2 never, 3 as 1 with one head per wave
 static std::atomic<int> g_prefill_form{0};   // test hook, see prefill_form()
 int prefill_form() { return g_prefill_form.load(); }
 thread_local hipEvent_t t_scan_start = nullptr;
@@ -192,11 +192,11 @@ int tw_kv_last_error(void) { return g_err; }
 const char* tw_kv_last_error_string(void) { return g_err_msg; }
 void tw_kv_clear_error(void) { g_err = 0; g_err_msg[0] = 0; }
 const char* tw_kv_build_info(void) { return "triebwerk_kv gfx950 " __DATE__ " " __TIME__; }
-void tw_kv_set_attention_variant(int v) { g_variant.store(v); }
-int tw_kv_get_attention_variant(void) { return g_variant.load(); }
-void tw_kv_set_num_splits(int n) { g_nsplit_override.store(n); }
-void tw_kv_set_prefill_form(int form) { g_prefill_form.store(form); }
-void tw_kv_set_decode_fused(int mode) { g_decode_fused.store(mode); }
+void tw_kv_debug_set_attention_variant(int v) { g_variant.store(v); }
+int tw_kv_debug_get_attention_variant(void) { return g_variant.load(); }
+void tw_kv_debug_set_num_splits(int n) { g_nsplit_override.store(n); }
+void tw_kv_debug_set_prefill_form(int form) { g_prefill_form.store(form); }
+void tw_kv_debug_set_decode_fused(int mode) { g_decode_fused.store(mode); }
 
 int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max) {
     if (G <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || (bits != 2 && bits != 4)) return 0;
@@ -214,12 +214,12 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
 }
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }
 
-void tw_kv_profile_attention(int enable) {
+void tw_kv_debug_profile_attention(int enable) {
     g_prof.enabled.store(enable);
     if (enable) g_prof.used = 0;
 }
 
-int tw_kv_profile_read(double* total_ms, int* launches) {
+int tw_kv_debug_profile_read(double* total_ms, int* launches) {
     double sum = 0.0;
     for (int i = 0; i < g_prof.used; i++) {
         if (hipEventSynchronize(g_prof.stop[i]) != hipSuccess) return -1;
@@ -1055,25 +1055,31 @@ void tw_paged_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const ui
 // ---------------------------------------------------------------- rotation (host)
 // engine.cpp:366-392, same recipe and same library calls so that the matrix is
 // the one the reference engine uploads.
-void tw_make_rotation_host(tw_half* out_host, int d, unsigned seed) {
-    std::mt19937 gen(seed);
-    std::normal_distribution<float> dist(0.0f, 1.0f);
-    std::vector<float> mat((size_t)d * d);
-    for (int i = 0; i < d * d; i++) mat[i] = dist(gen);
-    for (int i = 0; i < d; i++) {
-        for (int j = 0; j < i; j++) {
-            float dot = 0;
-            for (int k = 0; k < d; k++) dot += mat[i * d + k] * mat[j * d + k];
-            for (int k = 0; k < d; k++) mat[i * d + k] -= dot * mat[j * d + k];
+void tw_make_rotation_host(tw_half* out_host, int n, unsigned seed) {
+    // The recipe fixes every rounding: N(0,1) entries drawn row-major from mt19937(seed) through libstdc++'s
+    // normal_distribution<float>, then modified Gram-Schmidt over the rows in fp32 -- each earlier row's component
+    // is removed in turn (the projection is taken from the row as updated so far), each sum runs over the columns
+    // in ascending order with separate multiply and add, and the row is scaled by 1 / sqrtf(sum of squares).
+    std::mt19937 engine(seed);
+    std::normal_distribution<float> gauss(0.0f, 1.0f);
+    std::vector<float> rows((size_t)n * n);
+    for (float& x : rows) x = gauss(engine);
+    for (int r = 0; r < n; r++) {
+        float* row = &rows[(size_t)r * n];
+        for (int e = 0; e < r; e++) {
+            const float* earlier = &rows[(size_t)e * n];
+            float proj = 0.0f;
+            for (int c = 0; c < n; c++) proj += row[c] * earlier[c];
+            for (int c = 0; c < n; c++) row[c] -= proj * earlier[c];
         }
-        float norm = 0;
-        for (int k = 0; k < d; k++) norm += mat[i * d + k] * mat[i * d + k];
-        norm = 1.0f / sqrtf(norm);
-        for (int k = 0; k < d; k++) mat[i * d + k] *= norm;
+        float sq = 0.0f;
+        for (int c = 0; c < n; c++) sq += row[c] * row[c];
+        const float scale = 1.0f / sqrtf(sq);
+        for (int c = 0; c < n; c++) row[c] *= scale;
     }
-    for (int i = 0; i < d * d; i++) {
-        _Float16 hv = (_Float16)mat[i];
-        memcpy(&out_host[i], &hv, 2);
+    for (size_t i = 0; i < rows.size(); i++) {
+        const _Float16 h = (_Float16)rows[i];      // round to nearest even, as __float2half
+        memcpy(&out_host[i], &h, sizeof(h));
     }
 }
 

@@ -80,10 +80,7 @@ __device__ __forceinline__ long long cache_row(const int* __restrict__ block_tab
 // The MFMA scan runs an even and the following odd chunk on the two wave groups of one CU,
 // and the group in the upper wave slots gets ~5 % less of the CU (measured; s_setprio does
 // not change it), so an even split leaves the lower group idle at the end.
-#ifndef TW_PAIR_SHARE
-#define TW_PAIR_SHARE 33
-#endif
-constexpr unsigned kPairShare = TW_PAIR_SHARE;
+constexpr unsigned kPairShare = 33;
 __device__ __forceinline__ unsigned chunk_boundary(unsigned tiles, unsigned c, unsigned nsplit) {
     if (c >= nsplit) return tiles;
     if ((c & 1u) == 0) return (c * tiles) / nsplit;             // tiles * nsplit < 2^32 (nsplit <= 64)

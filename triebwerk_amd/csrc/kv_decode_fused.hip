@@ -59,7 +59,9 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
     // the scan's probabilities and partials; before the scan the same space holds R as 8 operand tiles
-    constexpr int kPBytes = NW * 16 * 32 * 2, kPartBytes = kFusedWaves * R * kRowFloats * 4;   // 16 (part, head) partials either way
+    constexpr int kParts = PAIR ? 2 * NW : NW;                 // (part, head) partials: a wave leaves one per head it scans
+    constexpr int kRotGroups = NW / 8;                         // groups of eight waves that rotate (a wave = 16 output coordinates)
+    constexpr int kPBytes = NW * 16 * 32 * 2, kPartBytes = kParts * R * kRowFloats * 4;
     constexpr int kRotBytes = 8 * kOperandTileDwords * 4;
     __shared__ __attribute__((aligned(16))) char scan_s[kPBytes + kPartBytes > kRotBytes ? kPBytes + kPartBytes : kRotBytes];
     half_t (*p_s)[16][32] = reinterpret_cast<half_t (*)[16][32]>(scan_s);
@@ -75,7 +77,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const int Hk = a.num_kv_heads;
     const int HKW = f.hkw;
     const int nhg = Hk / HKW;
-    const int SPLIT = kFusedWaves / HKW;               // parts of the context per head (PAIR: 8 waves, 2 heads each)
+    const int SPLIT = kParts / HKW;                    // parts of the context per head
 
     // ---- unit of this workgroup.  Workgroups are dealt to the 8 XCDs in turn; the units of one sequence
     // go to one XCD so that the norm rows they all read (16 bytes per token for 8 heads) come out of one L2.
@@ -96,7 +98,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     // the rotating waves fetch their 16 rows of R.
     const int nvec = HKW * (2 + R);
     const int rot_dblk = wave & 7;
-    const bool rotating = (wave >> 3) * 16 < nvec;
+    const bool rotating = wave < 8 * kRotGroups && (wave >> 3) * 16 < nvec;
     auto unit_vector = [&](int vc, int& kind, int& head) -> const half_t* {    // vc < nvec
         if (vc < HKW) {
             kind = 0; head = hg * HKW + vc;
@@ -268,7 +270,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     // for then queues behind them.)
 
     // ---- 1. rotations of the unit's vectors
-    {
+    auto rotate_unit = [&]() {
         const int i16 = ln, kk = kg;
         const int dblk = rot_dblk;
         // the centroid table while the loads are under way: entry e fills 256 bytes with replicas.  The centroids
@@ -322,7 +324,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             lds_barrier();
         }
 
-        for (int vt = wave >> 3; vt * 16 < nvec; vt += NW / 8) {  // uniform over the wave
+        for (int vt = wave >> 3; rotating && vt * 16 < nvec; vt += kRotGroups) {  // uniform over the wave
             const int vi = vt * 16 + i16;
             const int vc = vi < nvec ? vi : nvec - 1;              // clamp reads, mask stores
             int kind, head;
@@ -367,16 +369,16 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
                 if (dblk == 0) (kind == 0 ? f.k_norms : f.v_norms)[crow * Hk + head] = (half_t)sqrtf(n2 + 1e-12f);
             }
         }
-    }
-    __syncthreads();        // table, q_rot and the new cache row are in place; R has been read
-    // the wave's slice of the probabilities starts at zero (no other wave touches it)
-    *reinterpret_cast<uint4*>(&p_s[wave][0][0] + 8 * lane) = uint4{0u, 0u, 0u, 0u};
+        __syncthreads();        // table, q_rot and the new cache row are in place; R has been read
+        // the wave's slice of the probabilities starts at zero (no other wave touches it)
+        *reinterpret_cast<uint4*>(&p_s[wave][0][0] + 8 * lane) = uint4{0u, 0u, 0u, 0u};
+    };
     // ---- 3. the parts meet in LDS.  B operand of the rotate-back first (its loads run under the merge, and stay
     // hidden there: R brought in coalesced and passed through LDS instead was 0.25 us slower per launch):
     // R[32kk + s][16*dblk + i16], s = 0..31
     const int nv = HKW * R;                                  // output vectors of this unit
     const int dblk = wave & 7;
-    const bool back = (wave >> 3) * 16 < nv;
+    const bool back = wave < 8 * kRotGroups && (wave >> 3) * 16 < nv;
     uint16_t rb[32];
     auto load_rb = [&]() {
     if (back) {
@@ -472,18 +474,20 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
 #pragma unroll
         for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
 
-        if (ntiles > 0) {
-            // kTilesAhead register sets, used in turn (two tiles in flight measured 2 % slower than one: the wave is
-            // not waiting for memory)
-            uint32x4_t kreg[kTilesAhead][4];
-            uint32x2_t vreg[kTilesAhead][2][4];
-            uint32_t nreg[kTilesAhead][2][2] = {};
+        // kTilesAhead register sets, used in turn (two tiles in flight measured 2 % slower than one: the wave is
+        // not waiting for memory; asking for the first tile before the rotations: 0.4 us slower, as with one head
+        // per wave)
+        uint32x4_t kreg[kTilesAhead][4];
+        uint32x2_t vreg[kTilesAhead][2][4];
+        uint32_t nreg[kTilesAhead][2][2] = {};
+        rotate_unit();
 #pragma unroll
-            for (int d = 0; d < kTilesAhead; d++) {
-                issue_k(kreg[d], d);
-                issue_n(nreg[d], d);
-                issue_v(vreg[d], d);
-            }
+        for (int d = 0; d < kTilesAhead; d++) {
+            issue_k(kreg[d], d);
+            issue_n(nreg[d], d);
+            issue_v(vreg[d], d);
+        }
+        if (ntiles > 0) {
             // A operand of the score MFMAs: row m < 8: query head m % R of KV head m / R of the pair (fp16 value),
             // row m + 8 its rounding remainder; q_rot[..][32 pkg + 8 j + i]
             half8_t aq[4];
@@ -657,6 +661,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             }
         }
     } else {
+        rotate_unit();
         {
             int l2 = lane;
             asm volatile("" : "+v"(l2));
@@ -880,7 +885,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     lds_barrier();
 
     // ---- out[vector][d] = sum_k o[vector][k] R[k][d]; lane group kk owns k in [32kk, 32kk+32)
-    for (int vt = wave >> 3; vt * 16 < nv; vt += NW / 8) {
+    for (int vt = wave >> 3; back && vt * 16 < nv; vt += kRotGroups) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
         const float* orow = &o_s[vt * 16 + ln][32 * kg];
 #pragma unroll
@@ -937,11 +942,11 @@ bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
 }
 
 // Two KV heads per wave (PAIR) when the cache is 4 bit and the workgroup's heads come in pairs: eight waves, every
-// cache line fetched by one instruction.  The workgroup then has 512 threads: its HKW * (2 + R) vectors must fit
-// the 32 staging slots and its HKW * R outputs the 16 merge slots.
+// cache line fetched by one instruction.  The workgroup's HKW * (2 + R) vectors must fit its staging slots (a
+// vector per 16 threads) and its HKW * R outputs its merge slots (one per 32 threads).
 bool decode_fused_pairs(const AttnArgs& a, int hkw) {
     const int R = a.num_heads / a.num_kv_heads;
-    return a.bits == 4 && (hkw & 1) == 0 && hkw * (2 + R) <= 32 && hkw * R <= 16;
+    return a.bits == 4 && (hkw & 1) == 0 && (2 * kPairWaves) % hkw == 0 && hkw * (2 + R) <= 4 * kPairWaves && hkw * R <= 2 * kPairWaves;
 }
 
 void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s, bool allow_pairs) {

@@ -210,7 +210,7 @@ void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form);
 // same workspace and merge as the scan; form as for launch_prefill_f16_mfma
 bool prefill_tq_mfma_usable(const AttnArgs& a);
 void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form);
-// test hook (tw_kv_set_prefill_form): 0 = automatic; 1-3 force a form of the flash prefill kernels; 4 = the
+// test hook (tw_kv_debug_set_prefill_form): 0 = automatic; 1-3 force a form of the flash prefill kernels; 4 = the
 // compressed prefill kernel that expands tiles per wave
 int prefill_form();
 // 2-bit decode scan for 8 KV heads whose waves load whole cache rows together (kv_attention_mfma2c.hip)

@@ -253,21 +253,21 @@ def make_rotation(head_dim: int = 128, seed: int = 42) -> torch.Tensor:
 
 
 def set_attention_variant(variant: int) -> None:
-    _lib.load().tw_kv_set_attention_variant(int(variant))
+    _lib.load().tw_kv_debug_set_attention_variant(int(variant))
 
 
 def set_prefill_form(form: int) -> None:
-    _lib.load().tw_kv_set_prefill_form(int(form))
+    _lib.load().tw_kv_debug_set_prefill_form(int(form))
 
 
 def set_decode_fused(mode: int) -> None:
-    """tw_kv_set_decode_fused: 0 the library's own choice, 1 one launch whenever the shape allows it, 2 never,
+    """tw_kv_debug_set_decode_fused: 0 the library's own choice, 1 one launch whenever the shape allows it, 2 never,
     3 as 1 but with one KV head per wave also where the 4-bit kernel would give a wave two."""
-    _lib.load().tw_kv_set_decode_fused(int(mode))
+    _lib.load().tw_kv_debug_set_decode_fused(int(mode))
 
 
 def set_num_splits(nsplit: int) -> None:
-    _lib.load().tw_kv_set_num_splits(int(nsplit))
+    _lib.load().tw_kv_debug_set_num_splits(int(nsplit))
 
 
 # ---- producers of q and k (engine.cpp:126-127, 162-163), in place
