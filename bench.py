@@ -300,10 +300,14 @@ def paged_bench(args):
     def layers():
         for l in range(L):
             ck, cv, kn, vn = pools[l]
-            kvcache.tw_paged_turbo_kv_append_batch(ck, kn, cv, vn, k[l], v[l], rot, pos, d_bt, pages_per_seq, G, Hk, D,
-                                                   kv_dim, kv_bits)
-            kvcache.tw_paged_turbo_gqa_attention_batch(out[l], q[l], ck, cv, kn, vn, rot, ws, pos, d_bt, pages_per_seq,
-                                                       msl, G, H, Hk, D, q_dim, kv_dim, kv_bits)
+            if args.launchers == "reference":      # the two calls: append, then attention (four launches)
+                kvcache.tw_paged_turbo_kv_append_batch(ck, kn, cv, vn, k[l], v[l], rot, pos, d_bt, pages_per_seq, G, Hk, D,
+                                                       kv_dim, kv_bits)
+                kvcache.tw_paged_turbo_gqa_attention_batch(out[l], q[l], ck, cv, kn, vn, rot, ws, pos, d_bt, pages_per_seq,
+                                                           msl, G, H, Hk, D, q_dim, kv_dim, kv_bits)
+            else:                                  # the layer step in one call (three launches)
+                kvcache.tw_paged_turbo_append_attention_batch(out[l], q[l], k[l], v[l], ck, cv, kn, vn, rot, ws, pos, d_bt,
+                                                              pages_per_seq, msl, G, H, Hk, D, q_dim, kv_dim, kv_bits)
         pos.add_(1)
 
     use_graph = not args.no_graph
@@ -354,7 +358,9 @@ def paged_bench(args):
                    "kv_bits": kv_bits, "layers": L, "num_heads": H, "num_kv_heads": Hk, "head_dim": D, "batch": G,
                    "pages": n_pages, "context_first_timed_step": [int(ctx0.min()), int(ctx0.max())],
                    "tokens_attended_per_step": n_tokens_timed / K, "hipgraph": use_graph,
-                   "step": "paged append K,V + paged decode attention for every layer, positions += 1"},
+                   "step": ("paged append K,V + paged decode attention for every layer (two calls, four launches), positions += 1"
+                            if args.launchers == "reference" else
+                            "tw_paged_turbo_append_attention_batch for every layer (three launches), positions += 1")},
         "step_algorithmic_GB": step_bytes * 1e-9, "step_achieved_GBps": step_gbs,
         "step_frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": "paged decode attention (context scan), one launch per layer",

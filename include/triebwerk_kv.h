@@ -350,6 +350,18 @@ void tw_paged_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const ui
                                         int num_kv_heads, int head_dim, int q_dim, int kv_dim,
                                         int bits, hipStream_t s);
 
+/* One decode step of one layer over the paged compressed cache in a single call: append K and V at positions[g]
+ * (into the page block_table names), then attention over 0..positions[g] -- tw_turbo_append_attention_batch with
+ * the paged contract above.  The appended rows and the query are rotated in one launch, so the call is three
+ * launches where tw_paged_turbo_kv_append_batch + tw_paged_turbo_gqa_attention_batch are four; same cache bytes,
+ * same outputs.  ws and max_context as for tw_paged_turbo_gqa_attention_batch. */
+void tw_paged_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf, const tw_half* v_buf,
+                                           uint8_t* ck_q, uint8_t* cv_q, tw_half* k_norms, tw_half* v_norms,
+                                           const tw_half* rotation, float* ws, const int* positions,
+                                           const int* block_table, int bt_stride, int max_context, int G,
+                                           int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                           int bits, hipStream_t s);
+
 /* No counterpart in the reference.  launch_turbo_gqa_attention_batch for callers that cannot allocate and have
  * no scratch to hand over (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
  * the same arguments without `as`, same kernels and results; the split workspace is a device array inside the

@@ -250,6 +250,20 @@ def test_ragged_paged_batch64(kv, oracle, rotation_fixture, bits):
         err = rel_err_rows(host(out), want)
         assert err.max() <= TOL, f"variant {variant}: max rel err {err.max():.3e} (sequence {err.argmax() // H})"
     kv.set_attention_variant(0)
+    # the layer step in one call (append + attention, three launches): the appended rows are wiped first, so the
+    # call has to write them again -- same bytes through the block-table gather, same outputs
+    for g in range(G):
+        page, slot = int(bt[g, pos[g] // 16]), int(pos[g] % 16)
+        for pool in (p_ck, p_cv, p_kn, p_vn):
+            pool[page, slot] = 0
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    kv.tw_paged_turbo_append_attention_batch(out, dev(q), dev(k), dev(v), p_ck, p_cv, p_kn, p_vn, rot, ws, dev(pos), d_bt,
+                                             pages_per_seq, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+    assert np.array_equal(gather(p_ck), ock) and np.array_equal(gather(p_cv), ocv)
+    assert np.array_equal(gather(p_kn).view(np.uint16), okn.view(np.uint16))
+    assert np.array_equal(gather(p_vn).view(np.uint16), ovn.view(np.uint16))
+    err = rel_err_rows(host(out), want)
+    assert err.max() <= TOL, f"one call: max rel err {err.max():.3e} (sequence {err.argmax() // H})"
 
 
 def test_tq2_gqa4_context4097(kv, oracle, rotation_fixture):

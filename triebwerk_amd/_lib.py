@@ -80,6 +80,7 @@ SIGNATURES = {
     "tw_paged_turbo_kv_append_batch": (None, [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_paged_gqa_attention_batch": (None, [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
     "tw_paged_turbo_gqa_attention_batch": (None, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
+    "tw_paged_turbo_append_attention_batch": (None, [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
     "tw_turbo_gqa_attention_batch_noalloc": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P]),
     "tw_make_rotation_host": (None, [P, I, C.c_uint]),
     # Engine

@@ -1052,6 +1052,58 @@ void tw_paged_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const ui
     run_attention(a, s, "tw_paged_turbo_gqa_attention_batch");
 }
 
+// One decode step of a layer over the paged cache: the K and V rows of the new token and the query are rotated in
+// one launch (the appended rows quantized into their pages), then the scan over the pages and the merge -- three
+// launches where tw_paged_turbo_kv_append_batch + tw_paged_turbo_gqa_attention_batch take four.
+void tw_paged_turbo_append_attention_batch(tw_half* out, const tw_half* q, const tw_half* k_buf, const tw_half* v_buf,
+                                           uint8_t* ck_q, uint8_t* cv_q, tw_half* k_norms, tw_half* v_norms,
+                                           const tw_half* rotation, float* ws, const int* positions,
+                                           const int* block_table, int bt_stride, int max_context, int G,
+                                           int num_heads, int num_kv_heads, int head_dim, int q_dim, int kv_dim,
+                                           int bits, hipStream_t s) {
+    const char* fn = "tw_paged_turbo_append_attention_batch";
+    if (!check_shape(fn, num_heads, num_kv_heads, head_dim) || !check_bits(fn, bits)) return;
+    if (!block_table) { set_error(1, "%s: block_table is NULL", fn); return; }
+    if (kv_dim != num_kv_heads * head_dim) {
+        set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, kv_dim);
+        return;
+    }
+    AttnArgs a;
+    fill_common(a, out, q, q_dim, ck_q, cv_q, k_norms, v_norms, rotation, G, num_heads, num_kv_heads, bits, ws);
+    a.pos_mode = kPosArray; a.positions = positions;
+    a.block_table = block_table; a.bt_stride = bt_stride;
+    plan_splits(a, max_context, kPagedBlockFloats);
+    const int R = num_heads / num_kv_heads;
+    const bool fuse_q = mfma_wanted(a) && a.qrot && (R == 1 || R == 2 || R == 4) &&
+                        (reinterpret_cast<uintptr_t>(a.qrot) & 15u) == 0;
+    if (!fuse_q) {                 // shapes the MFMA kernels do not take: the two calls
+        tw_paged_turbo_kv_append_batch(ck_q, k_norms, cv_q, v_norms, k_buf, v_buf, rotation, positions, block_table,
+                                       bt_stride, G, num_kv_heads, head_dim, kv_dim, bits, s);
+        run_attention(a, s, fn);
+        return;
+    }
+    RotArgs r;
+    memset(&r, 0, sizeof(r));
+    fill_quant_segments(r, ck_q, k_norms, k_buf, cv_q, v_norms, v_buf, 2, G, num_kv_heads, kv_dim);
+    int k = r.nseg++;
+    r.seg_src[k] = H(q);
+    r.seg_stride[k] = q_dim;
+    r.seg_heads[k] = num_heads;
+    r.seg_nvec[k] = G * num_heads;
+    r.seg_units[k] = (r.seg_nvec[k] + 15) / 16 * 8;
+    r.seg_kind[k] = 1;
+    r.rotation = H(rotation);
+    r.positions = positions;
+    r.block_table = block_table;
+    r.bt_stride = bt_stride;
+    r.num_kv_heads = num_kv_heads;
+    r.qrot = a.qrot;
+    r.qrot_stride = a.ws_stride;
+    r.q_scale = attention_mfma_q_scale(bits);
+    launch_rotate(r, bits, s);
+    run_attention(a, s, fn, /*query_done=*/true);
+}
+
 // ---------------------------------------------------------------- rotation (host)
 // engine.cpp:366-392, same recipe and same library calls so that the matrix is
 // the one the reference engine uploads.

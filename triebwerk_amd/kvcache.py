@@ -241,6 +241,20 @@ def tw_paged_turbo_gqa_attention_batch(out, q, ck_q, cv_q, k_norms, v_norms, rot
     _done(lib)
 
 
+def tw_paged_turbo_append_attention_batch(out, q, k_buf, v_buf, ck_q, cv_q, k_norms, v_norms, rotation, ws, positions,
+                                          block_table, bt_stride, max_context, G, num_heads, num_kv_heads, head_dim,
+                                          q_dim, kv_dim, bits, stream=None):
+    lib = _lib.load()
+    lib.tw_paged_turbo_append_attention_batch(_ptr(out, "f16", "out"), _ptr(q, "f16", "q"), _ptr(k_buf, "f16", "k_buf"),
+                                              _ptr(v_buf, "f16", "v_buf"), _ptr(ck_q, "u8", "ck_q"),
+                                              _ptr(cv_q, "u8", "cv_q"), _ptr(k_norms, "f16", "k_norms"),
+                                              _ptr(v_norms, "f16", "v_norms"), _ptr(rotation, "f16", "rotation"),
+                                              _ptr(ws, "f32", "ws"), _ptr(positions, "i32", "positions"),
+                                              _ptr(block_table, "i32", "block_table"), bt_stride, max_context, G,
+                                              num_heads, num_kv_heads, head_dim, q_dim, kv_dim, bits, _stream(stream))
+    _done(lib)
+
+
 def attention_workspace_floats(G, num_heads, max_context) -> int:
     return int(_lib.load().tw_attention_workspace_floats(G, num_heads, max_context))
 
