@@ -160,7 +160,8 @@ const char* tw_kv_build_info(void);
  * are process-wide switches read at every launch and not synchronised with launches on other threads: set them
  * while no other thread is inside the library. */
 
-/* Compressed-attention kernel family: 0 = automatic, 1 = fp32 vector-ALU kernels, 2 = MFMA kernels. */
+/* Compressed-attention kernel family: 0 = automatic, 1 = fp32 vector-ALU kernels, 2 = MFMA kernels, 3 = MFMA kernels
+ * with one KV head per wave also where the 4-bit scan would give a wave two. */
 void tw_kv_debug_set_attention_variant(int variant);
 int tw_kv_debug_get_attention_variant(void);
 /* Split count of decode attention (0 = automatic). */

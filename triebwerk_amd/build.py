@@ -25,6 +25,7 @@ SOURCES = [
     "kv_attention_valu.hip",
     "kv_attention_mfma.hip",
     "kv_attention_mfma2c.hip",
+    "kv_attention_pair.hip",
     "kv_decode_fused.hip",
     "kv_prefill_mfma.hip",
     "kv_prefill_f16_mfma.hip",

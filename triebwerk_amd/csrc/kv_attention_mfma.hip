@@ -692,6 +692,10 @@ bool launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
         launch_attention_mfma2c_scan(a, s);
         return false;
     }
+    if (attention_variant() != 3 && attention_pair_usable(a)) {      // 4 bit, KV heads in pairs: two heads per wave
+        launch_attention_pair_scan(a, s);
+        return false;
+    }
     const int waves = scan_waves(a);
     const int hgroups = a.num_kv_heads / waves;
     const int items = a.G * a.nsplit * hgroups;

@@ -22,6 +22,8 @@ static std::atomic<long long> g_fused_launches{0};   // one-launch decode steps 
 static std::atomic<int> g_decode_fused{0};   // tw_kv_debug_set_decode_fused: 0 by context bound, 1 whenever possible, 2 never, 3 as 1 with one head per wave
 static std::atomic<int> g_prefill_form{0};   // test hook, see prefill_form()
 int prefill_form() { return g_prefill_form.load(); }
+static std::atomic<int> g_attention_variant{0};   // tw_kv_debug_set_attention_variant, see attention_variant()
+int attention_variant() { return g_attention_variant.load(); }
 thread_local hipEvent_t t_scan_start = nullptr;
 thread_local hipEvent_t t_scan_stop = nullptr;
 }  // namespace twkv
@@ -30,7 +32,7 @@ thread_local hipEvent_t t_scan_stop = nullptr;
 namespace {
 thread_local int g_err = 0;
 thread_local char g_err_msg[256] = "";
-std::atomic<int> g_variant{0};
+std::atomic<int> g_variant{0};   // tw_kv_debug_set_attention_variant
 std::atomic<int> g_nsplit_override{0};
 
 constexpr int kMaxSplits = 64;
@@ -192,7 +194,7 @@ int tw_kv_last_error(void) { return g_err; }
 const char* tw_kv_last_error_string(void) { return g_err_msg; }
 void tw_kv_clear_error(void) { g_err = 0; g_err_msg[0] = 0; }
 const char* tw_kv_build_info(void) { return "triebwerk_kv gfx950 " __DATE__ " " __TIME__; }
-void tw_kv_debug_set_attention_variant(int v) { g_variant.store(v); }
+void tw_kv_debug_set_attention_variant(int v) { g_variant.store(v); twkv::g_attention_variant.store(v); }
 int tw_kv_debug_get_attention_variant(void) { return g_variant.load(); }
 void tw_kv_debug_set_num_splits(int n) { g_nsplit_override.store(n); }
 void tw_kv_debug_set_prefill_form(int form) { g_prefill_form.store(form); }

@@ -30,6 +30,7 @@
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 #include "kv_mfma_util.hpp"
+#include "kv_pair_scan.hpp"
 #include "kv_producer_util.hpp"
 #include "kv_rotate_util.hpp"
 
@@ -40,7 +41,6 @@ namespace {
 constexpr int kFusedWaves = 16;
 constexpr int kPairWaves = 8;                  // waves of a workgroup whose waves scan two KV heads each
 constexpr unsigned kFusedShare = 33;           // 64ths of a sequence's tiles that go to the lower eight waves
-constexpr int kTilesAhead = 1;                 // tiles of loads a wave of that kernel keeps in flight
 constexpr unsigned kPairTileShare = 32;        // the same with eight waves in all: two per SIMD, no upper slots
 constexpr int kFusedMaxQ = 32;                 // query heads of a unit: HKW * R <= 8 * 4
 constexpr int kRowFloats = kHeadDim + 4;       // LDS row of a vector: conflict-free 16-byte accesses
@@ -388,38 +388,16 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     }
     };
     if constexpr (PAIR) {
-        // ---- 2 (PAIR). scan of this wave's part, two KV heads per wave.  A 128-byte line of a cache row is two
-        // 4-bit heads: with a head per wave two waves fetch every line, each for its half.  Here a wave takes both
-        // halves, so every load instruction covers whole lines that no other instruction touches, and the loads
-        // carry the non-temporal hint (see kStreamCodes): the same bytes arrive ~11 % faster.  The two heads share
-        // the MFMAs: score columns 0-7 are 8 tokens of the first head, columns 8-15 the same tokens of the second;
-        // P.V columns 0-7 are dims of the first head, 8-15 of the second; the A operands carry the query heads
-        // (probabilities) of both KV heads in rows hd * R + r (+ 8: rounding remainders).  A product of a row with
-        // a column of the other head is computed and never used.
+        // ---- 2 (PAIR). scan of this wave's part, two KV heads per wave (kv_pair_scan.hpp has the tile and why)
         int l2 = lane;
         asm volatile("" : "+v"(l2));
-        const int pn = l2 & 15, pkg = l2 >> 4;
-        const int hd = pn >> 3;                                   // head of the pair this lane's columns belong to
-        const int pw = hk_local >> 1;
-        const uint32_t lane_rep = (uint32_t)l2 * 4u;
+        PairLane<R> L;
+        L.init(l2, p_s[wave], tab_s);
         const uint32_t kvp = (uint32_t)Hk * kHeadBytes;
         const uint32_t nrow = (uint32_t)Hk * 2u;
-        // K: instruction c of a tile covers tokens 8c .. 8c+7, lane l the 16-byte piece l % 8 of token l / 8
-        const uint32_t koff = (uint32_t)(l2 >> 3) * kvp + 16u * (uint32_t)(l2 & 7);
-        // operand order: lane (pn, pkg) takes token pn % 8, head pn / 8, dims 32 pkg .. +31 = piece 4 hd + pkg
-        const int ksrc = 4 * (8 * (pn & 7) + 4 * hd + pkg);
-        // V: lane (pn, pkg) loads 8 bytes (16 dims: head pn / 8, dims 16 (pn % 8) ..) of tokens 4 pkg + i (+ 16)
-        const uint32_t voff = (uint32_t)(4 * pkg) * kvp + 8u * (uint32_t)pn;
-        // softmax: a lane owns the scores of tokens tok0 and tok0 + 16 of its head
-        const bool useful = R == 4 ? ((pkg & 1) == hd) : ((pkg & 1) == 0);
-        const int tok0 = 8 * (pkg >> 1) + (pn & 7);
-        const uint32_t noff = (uint32_t)tok0 * nrow;
-        half_t* p_w = &p_s[wave][hd * R][8 * (tok0 >> 2) + (tok0 & 3)];     // row + r (+ 8), token tok0 + 16: + 4
-        const uint4* p_r = reinterpret_cast<const uint4*>(&p_s[wave][pn][8 * pkg]);
-        constexpr float kRaise = 5.0f;
-        const char* tab_lane = reinterpret_cast<const char*>(tab_s);
-        auto lut32 = [&](uint32_t addr) -> uint32_t { return *reinterpret_cast<const uint32_t*>(tab_lane + addr); };
-
+        const uint32_t koff = L.koff_rows * kvp + L.koff_bytes;
+        const uint32_t voff = L.voff_rows * kvp + L.voff_bytes;
+        const uint32_t noff = (uint32_t)L.tok0 * nrow;
         const long long seq_row0 = (long long)g * a.seq_stride_rows;
         const char* kpair = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes;
         const char* vpair = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes;
@@ -427,239 +405,60 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         const char* vnpair = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
         // (loads of a tile index past the wave's last one are given an empty extent: they return zeros without touching memory)
         auto tile_rows = [&](int i, int tile) -> int { return i < ntiles ? max(min(n - tile, 32), 0) : 0; };
-        auto issue_k = [&](uint32x4_t (&kr)[4], int i) {
+        auto issue_k = [&](PairTileRegs& t, int i) {
             const int tile = tile_at(i);
             __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (seq_row0 + tile) * kvp, tile_rows(i, tile) * (int)kvp);
 #pragma unroll
-            for (int c = 0; c < 4; c++) kr[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kStreamCodes);
+            for (int c = 0; c < 4; c++) t.k[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kStreamCodes);
         };
-        auto issue_v = [&](uint32x2_t (&vr)[2][4], int i) {
+        auto issue_v = [&](PairTileRegs& t, int i) {
             const int tile = tile_at(i);
             __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (seq_row0 + tile) * kvp, tile_rows(i, tile) * (int)kvp);
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    vr[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kStreamCodes);
+                    t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kStreamCodes);
             }
         };
-        // norms of the pair (two fp16) for the lane's two tokens: [token][K | V]
-        auto issue_n = [&](uint32_t (&nr)[2][2], int i) {
+        auto issue_n = [&](PairTileRegs& t, int i) {
             const int tile = tile_at(i);
             const int rows = tile_rows(i, tile);
             __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
             __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
-            if (useful) {
-                nr[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
-                nr[1][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)(noff + 16u * nrow), 0, kStreamNorms);
-                nr[0][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
-                nr[1][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)(noff + 16u * nrow), 0, kStreamNorms);
+            if (L.useful) {
+                t.n[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
+                t.n[1][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)(noff + 16u * nrow), 0, kStreamNorms);
+                t.n[0][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
+                t.n[1][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)(noff + 16u * nrow), 0, kStreamNorms);
             }
         };
-        auto head_max = [&](float v) -> float {                   // over the lanes of this lane's head
-            v = fmaxf(v, __shfl_xor(v, 1, 64)); v = fmaxf(v, __shfl_xor(v, 2, 64)); v = fmaxf(v, __shfl_xor(v, 4, 64));
-            v = fmaxf(v, __shfl_xor(v, 16, 64)); v = fmaxf(v, __shfl_xor(v, 32, 64));
-            return v;
-        };
-        auto head_sum = [&](float v) -> float {
-            v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64);
-            v += __shfl_xor(v, 16, 64); v += __shfl_xor(v, 32, 64);
-            return v;
-        };
 
-        float4_t o[16];
-#pragma unroll
-        for (int j = 0; j < 16; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-        float m_run[R], l_run[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
-
-        // kTilesAhead register sets, used in turn (two tiles in flight measured 2 % slower than one: the wave is
-        // not waiting for memory; asking for the first tile before the rotations: 0.4 us slower, as with one head
-        // per wave)
-        uint32x4_t kreg[kTilesAhead][4];
-        uint32x2_t vreg[kTilesAhead][2][4];
-        uint32_t nreg[kTilesAhead][2][2] = {};
+        PairState<R> S;
+        S.reset();
+        // One tile of loads in flight per wave.  (Tried: two tiles, 2 % slower -- the wave is not waiting for memory;
+        // the first tile asked for before the rotations, 0.4 us slower, as with one head per wave; the scores of tile
+        // i + 1 placed beside the P.V of tile i for the scheduler to interleave, 3 % slower.)
+        PairTileRegs t;
+        t.n[0][0] = t.n[0][1] = t.n[1][0] = t.n[1][1] = 0u;
         rotate_unit();
-#pragma unroll
-        for (int d = 0; d < kTilesAhead; d++) {
-            issue_k(kreg[d], d);
-            issue_n(nreg[d], d);
-            issue_v(vreg[d], d);
-        }
+        issue_k(t, 0);
+        issue_n(t, 0);
+        issue_v(t, 0);
         if (ntiles > 0) {
-            // A operand of the score MFMAs: row m < 8: query head m % R of KV head m / R of the pair (fp16 value),
-            // row m + 8 its rounding remainder; q_rot[..][32 pkg + 8 j + i]
-            half8_t aq[4];
-            {
-                const int m = pn & 7;
-                const bool lo_part = (pn & 8) != 0;
-                const bool live = m < 2 * R;
-                const float* qr = &qrot_s[(hk_local + (live ? m / R : 0)) * R + (live ? m % R : 0)][32 * pkg];
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
-                    float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
-                    float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        float x = live ? v[i] : 0.0f;
-                        half_t hi = (half_t)x;
-                        half_t lo = (half_t)(x - (float)hi);
-                        aq[j][i] = lo_part ? lo : hi;
-                    }
-                }
-            }
-
-            auto scan_tile = [&](int it, uint32x4_t (&kreg)[4], uint32x2_t (&vreg)[2][4], uint32_t (&nreg)[2][2]) {
-                const int tile = tile_at(it);
-                const int ahead = it + kTilesAhead;              // the tile this register set is asked for next
-
-                // ---- scores: set c = tokens 8c .. 8c+7 of both heads
-                float4_t s[4];
-#pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    union { uint32_t u[4]; half8_t h; } kv[4];
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const uint32_t w = (uint32_t)__builtin_amdgcn_ds_bpermute(ksrc, (int)kreg[c][j]);
-                        kv[j].u[0] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0400u));
-                        kv[j].u[1] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0500u));
-                        kv[j].u[2] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0600u));
-                        kv[j].u[3] = lut32(__builtin_amdgcn_perm(w, lane_rep, 0x0c0c0700u));
-                    }
-                    s[c] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int j = 0; j < 4; j++) s[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[j], kv[j].h, s[c], 0, 0, 0);
-                }
-                issue_k(kreg, ahead);
-
-                // ---- online softmax (base 2): this lane owns tokens tok0 and tok0 + 16 of head hd
-                float kn[2], vn[2];
-#pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    kn[t] = h2f_bits(hd ? (nreg[t][0] >> 16) : (nreg[t][0] & 0xffffu));
-                    vn[t] = h2f_bits(hd ? (nreg[t][1] >> 16) : (nreg[t][1] & 0xffffu));
-                }
-                issue_n(nreg, ahead);
-                const bool valid[2] = {useful && (tile + tok0 < n), useful && (tile + tok0 + 16 < n)};
-                float raw[2][R], x[2][R];
-                bool raise = false;
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    // the row of (hd, r): hd * R + r; rows 0-3 sit in lane group 0 (R = 4: the second head's in group 1),
-                    // their remainders 32 lanes further on
-                    float v[4];
-#pragma unroll
-                    for (int c = 0; c < 4; c++) v[c] = R == 4 ? s[c][r] : (hd ? s[c][R + r] : s[c][r]);
-                    uint32x2_t s01 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[1]), false, false);
-                    uint32x2_t s23 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[2]), __float_as_uint(v[3]), false, false);
-                    raw[0][r] = (__uint_as_float(s01[0]) + __uint_as_float(s01[1])) * kn[0];    // kernels.cu:1707
-                    raw[1][r] = (__uint_as_float(s23[0]) + __uint_as_float(s23[1])) * kn[1];
-#pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        x[t][r] = valid[t] ? raw[t][r] - m_run[r] : kNegBig;
-                        raise = raise || (x[t][r] > kRaise);
-                    }
-                }
-                if (__any(raise)) {
-#pragma unroll
-                    for (int r = 0; r < R; r++) {
-                        const float mine = fmaxf(valid[0] ? raw[0][r] : kNegBig, valid[1] ? raw[1][r] : kNegBig);
-                        const float m_new = fmaxf(m_run[r], head_max(mine));
-                        const float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_new);
-                        m_run[r] = m_new;
-                        l_run[r] *= alpha;
-#pragma unroll
-                        for (int t = 0; t < 2; t++) x[t][r] = valid[t] ? raw[t][r] - m_new : kNegBig;
-                        // accumulator register i of a lane is row 4 pkg + i: query head i % R (of either KV head)
-#pragma unroll
-                        for (int j = 0; j < 16; j++) {
-#pragma unroll
-                            for (int i = r; i < 4; i += R) o[j][i] *= alpha;
-                        }
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-#pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        const float pe = __builtin_amdgcn_exp2f(x[t][r]);
-                        l_run[r] += pe;
-                        const float pf = pe * vn[t];                            // (s * vn) * centroid, kernels.cu:1765
-                        const half_t hi = (half_t)pf;
-                        const half_t lo = (half_t)(pf - (float)hi);
-                        if (useful) {
-                            p_w[r * 32 + 4 * t] = hi;
-                            p_w[(r + 8) * 32 + 4 * t] = lo;
-                        }
-                    }
-                }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                union { uint4 q; half8_t h; } pa;
-                pa.q = *p_r;
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-
-                // ---- O[row][dim 16 (pn % 8) + j of head pn / 8] += P[row][token] V[token][dim]
-                uint32_t xe[2][4], xo[2][4];
-#pragma unroll
-                for (int dw = 0; dw < 2; dw++) {
-#pragma unroll
-                    for (int sub = 0; sub < 2; sub++) {
-#pragma unroll
-                        for (int pr = 0; pr < 2; pr++) {
-                            const uint32_t wa = vreg[sub][2 * pr][dw], wb = vreg[sub][2 * pr + 1][dw];
-                            xe[dw][2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
-                            xo[dw][2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
-                        }
-                    }
-                }
-                issue_v(vreg, ahead);
-#pragma unroll
-                for (int dw = 0; dw < 2; dw++) {
-#pragma unroll
-                    for (int jp = 0; jp < 4; jp++) {
-                        const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
-                        union { uint32_t u[4]; half8_t h; } be, bo;
-#pragma unroll
-                        for (int q4 = 0; q4 < 4; q4++) {
-                            be.u[q4] = lut32(__builtin_amdgcn_perm(xe[dw][q4], lane_rep, sel));
-                            bo.u[q4] = lut32(__builtin_amdgcn_perm(xo[dw][q4], lane_rep, sel));
-                        }
-                        o[8 * dw + 2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[8 * dw + 2 * jp], 0, 0, 0);
-                        o[8 * dw + 2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[8 * dw + 2 * jp + 1], 0, 0, 0);
-                    }
-                }
-            };
-            for (int it = 0; it < ntiles; it += kTilesAhead) {
-#pragma unroll
-                for (int d = 0; d < kTilesAhead; d++) {
-                    if (it + d < ntiles) scan_tile(it + d, kreg[d], vreg[d], nreg[d]);
-                }
-            }
+            S.load_query(L, [&](int i) -> const float* { return &qrot_s[hk_local * R + i][0]; });
+            for (int it = 0; it < ntiles; it++)
+                pair_scan_tile<R>(L, S, t, tile_at(it), n, [&]() { issue_k(t, it + 1); }, [&]() { issue_n(t, it + 1); },
+                                  [&]() { issue_v(t, it + 1); });
         }
         load_rb();
-        // the wave's partials: rows hd * R + r of the columns of head hd, value + remainder rows added
-        const int khi = R == 4 ? hd : 0;                          // lane group that holds the rows of head hd
+        pair_scan_finish<R>(L, S, 1.0f / kAlpha, [&](int hd, int r, const float (&ov)[16]) {
+            float* pr = &part_s[part * HKW + hk_local + hd][r][0];
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            l_run[r] = head_sum(l_run[r]);
-            float ov[16];
-#pragma unroll
-            for (int j = 0; j < 16; j++) {
-                float v = R == 4 ? o[j][r] : (hd ? o[j][R + r] : o[j][r]);
-                ov[j] = (v + __shfl_xor(v, 32, 64)) * (1.0f / kAlpha);
-            }
-            if (pkg == khi) {
-                float* pr = &part_s[part * HKW + hk_local + hd][r][0];
-#pragma unroll
-                for (int j4 = 0; j4 < 4; j4++)
-                    *reinterpret_cast<float4*>(pr + 16 * (pn & 7) + 4 * j4) = float4{ov[4 * j4], ov[4 * j4 + 1], ov[4 * j4 + 2], ov[4 * j4 + 3]};
-                if ((pn & 7) == 0) { pr[kHeadDim] = m_run[r]; pr[kHeadDim + 1] = l_run[r]; }
-            }
-        }
+            for (int j4 = 0; j4 < 4; j4++)
+                *reinterpret_cast<float4*>(pr + 16 * (L.pn & 7) + 4 * j4) = float4{ov[4 * j4], ov[4 * j4 + 1], ov[4 * j4 + 2], ov[4 * j4 + 3]};
+            if ((L.pn & 7) == 0) { pr[kHeadDim] = S.m_run[r]; pr[kHeadDim + 1] = S.l_run[r]; }
+        });
     } else {
         rotate_unit();
         {

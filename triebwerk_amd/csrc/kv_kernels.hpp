@@ -213,6 +213,13 @@ void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form);
 // test hook (tw_kv_debug_set_prefill_form): 0 = automatic; 1-3 force a form of the flash prefill kernels; 4 = the
 // compressed prefill kernel that expands tiles per wave
 int prefill_form();
+// 4-bit decode scan whose waves take two KV heads each and read whole cache lines (kv_attention_pair.hip); same
+// workspace, partials and merge as attention_mfma_kernel
+bool attention_pair_usable(const AttnArgs& a);
+void launch_attention_pair_scan(const AttnArgs& a, hipStream_t s);
+// test hook (tw_kv_debug_set_attention_variant): 0 automatic, 1 vector-ALU kernels, 2 MFMA kernels, 3 MFMA kernels
+// with one KV head per wave also where the 4-bit scan would give a wave two
+int attention_variant();
 // 2-bit decode scan for 8 KV heads whose waves load whole cache rows together (kv_attention_mfma2c.hip)
 bool attention_mfma2c_usable(const AttnArgs& a);
 void launch_attention_mfma2c_scan(const AttnArgs& a, hipStream_t s);

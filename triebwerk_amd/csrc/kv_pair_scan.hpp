@@ -1,0 +1,265 @@
+// kv_pair_scan.hpp -- the 32-token tile of the 4-bit decode scan with TWO KV heads per wave, shared by the kernels
+// that use it (kv_decode_fused.hip: the one-launch decode step; kv_attention_pair.hip: the stand-alone scan).
+//
+// Why pairs.  A 128-byte line of a compressed cache row is two 4-bit heads (2 x 64 bytes of codes).  With one head
+// per wave two waves fetch every line, each for its half.  When a wave takes both halves every load instruction
+// covers whole lines that no other instruction touches, and the loads can carry the non-temporal hint
+// (kStreamCodes): a launch that only reads 554 MB then takes 78-82 us instead of 88-90 us on MI355X.  With
+// half-line loads the hint doubles the fetches, so the two go together.
+//
+// Mathematics as turbo_gqa_attention_batch_kernel of the reference (kernels.cu:1688-1766): scores
+// s_p = (q_rot . c(K codes_p)) * kn_p (q_rot pre-scaled by log2(e) / sqrt(D) / alpha), online softmax in base 2,
+// acc += (w_p * vn_p) * c(V codes_p).  The operand conventions (table look-up by v_perm_b32 address, fp16 value +
+// rounding remainder rows for q_rot and the probabilities, running maximum raised only past 2^5) are those of
+// kv_attention_mfma.hip.
+//
+// Layout of a tile in a wave (lane = (pn = lane % 16, pkg = lane / 16), hd = pn / 8 the head of the pair):
+//   loads    K: instruction c (0..3) covers tokens 8c .. 8c+7, lane l the 16-byte piece l % 8 of token l / 8 of the
+//            pair's 128-byte row.  V: lane (pn, pkg) loads 8 bytes (16 dims of head hd: dims 16 (pn % 8) ..) of tokens
+//            4 pkg + i and 16 + 4 pkg + i, i = 0..3.  Norms: 4 bytes (the pair's two fp16) of tokens tok0 and tok0 + 16.
+//   scores   MFMA set c: columns 0-7 = tokens 8c .. 8c+7 of the first head, columns 8-15 the same tokens of the second
+//            (one ds_bpermute per dword brings piece 4 hd + pkg of token pn % 8 to lane (pn, pkg)); the A operand holds
+//            the query heads of both KV heads: row hd * R + r the fp16 value, row + 8 the rounding remainder.
+//   softmax  two permlane32 swaps per query head add value and remainder rows and leave lane (pn, pkg) with the scores
+//            of tokens tok0 = 8 (pkg / 2) + pn % 8 and tok0 + 16 of head hd (R = 4: lane groups of the other parity
+//            hold the other head's rows and own nothing).
+//   P.V      the probabilities times the V norms go through the wave's 1 KB LDS tile into A-operand order (rows as
+//            above); MFMA j: columns 0-7 = dim 16 (pn % 8) + j of the first head, 8-15 of the second.
+// A product of a row with a column of the other head is computed and never used.
+#pragma once
+
+#include "kv_common.hpp"
+#include "kv_mfma_util.hpp"
+
+namespace twkv {
+
+constexpr uint32_t kPairRowBytes = 128;      // two 4-bit heads of one token
+
+// What a lane knows about itself (derive once, after any code that would otherwise keep these alive in registers).
+template <int R>
+struct PairLane {
+    int pn, pkg, hd;
+    uint32_t lane_rep;      // byte offset of the lane's replica inside a table entry
+    int ksrc;               // ds_bpermute address: source lane of the K operand
+    bool useful;            // owns two (token, head) pairs of every tile
+    int tok0;               // the first of them (the other: tok0 + 16)
+    half_t* p_w;            // where its probabilities go in the wave's P tile (row hd * R, column of tok0)
+    const uint4* p_r;       // its A operand of the P.V MFMAs
+    const char* tab;        // the centroid table
+    uint32_t koff_rows, koff_bytes;   // K: row l / 8 and byte 16 (l % 8) inside a pair row
+    uint32_t voff_rows, voff_bytes;   // V: row 4 pkg and byte 8 pn
+
+    __device__ __forceinline__ void init(int lane, half_t (*p_tile)[32], const uint32_t* table) {
+        pn = lane & 15; pkg = lane >> 4; hd = pn >> 3;
+        lane_rep = (uint32_t)lane * 4u;
+        ksrc = 4 * (8 * (pn & 7) + 4 * hd + pkg);
+        useful = R == 4 ? ((pkg & 1) == hd) : ((pkg & 1) == 0);
+        tok0 = 8 * (pkg >> 1) + (pn & 7);
+        p_w = &p_tile[hd * R][8 * (tok0 >> 2) + (tok0 & 3)];
+        p_r = reinterpret_cast<const uint4*>(&p_tile[pn][8 * pkg]);
+        tab = reinterpret_cast<const char*>(table);
+        koff_rows = (uint32_t)(lane >> 3); koff_bytes = 16u * (uint32_t)(lane & 7);
+        voff_rows = (uint32_t)(4 * pkg); voff_bytes = 8u * (uint32_t)pn;
+    }
+    __device__ __forceinline__ uint32_t lut32(uint32_t addr) const { return *reinterpret_cast<const uint32_t*>(tab + addr); }
+    // reductions over the lanes of this lane's head (lane groups of both parities included: those that own nothing
+    // contribute the neutral element)
+    __device__ __forceinline__ float head_max(float v) const {
+        v = fmaxf(v, __shfl_xor(v, 1, 64)); v = fmaxf(v, __shfl_xor(v, 2, 64)); v = fmaxf(v, __shfl_xor(v, 4, 64));
+        v = fmaxf(v, __shfl_xor(v, 16, 64)); v = fmaxf(v, __shfl_xor(v, 32, 64));
+        return v;
+    }
+    __device__ __forceinline__ float head_sum(float v) const {
+        v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64);
+        v += __shfl_xor(v, 16, 64); v += __shfl_xor(v, 32, 64);
+        return v;
+    }
+};
+
+// The registers of one tile in flight.
+struct PairTileRegs {
+    uint32x4_t k[4];        // instruction c
+    uint32x2_t v[2][4];     // [sub-tile][i]
+    uint32_t n[2][2];       // [token tok0 | tok0 + 16][K | V]: the pair's two fp16 norms
+};
+
+template <int R>
+struct PairState {
+    float4_t o[16];         // accumulator of P.V MFMA j
+    float m_run[R], l_run[R];
+    half8_t aq[4];          // A operand of the score MFMAs
+
+    __device__ __forceinline__ void reset() {
+#pragma unroll
+        for (int j = 0; j < 16; j++) o[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
+    }
+    // q_rot of the pair's query heads: row(i) -> the 128 floats of query head i (i = hd * R + r, 0 <= i < 2 R)
+    template <class RowOf>
+    __device__ __forceinline__ void load_query(const PairLane<R>& L, RowOf row_of) {
+        const int m = L.pn & 7;
+        const bool lo_part = (L.pn & 8) != 0;
+        const bool live = m < 2 * R;
+        const float* qr = row_of(live ? m : 0) + 32 * L.pkg;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
+            float4 v1 = *reinterpret_cast<const float4*>(qr + 8 * j + 4);
+            float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float x = live ? v[i] : 0.0f;
+                half_t hi = (half_t)x;
+                half_t lo = (half_t)(x - (float)hi);
+                aq[j][i] = lo_part ? lo : hi;
+            }
+        }
+    }
+};
+
+// One tile.  `tile` is its first token, `n` the tokens of the sequence; after_k / after_n / after_v are called as
+// soon as the K, norm and V registers of `t` have been consumed (the caller re-issues them for a later tile there).
+template <int R, class AfterK, class AfterN, class AfterV>
+__device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R>& S, PairTileRegs& t, int tile, int n,
+                                               AfterK after_k, AfterN after_n, AfterV after_v) {
+    constexpr float kRaise = 5.0f;                     // raise the running max only past 2^5
+    // ---- scores: set c = tokens 8c .. 8c+7 of both heads
+    float4_t s[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        union { uint32_t u[4]; half8_t h; } kv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t w = (uint32_t)__builtin_amdgcn_ds_bpermute(L.ksrc, (int)t.k[c][j]);
+            kv[j].u[0] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0400u));
+            kv[j].u[1] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0500u));
+            kv[j].u[2] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0600u));
+            kv[j].u[3] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0700u));
+        }
+        s[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; j++) s[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(S.aq[j], kv[j].h, s[c], 0, 0, 0);
+    }
+    after_k();
+
+    // ---- online softmax (base 2): this lane owns tokens tok0 and tok0 + 16 of head hd
+    float kn[2], vn[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        kn[i] = h2f_bits(L.hd ? (t.n[i][0] >> 16) : (t.n[i][0] & 0xffffu));
+        vn[i] = h2f_bits(L.hd ? (t.n[i][1] >> 16) : (t.n[i][1] & 0xffffu));
+    }
+    after_n();
+    const bool valid[2] = {L.useful && (tile + L.tok0 < n), L.useful && (tile + L.tok0 + 16 < n)};
+    float raw[2][R], x[2][R];
+    bool raise = false;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        // the row of (hd, r): hd * R + r; rows 0-3 sit in lane group 0 (R = 4: the second head's in group 1), their
+        // remainders 32 lanes further on
+        float v[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) v[c] = R == 4 ? s[c][r] : (L.hd ? s[c][R + r] : s[c][r]);
+        uint32x2_t s01 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[1]), false, false);
+        uint32x2_t s23 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[2]), __float_as_uint(v[3]), false, false);
+        raw[0][r] = (__uint_as_float(s01[0]) + __uint_as_float(s01[1])) * kn[0];    // kernels.cu:1707
+        raw[1][r] = (__uint_as_float(s23[0]) + __uint_as_float(s23[1])) * kn[1];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            x[i][r] = valid[i] ? raw[i][r] - S.m_run[r] : kNegBig;
+            raise = raise || (x[i][r] > kRaise);
+        }
+    }
+    if (__any(raise)) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float mine = fmaxf(valid[0] ? raw[0][r] : kNegBig, valid[1] ? raw[1][r] : kNegBig);
+            const float m_new = fmaxf(S.m_run[r], L.head_max(mine));
+            const float alpha = __builtin_amdgcn_exp2f(S.m_run[r] - m_new);
+            S.m_run[r] = m_new;
+            S.l_run[r] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 2; i++) x[i][r] = valid[i] ? raw[i][r] - m_new : kNegBig;
+            // accumulator register i of a lane is row 4 pkg + i: query head i % R (of either KV head)
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+#pragma unroll
+                for (int i = r; i < 4; i += R) S.o[j][i] *= alpha;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const float pe = __builtin_amdgcn_exp2f(x[i][r]);
+            S.l_run[r] += pe;
+            const float pf = pe * vn[i];                            // (s * vn) * centroid, kernels.cu:1765
+            const half_t hi = (half_t)pf;
+            const half_t lo = (half_t)(pf - (float)hi);
+            if (L.useful) {
+                L.p_w[r * 32 + 4 * i] = hi;
+                L.p_w[(r + 8) * 32 + 4 * i] = lo;
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    union { uint4 q; half8_t h; } pa;
+    pa.q = *L.p_r;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- O[row][dim 16 (pn % 8) + j of head pn / 8] += P[row][token] V[token][dim]
+    uint32_t xe[2][4], xo[2][4];
+#pragma unroll
+    for (int dw = 0; dw < 2; dw++) {
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+            for (int pr = 0; pr < 2; pr++) {
+                const uint32_t wa = t.v[sub][2 * pr][dw], wb = t.v[sub][2 * pr + 1][dw];
+                xe[dw][2 * sub + pr] = (wa & 0x0f0f0f0fu) | ((wb << 4) & 0xf0f0f0f0u);
+                xo[dw][2 * sub + pr] = ((wa >> 4) & 0x0f0f0f0fu) | (wb & 0xf0f0f0f0u);
+            }
+        }
+    }
+    after_v();
+#pragma unroll
+    for (int dw = 0; dw < 2; dw++) {
+#pragma unroll
+        for (int jp = 0; jp < 4; jp++) {
+            const uint32_t sel = 0x0c0c0400u + ((uint32_t)jp << 8);
+            union { uint32_t u[4]; half8_t h; } be, bo;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                be.u[q4] = L.lut32(__builtin_amdgcn_perm(xe[dw][q4], L.lane_rep, sel));
+                bo.u[q4] = L.lut32(__builtin_amdgcn_perm(xo[dw][q4], L.lane_rep, sel));
+            }
+            S.o[8 * dw + 2 * jp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, S.o[8 * dw + 2 * jp], 0, 0, 0);
+            S.o[8 * dw + 2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, S.o[8 * dw + 2 * jp + 1], 0, 0, 0);
+        }
+    }
+}
+
+// The wave's partial result per (head of the pair, query head): sink(hd, r, dims) is called by the 16 lanes that
+// hold the rows of head hd with dims = the lane's 16 values of dim 16 (pn % 8) .. +15 (value + remainder rows added,
+// 1 / alpha applied); all lanes end with l_run summed over the head.
+template <int R, class Sink>
+__device__ __forceinline__ void pair_scan_finish(const PairLane<R>& L, PairState<R>& S, float inv_alpha, Sink sink) {
+    const int khi = R == 4 ? L.hd : 0;                          // lane group that holds the rows of head hd
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        S.l_run[r] = L.head_sum(S.l_run[r]);
+        float ov[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            float v = R == 4 ? S.o[j][r] : (L.hd ? S.o[j][R + r] : S.o[j][r]);
+            ov[j] = (v + __shfl_xor(v, 32, 64)) * inv_alpha;
+        }
+        if (L.pkg == khi) sink(L.hd, r, ov);
+    }
+}
+
+}  // namespace twkv
