@@ -381,7 +381,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const bool back = wave < 8 * kRotGroups && (wave >> 3) * 16 < nv;
     uint16_t rb[32];
     auto load_rb = [&]() {
-    if (back) {
+    if (PAIR || back) {          // (PAIR: eight waves, every one of them rotates back)
         const uint16_t* rp = reinterpret_cast<const uint16_t*>(a.rotation) + (32 * kg) * kHeadDim + 16 * dblk + ln;
 #pragma unroll
         for (int s = 0; s < 32; s++) rb[s] = rp[s * kHeadDim];
@@ -445,13 +445,13 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         issue_k(t, 0);
         issue_n(t, 0);
         issue_v(t, 0);
+        load_rb();              // behind the first tile's loads; the registers are there, and the epilogue need not wait
         if (ntiles > 0) {
             S.load_query(L, [&](int i) -> const float* { return &qrot_s[hk_local * R + i][0]; });
             for (int it = 0; it < ntiles; it++)
                 pair_scan_tile<R>(L, S, t, tile_at(it), n, [&]() { issue_k(t, it + 1); }, [&]() { issue_n(t, it + 1); },
                                   [&]() { issue_v(t, it + 1); });
         }
-        load_rb();
         pair_scan_finish<R>(L, S, 1.0f / kAlpha, [&](int hd, int r, const float (&ov)[16]) {
             float* pr = &part_s[part * HKW + hk_local + hd][r][0];
 #pragma unroll
@@ -683,20 +683,28 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     }
     lds_barrier();
 
-    // ---- out[vector][d] = sum_k o[vector][k] R[k][d]; lane group kk owns k in [32kk, 32kk+32)
+    // ---- out[vector][d] = sum_k o[vector][k] R[k][d]; lane group kk owns k in [32kk, 32kk+32).  On fp16 MFMAs: R is
+    // exact in fp16, o enters as fp16 value + rounding remainder, every product is exact in the fp32 accumulator --
+    // only the order of the additions differs from the reference's chain (kernels.cu:1769-1775), far inside what the
+    // fp16 result resolves -- and the chain is 8 MFMAs instead of 32.
     for (int vt = wave >> 3; back && vt * 16 < nv; vt += kRotGroups) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
         const float* orow = &o_s[vt * 16 + ln][32 * kg];
 #pragma unroll
-        for (int s4 = 0; s4 < 8; s4++) {
-            float4 o4 = *reinterpret_cast<const float4*>(orow + 4 * s4);
-            const float ov[4] = {o4.x, o4.y, o4.z, o4.w};
+        for (int st = 0; st < 4; st++) {
+            float4 oa = *reinterpret_cast<const float4*>(orow + 8 * st);
+            float4 ob = *reinterpret_cast<const float4*>(orow + 8 * st + 4);
+            const float ov[8] = {oa.x, oa.y, oa.z, oa.w, ob.x, ob.y, ob.z, ob.w};
+            half8_t ahi, alo;
+            union { uint16_t u[8]; half8_t h; } bm;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                union { uint16_t u; half_t h; } cv;
-                cv.u = rb[4 * s4 + j];
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ov[j], (float)cv.h, acc, 0, 0, 0);
+            for (int i = 0; i < 8; i++) {
+                ahi[i] = (half_t)ov[i];
+                alo[i] = (half_t)(ov[i] - (float)ahi[i]);
+                bm.u[i] = rb[8 * st + i];
             }
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bm.h, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bm.h, acc, 0, 0, 0);
         }
         // lane holds out[vector vt*16 + 4kk + r][d = 16*dblk + i16]
 #pragma unroll
