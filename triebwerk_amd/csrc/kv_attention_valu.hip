@@ -10,10 +10,15 @@
 //   - a workgroup owns (sequence, KV head, context chunk): the query heads of a
 //     GQA group share every byte that is loaded, and long contexts are split
 //     over workgroups (split-K) with a log-sum-exp merge;
-//   - four adjacent lanes own one token: each loads 16 bytes (32 codes) of the
+//   - compressed cache: four adjacent lanes own one token: each loads 16 bytes (32 codes) of the
 //     64-byte K row, so a wave reads 16 tokens per load instruction, dequantizes
 //     in registers through a 16-entry LDS centroid table and reduces the dot
 //     product over the quad with two cross-lane shuffles;
+//   - fp16 cache: EIGHT adjacent lanes own one token and each load instruction takes 16 bytes
+//     per lane, i.e. one whole 128-byte line of the head's 256-byte row per token: a line that one
+//     instruction covers in full can be loaded non-temporally (every cache byte is read once per
+//     launch; a plain read of the same bytes runs at 7.0 instead of 6.2 TB/s with the hint), while
+//     a line that two instructions share would be fetched twice under it;
 //   - softmax is online (running max / running sum per lane), so no score ever
 //     goes to memory; V is accumulated in registers in the rotated basis and
 //     rotated back once per (sequence, head) (kernels.cu:1769-1775).
@@ -26,7 +31,8 @@ namespace twkv {
 
 constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / kWave;
-constexpr int kTokensPerIter = kAttnWaves * 16;  // 16 token quads per wave
+// lanes that own one token, and the values of its head each of them holds
+template <int MODE> struct LanesPerToken { static constexpr int value = MODE == 0 ? 8 : 4; };
 constexpr float kNegBig = -1e30f;                // the reference's max init (kernels.cu:1686)
 
 __device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
@@ -35,14 +41,14 @@ __device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
     return g;
 }
 
-// Dimension owned by element e (0..31) of lane-in-quad c.
+// Dimension owned by element e of lane c of a token's lanes.
 template <int MODE>
 __device__ __forceinline__ int lane_dim(int c, int e) {
-    if (MODE == 0) return 32 * (e / 8) + 8 * c + (e % 8);  // four 16-byte pieces, interleaved over the quad
+    if (MODE == 0) return 64 * (e / 8) + 8 * c + (e % 8);  // two 16-byte pieces, one per 128-byte line
     return 32 * c + e;                                     // one contiguous piece of codes
 }
 
-// Load and dequantize the lane's 32 values of one cache row (one KV head).
+// Load and dequantize the lane's values (16 of an fp16 row, 32 of a compressed one) of one cache row (one KV head).
 // fresh: fp16 only, the head's 128 halves come from there instead (the row of the token being appended), or NULL.
 template <int MODE>
 __device__ __forceinline__ void load_vals(const void* __restrict__ base, long long row, int num_kv_heads,
@@ -50,10 +56,11 @@ __device__ __forceinline__ void load_vals(const void* __restrict__ base, long lo
                                           const half_t* fresh = nullptr) {
     if (MODE == 0) {
         const half_t* p = reinterpret_cast<const half_t*>(base) + (row * num_kv_heads + h) * kHeadDim;
-        if (fresh) p = fresh;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            half8_t h8 = *reinterpret_cast<const half8_t*>(p + 32 * j + 8 * c);
+        for (int j = 0; j < 2; j++) {
+            // the eight lanes of a token take one whole line per instruction: non-temporal
+            half8_t h8 = fresh ? *reinterpret_cast<const half8_t*>(fresh + 64 * j + 8 * c)
+                               : __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(p + 64 * j + 8 * c));
 #pragma unroll
             for (int i = 0; i < 8; i++) vals[8 * j + i] = (float)h8[i];
         }
@@ -109,7 +116,11 @@ attention_valu_kernel(AttnArgs a) {
 
     const int tid = threadIdx.x;
     const int wave = tid / kWave, lane = tid % kWave;
-    const int qd = lane / 4, c = lane % 4;
+    constexpr int LPT = LanesPerToken<MODE>::value;      // lanes per token
+    constexpr int E = kHeadDim / LPT;                     // values of the head per lane
+    constexpr int kTokensPerWave = kWave / LPT;
+    constexpr int kTokensPerIter = kAttnWaves * kTokensPerWave;
+    const int qd = lane / LPT, c = lane % LPT;
     const int chunk = blockIdx.x;
     const int g = blockIdx.z;
     const int group = a.num_heads / a.num_kv_heads;
@@ -158,15 +169,15 @@ attention_valu_kernel(AttnArgs a) {
     }
     __syncthreads();
 
-    float qreg[RT][32];
-    float acc[RT][32];
+    float qreg[RT][E];
+    float acc[RT][E];
     float m[RT], l[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) {
         m[r] = kNegBig;
         l[r] = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 32; e++) {
+        for (int e = 0; e < E; e++) {
             qreg[r][e] = q_s[r][lane_dim<MODE>(c, e)];
             acc[r][e] = 0.0f;
         }
@@ -174,16 +185,16 @@ attention_valu_kernel(AttnArgs a) {
     const float scale = 0.08838834764831845f;   // 1/sqrt(128)
 
     for (int tb = t0; tb < t1; tb += kTokensPerIter) {
-        const int t = tb + wave * 16 + qd;
+        const int t = tb + wave * kTokensPerWave + qd;
         const bool valid = t < t1;
-        const int tc = valid ? t : (t1 - 1);    // clamp: keep the quad shuffles convergent
+        const int tc = valid ? t : (t1 - 1);    // clamp: keep the shuffles among a token's lanes convergent
         const long long row = cache_row(a.block_table, a.bt_stride, a.seq_stride_rows, g, tc);
         float kn = 1.0f, vn = 1.0f;
         if (MODE != 0) {
             kn = (float)a.k_norms[row * a.num_kv_heads + h];
             vn = (float)a.v_norms[row * a.num_kv_heads + h];
         }
-        float vals[32];
+        float vals[E];
         const bool fresh = APPEND && tc == n - 1;
         load_vals<MODE>(a.k, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? k_fresh : nullptr);
         float s[RT];
@@ -191,9 +202,9 @@ attention_valu_kernel(AttnArgs a) {
         for (int r = 0; r < RT; r++) {
             float dot = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 32; e++) dot = __builtin_fmaf(qreg[r][e], vals[e], dot);
-            dot += __shfl_xor(dot, 1, 64);
-            dot += __shfl_xor(dot, 2, 64);
+            for (int e = 0; e < E; e++) dot = __builtin_fmaf(qreg[r][e], vals[e], dot);
+#pragma unroll
+            for (int off = 1; off < LPT; off <<= 1) dot += __shfl_xor(dot, off, 64);
             s[r] = dot * (kn * scale);          // kernels.cu:1707
         }
         load_vals<MODE>(a.v, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? v_fresh : nullptr);
@@ -204,19 +215,19 @@ attention_valu_kernel(AttnArgs a) {
                     float alpha = __expf(m[r] - s[r]);
                     l[r] *= alpha;
 #pragma unroll
-                    for (int e = 0; e < 32; e++) acc[r][e] *= alpha;
+                    for (int e = 0; e < E; e++) acc[r][e] *= alpha;
                     m[r] = s[r];
                 }
                 float p = __expf(s[r] - m[r]);
                 l[r] += p;
                 float pv = p * vn;              // (s * vn) * centroid, kernels.cu:1765
 #pragma unroll
-                for (int e = 0; e < 32; e++) acc[r][e] = __builtin_fmaf(pv, vals[e], acc[r][e]);
+                for (int e = 0; e < E; e++) acc[r][e] = __builtin_fmaf(pv, vals[e], acc[r][e]);
             }
         }
     }
 
-    // ---- merge the 64 token streams of the workgroup (16 quads x 4 waves)
+    // ---- merge the token streams of the workgroup (64 / LPT per wave, 4 waves)
     float mw[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) mw[r] = wave_max(m[r]);
@@ -234,20 +245,20 @@ attention_valu_kernel(AttnArgs a) {
         m[r] = mg;
         l[r] *= f;
 #pragma unroll
-        for (int e = 0; e < 32; e++) acc[r][e] *= f;
-        // sum over the 16 quads of the wave (lanes with equal c)
+        for (int e = 0; e < E; e++) acc[r][e] *= f;
+        // sum over the token streams of the wave (lanes with equal c)
 #pragma unroll
-        for (int off = 4; off < 64; off <<= 1) {
+        for (int off = LPT; off < 64; off <<= 1) {
             l[r] += __shfl_xor(l[r], off, 64);
 #pragma unroll
-            for (int e = 0; e < 32; e++) acc[r][e] += __shfl_xor(acc[r][e], off, 64);
+            for (int e = 0; e < E; e++) acc[r][e] += __shfl_xor(acc[r][e], off, 64);
         }
     }
     if (qd == 0) {
 #pragma unroll
         for (int r = 0; r < RT; r++) {
 #pragma unroll
-            for (int e = 0; e < 32; e++) red_s[wave][r][lane_dim<MODE>(c, e)] = acc[r][e];
+            for (int e = 0; e < E; e++) red_s[wave][r][lane_dim<MODE>(c, e)] = acc[r][e];
             if (c == 0) ml_s[wave][r][1] = l[r];
         }
     }
