@@ -119,7 +119,7 @@ def cpu_baseline(w, kv_bits, seconds_budget=15.0):
     bounded sample of the workload: one layer, as many sequences as fit the time budget."""
     import gen
     import oracle_lib
-    o = oracle_lib.load()
+    o = oracle_lib.load_o3()          # the oracle's source built -O3 for x86-64-v3 (oracle/Makefile)
     threads = o.num_threads()
     H, Hk, D = w["H"], w["Hk"], 128
     kv_dim, q_dim = Hk * D, H * D
@@ -161,7 +161,7 @@ def cpu_baseline(w, kv_bits, seconds_budget=15.0):
     tokens_per_s = S * layers / (t * w["L"])   # `layers` layers measured; a step needs L of them
     return dict(value=tokens_per_s, unit="tokens/s", cores=threads, kind="port",
                 sample=f"{layers} of {w['L']} layers x {S} of {w['G']} sequences at context {ctx}, "
-                       f"{t:.2f} s of CPU time, scaled linearly; OpenMP over (sequence, head), "
+                       f"{t:.2f} s of CPU time, scaled linearly; oracle/kv_oracle.cpp built -O3 -march=x86-64-v3, OpenMP over (sequence, head), "
                        f"{os.cpu_count()} logical CPUs visible")
 
 

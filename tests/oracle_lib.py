@@ -167,6 +167,10 @@ class Oracle:
 _cached = None
 
 
+LIB_O3 = ROOT / "oracle" / "libkv_oracle_o3.so"
+_cached_o3 = None
+
+
 def load() -> Oracle:
     global _cached
     if _cached is None:
@@ -174,3 +178,13 @@ def load() -> Oracle:
             subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
         _cached = Oracle(C.CDLL(str(LIB)))
     return _cached
+
+
+def load_o3() -> Oracle:
+    """The -O3 build of the same source (oracle/Makefile): what the benchmark times as the CPU baseline."""
+    global _cached_o3
+    if _cached_o3 is None:
+        if not LIB_O3.exists():
+            subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
+        _cached_o3 = Oracle(C.CDLL(str(LIB_O3)))
+    return _cached_o3

@@ -672,3 +672,33 @@ def test_sigmoid_gate_is_x_times_sigmoid(oracle):
     assert data[1].view(np.uint16) == d0[1].view(np.uint16)
     assert data[2] == 0
     assert np.array_equal(data[n:].view(np.uint16), d0[n:].view(np.uint16))
+
+
+def test_o3_build_of_the_oracle_gives_the_same_bits(oracle, rotation_fixture):
+    """The benchmark times the oracle's source built -O3 -march=x86-64-v3 (oracle/Makefile); it must be the same
+    arithmetic: compressed append and attention of a small case, bit for bit against the -O2 build the tests use."""
+    import oracle_lib
+    o3 = oracle_lib.load_o3()
+    r = gen.rng(4242)
+    G, H, Hk, msl, D = 3, 8, 4, 70, 128
+    kv_dim, q_dim = Hk * D, H * D
+    for bits in (4, 2):
+        outs = []
+        for o in (oracle, o3):
+            rr = gen.rng(4242 + bits)
+            kvp = kv_dim * bits // 8
+            ck = np.zeros((G, msl, kvp), np.uint8); cv = np.zeros_like(ck)
+            kn = np.zeros((G, msl, Hk), np.float16); vn = np.zeros_like(kn)
+            for g in range(G):
+                n = 40 + 10 * g
+                k_rows = gen.normal_f16(rr, (n, kv_dim)); v_rows = gen.normal_f16(rr, (n, kv_dim))
+                p = np.arange(n, dtype=np.int32)
+                o.turbo_kv_quantize(ck[g], kn[g], k_rows, rotation_fixture, p, msl, n, Hk, D, kv_dim, bits)
+                o.turbo_kv_quantize(cv[g], vn[g], v_rows, rotation_fixture, p, msl, n, Hk, D, kv_dim, bits)
+            q = gen.normal_f16(rr, (G, q_dim))
+            pos = np.array([39, 49, 59], np.int32)
+            out = np.zeros((G, q_dim), np.float16)
+            o.turbo_gqa_attention_batch(out, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
+            outs.append((ck.copy(), cv.copy(), kn.copy(), vn.copy(), out.copy()))
+        for a, b in zip(*outs):
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
