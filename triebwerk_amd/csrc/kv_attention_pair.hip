@@ -49,15 +49,15 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     int chunk = 0, g = 0, h = 0, n = 0, t0 = 0, t1 = 0;
     const char *kpair = nullptr, *vpair = nullptr, *knpair = nullptr, *vnpair = nullptr;
     const int* bt = nullptr;
-    long long seq_row0 = 0;
     int nseg = 0;                                             // balanced walk: partials sequence g gets; 0 = even chunks
     auto set_bases = [&]() {                                  // scalar bases of this wave's pair of heads
-        kpair = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes4;
-        vpair = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes4;
-        knpair = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
-        vnpair = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
+        // (contiguous cache: from the sequence's first row, which leaves one multiplication per tile and array)
+        const long long row0 = PAGED ? 0 : (long long)g * a.seq_stride_rows;
+        kpair = reinterpret_cast<const char*>(a.k) + row0 * kvp + (long long)h * kHeadBytes4;
+        vpair = reinterpret_cast<const char*>(a.v) + row0 * kvp + (long long)h * kHeadBytes4;
+        knpair = reinterpret_cast<const char*>(a.k_norms) + row0 * nrow + (long long)h * 2;
+        vnpair = reinterpret_cast<const char*>(a.v_norms) + row0 * nrow + (long long)h * 2;
         bt = PAGED ? a.block_table + (long long)g * a.bt_stride : nullptr;
-        seq_row0 = (long long)g * a.seq_stride_rows;
     };
     auto decode = [&](int item) -> bool {                    // false: the chunk holds no token
         const int hg = item % hgroups;
@@ -91,7 +91,8 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     };
 
     // Loads of a tile.  Contiguous cache: one descriptor over the rows of the tile that exist (rows past the
-    // sequence's end read as zeros).  Paged cache: a tile is two 16-token pages, each with its own descriptor; the
+    // sequence's end read as zeros, and so does a tile past the chunk's last one, which is asked for with no rows
+    // rather than skipped by a branch).  Paged cache: a tile is two 16-token pages, each with its own descriptor; the
     // two block-table entries of a tile are fetched one tile ahead (even lanes the first page, odd lanes the second),
     // before the loads of the tile in between, so they have returned, in order, by the time they are needed.  Past
     // the end the last page is re-read (its tokens are masked).
@@ -100,6 +101,8 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
         return (long long)__builtin_amdgcn_readlane(pages, sub) * kPageTokens;
     };
     int pages_next = 0;                          // entries of the tile whose loads are issued next in the loop
+    // `pages`: paged cache, the tile's two block-table entries; contiguous cache, the rows of the tile that exist
+    auto tile_rows = [&](int tile) -> int { return max(min(n - tile, 32), 0); };
     auto issue_k = [&](PairTileRegs& t, int tile, int pages) {
         if (PAGED) {
 #pragma unroll
@@ -109,7 +112,7 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
                 t.k[2 * sub + 1] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + 8u * kvp), 0, kStreamCodes);
             }
         } else {
-            __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
+            __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (long long)tile * kvp, pages * (int)kvp);
 #pragma unroll
             for (int c = 0; c < 4; c++) t.k[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kStreamCodes);
         }
@@ -123,7 +126,7 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
                 for (int j = 0; j < 4; j++) t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)j * kvp), 0, kStreamCodes);
             }
         } else {
-            __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (seq_row0 + tile) * kvp, max(min(n - tile, 32), 0) * (int)kvp);
+            __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (long long)tile * kvp, pages * (int)kvp);
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
@@ -139,30 +142,25 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
             for (int i = 0; i < 2; i++) {
                 __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + page_row(pages, i) * nrow, kPageTokens * (int)nrow);
                 __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + page_row(pages, i) * nrow, kPageTokens * (int)nrow);
-                if (L.useful) {
-                    t.n[i][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
-                    t.n[i][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
-                }
+                t.n[i][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
+                t.n[i][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
             }
         } else {
-            const int rows = max(min(n - tile, 32), 0);
-            __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
-            __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
-            if (L.useful) {
-                t.n[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
-                t.n[1][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)(noff + 16u * nrow), 0, kStreamNorms);
-                t.n[0][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
-                t.n[1][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)(noff + 16u * nrow), 0, kStreamNorms);
-            }
+            // (every lane asks, also those that own no token: they repeat a neighbour's address)
+            __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + (long long)tile * nrow, pages * (int)nrow);
+            __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + (long long)tile * nrow, pages * (int)nrow);
+            t.n[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
+            t.n[1][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)(noff + 16u * nrow), 0, kStreamNorms);
+            t.n[0][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
+            t.n[1][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)(noff + 16u * nrow), 0, kStreamNorms);
         }
     };
 
     // One tile of loads is in flight per wave; each register set is re-issued for the next tile as soon as its
     // contents have been expanded.
     PairTileRegs t;
-    t.n[0][0] = t.n[0][1] = t.n[1][0] = t.n[1][1] = 0u;
     auto issue_first = [&]() {
-        int pg0 = 0;
+        int pg0 = PAGED ? 0 : tile_rows(t0);
         if (PAGED) {
             pg0 = fetch_pages(t0);
             pages_next = fetch_pages(t0 + 32);
@@ -265,8 +263,14 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
                 pages = pages_next;                                  // the next tile's pages, already here
                 if (more) pages_next = fetch_pages(tile + 64);       // and the one after: before the next tile's loads
             }
-            pair_scan_tile<R>(L, S, t, tile, n, [&]() { if (more) issue_k(t, tile + 32, pages); },
-                              [&]() { if (more) issue_n(t, tile + 32, pages); }, [&]() { if (more) issue_v(t, tile + 32, pages); });
+            if (PAGED) {
+                pair_scan_tile<R>(L, S, t, tile, n, [&]() { if (more) issue_k(t, tile + 32, pages); },
+                                  [&]() { if (more) issue_n(t, tile + 32, pages); }, [&]() { if (more) issue_v(t, tile + 32, pages); });
+            } else {
+                const int rows = more ? tile_rows(tile + 32) : 0;
+                pair_scan_tile<R>(L, S, t, tile, n, [&]() { issue_k(t, tile + 32, rows); }, [&]() { issue_n(t, tile + 32, rows); },
+                                  [&]() { issue_v(t, tile + 32, rows); });
+            }
         }
 
         // ---- partial results of this (sequence, pair of KV heads, chunk)

@@ -398,22 +398,26 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         const uint32_t koff = L.koff_rows * kvp + L.koff_bytes;
         const uint32_t voff = L.voff_rows * kvp + L.voff_bytes;
         const uint32_t noff = (uint32_t)L.tok0 * nrow;
+        // the sequence's rows of this pair: a tile is one multiplication per array away
         const long long seq_row0 = (long long)g * a.seq_stride_rows;
-        const char* kpair = reinterpret_cast<const char*>(a.k) + (long long)h * kHeadBytes;
-        const char* vpair = reinterpret_cast<const char*>(a.v) + (long long)h * kHeadBytes;
-        const char* knpair = reinterpret_cast<const char*>(a.k_norms) + (long long)h * 2;
-        const char* vnpair = reinterpret_cast<const char*>(a.v_norms) + (long long)h * 2;
-        // (loads of a tile index past the wave's last one are given an empty extent: they return zeros without touching memory)
-        auto tile_rows = [&](int i, int tile) -> int { return i < ntiles ? max(min(n - tile, 32), 0) : 0; };
-        auto issue_k = [&](PairTileRegs& t, int i) {
-            const int tile = tile_at(i);
-            __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (seq_row0 + tile) * kvp, tile_rows(i, tile) * (int)kvp);
+        const char* kpair = reinterpret_cast<const char*>(a.k) + seq_row0 * kvp + (long long)h * kHeadBytes;
+        const char* vpair = reinterpret_cast<const char*>(a.v) + seq_row0 * kvp + (long long)h * kHeadBytes;
+        const char* knpair = reinterpret_cast<const char*>(a.k_norms) + seq_row0 * nrow + (long long)h * 2;
+        const char* vnpair = reinterpret_cast<const char*>(a.v_norms) + seq_row0 * nrow + (long long)h * 2;
+        // The tile whose loads are issued during the current one: first token and rows that exist.  (Loads of a tile
+        // past the wave's last one get an empty extent: they return zeros without touching memory.)
+        int next_tile = 0, next_rows = 0;
+        auto set_next = [&](int i) {
+            next_tile = tile_at(i);
+            next_rows = i < ntiles ? max(min(n - next_tile, 32), 0) : 0;
+        };
+        auto issue_k = [&](PairTileRegs& t) {
+            __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (long long)next_tile * kvp, next_rows * (int)kvp);
 #pragma unroll
             for (int c = 0; c < 4; c++) t.k[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kStreamCodes);
         };
-        auto issue_v = [&](PairTileRegs& t, int i) {
-            const int tile = tile_at(i);
-            __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (seq_row0 + tile) * kvp, tile_rows(i, tile) * (int)kvp);
+        auto issue_v = [&](PairTileRegs& t) {
+            __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (long long)next_tile * kvp, next_rows * (int)kvp);
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
@@ -421,17 +425,15 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
                     t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kStreamCodes);
             }
         };
-        auto issue_n = [&](PairTileRegs& t, int i) {
-            const int tile = tile_at(i);
-            const int rows = tile_rows(i, tile);
-            __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
-            __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + (seq_row0 + tile) * nrow, rows * (int)nrow);
-            if (L.useful) {
-                t.n[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
-                t.n[1][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)(noff + 16u * nrow), 0, kStreamNorms);
-                t.n[0][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
-                t.n[1][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)(noff + 16u * nrow), 0, kStreamNorms);
-            }
+        // (every lane asks, also those that own no token: they repeat a neighbour's address, which costs nothing, and
+        // the loop has no branch here)
+        auto issue_n = [&](PairTileRegs& t) {
+            __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + (long long)next_tile * nrow, next_rows * (int)nrow);
+            __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + (long long)next_tile * nrow, next_rows * (int)nrow);
+            t.n[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
+            t.n[1][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)(noff + 16u * nrow), 0, kStreamNorms);
+            t.n[0][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
+            t.n[1][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)(noff + 16u * nrow), 0, kStreamNorms);
         };
 
         PairState<R> S;
@@ -440,17 +442,19 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         // the first tile asked for before the rotations, 0.4 us slower, as with one head per wave; the scores of tile
         // i + 1 placed beside the P.V of tile i for the scheduler to interleave, 3 % slower.)
         PairTileRegs t;
-        t.n[0][0] = t.n[0][1] = t.n[1][0] = t.n[1][1] = 0u;
         rotate_unit();
-        issue_k(t, 0);
-        issue_n(t, 0);
-        issue_v(t, 0);
+        set_next(0);
+        issue_k(t);
+        issue_n(t);
+        issue_v(t);
         load_rb();              // behind the first tile's loads; the registers are there, and the epilogue need not wait
         if (ntiles > 0) {
             S.load_query(L, [&](int i) -> const float* { return &qrot_s[hk_local * R + i][0]; });
-            for (int it = 0; it < ntiles; it++)
-                pair_scan_tile<R>(L, S, t, tile_at(it), n, [&]() { issue_k(t, it + 1); }, [&]() { issue_n(t, it + 1); },
-                                  [&]() { issue_v(t, it + 1); });
+            for (int it = 0; it < ntiles; it++) {
+                const int tile = next_tile;
+                set_next(it + 1);
+                pair_scan_tile<R>(L, S, t, tile, n, [&]() { issue_k(t); }, [&]() { issue_n(t); }, [&]() { issue_v(t); });
+            }
         }
         pair_scan_finish<R>(L, S, 1.0f / kAlpha, [&](int hd, int r, const float (&ov)[16]) {
             float* pr = &part_s[part * HKW + hk_local + hd][r][0];

@@ -14,11 +14,13 @@
 // kv_attention_mfma.hip.
 //
 // Layout of a tile in a wave (lane = (pn = lane % 16, pkg = lane / 16), hd = pn / 8 the head of the pair):
-//   loads    K: instruction c (0..3) covers tokens 8c .. 8c+7, lane l the 16-byte piece l % 8 of token l / 8 of the
-//            pair's 128-byte row.  V: lane (pn, pkg) loads 8 bytes (16 dims of head hd: dims 16 (pn % 8) ..) of tokens
+//   loads    K: instruction c (0..3) covers tokens 8c .. 8c+7 whole, and every lane asks for the piece it multiplies:
+//            lane (pn, pkg) the 16 bytes 16 (4 hd + pkg) .. of token 8c + pn % 8 of the pair's 128-byte row (an
+//            instruction that covers the same lines in address order and a ds_bpermute per dword to hand the pieces
+//            on costs 3 us of 104 at 64 x 8192 tokens: the scan has no LDS issue slots to spare).  V: lane (pn, pkg) loads 8 bytes (16 dims of head hd: dims 16 (pn % 8) ..) of tokens
 //            4 pkg + i and 16 + 4 pkg + i, i = 0..3.  Norms: 4 bytes (the pair's two fp16) of tokens tok0 and tok0 + 16.
-//   scores   MFMA set c: columns 0-7 = tokens 8c .. 8c+7 of the first head, columns 8-15 the same tokens of the second
-//            (one ds_bpermute per dword brings piece 4 hd + pkg of token pn % 8 to lane (pn, pkg)); the A operand holds
+//   scores   MFMA set c: columns 0-7 = tokens 8c .. 8c+7 of the first head, columns 8-15 the same tokens of the second;
+//            the A operand holds
 //            the query heads of both KV heads: row hd * R + r the fp16 value, row + 8 the rounding remainder.
 //   softmax  two permlane32 swaps per query head add value and remainder rows and leave lane (pn, pkg) with the scores
 //            of tokens tok0 = 8 (pkg / 2) + pn % 8 and tok0 + 16 of head hd (R = 4: lane groups of the other parity
@@ -40,25 +42,25 @@ template <int R>
 struct PairLane {
     int pn, pkg, hd;
     uint32_t lane_rep;      // byte offset of the lane's replica inside a table entry
-    int ksrc;               // ds_bpermute address: source lane of the K operand
     bool useful;            // owns two (token, head) pairs of every tile
     int tok0;               // the first of them (the other: tok0 + 16)
-    half_t* p_w;            // where its probabilities go in the wave's P tile (row hd * R, column of tok0)
+    half_t* p_w;            // where its probabilities go in the wave's P tile (row hd * R, column of tok0); with R = 2
+                            // the lanes that own nothing write their zeros to the spare rows 4-7 and 12-15 instead
+                            // of being masked off (four exec-mask regions less per tile)
     const uint4* p_r;       // its A operand of the P.V MFMAs
     const char* tab;        // the centroid table
-    uint32_t koff_rows, koff_bytes;   // K: row l / 8 and byte 16 (l % 8) inside a pair row
+    uint32_t koff_rows, koff_bytes;   // K: row pn % 8 and byte 16 (4 hd + pkg) inside a pair row
     uint32_t voff_rows, voff_bytes;   // V: row 4 pkg and byte 8 pn
 
     __device__ __forceinline__ void init(int lane, half_t (*p_tile)[32], const uint32_t* table) {
         pn = lane & 15; pkg = lane >> 4; hd = pn >> 3;
         lane_rep = (uint32_t)lane * 4u;
-        ksrc = 4 * (8 * (pn & 7) + 4 * hd + pkg);
         useful = R == 4 ? ((pkg & 1) == hd) : ((pkg & 1) == 0);
         tok0 = 8 * (pkg >> 1) + (pn & 7);
-        p_w = &p_tile[hd * R][8 * (tok0 >> 2) + (tok0 & 3)];
+        p_w = &p_tile[hd * R + ((R == 2 && !useful) ? 4 : 0)][8 * (tok0 >> 2) + (tok0 & 3)];
         p_r = reinterpret_cast<const uint4*>(&p_tile[pn][8 * pkg]);
         tab = reinterpret_cast<const char*>(table);
-        koff_rows = (uint32_t)(lane >> 3); koff_bytes = 16u * (uint32_t)(lane & 7);
+        koff_rows = (uint32_t)(pn & 7); koff_bytes = 16u * (uint32_t)(4 * hd + pkg);
         voff_rows = (uint32_t)(4 * pkg); voff_bytes = 8u * (uint32_t)pn;
     }
     __device__ __forceinline__ uint32_t lut32(uint32_t addr) const { return *reinterpret_cast<const uint32_t*>(tab + addr); }
@@ -131,7 +133,7 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
         union { uint32_t u[4]; half8_t h; } kv[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint32_t w = (uint32_t)__builtin_amdgcn_ds_bpermute(L.ksrc, (int)t.k[c][j]);
+            const uint32_t w = t.k[c][j];
             kv[j].u[0] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0400u));
             kv[j].u[1] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0500u));
             kv[j].u[2] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0600u));
@@ -198,7 +200,7 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
             const float pf = pe * vn[i];                            // (s * vn) * centroid, kernels.cu:1765
             const half_t hi = (half_t)pf;
             const half_t lo = (half_t)(pf - (float)hi);
-            if (L.useful) {
+            if (R == 2 || L.useful) {
                 L.p_w[r * 32 + 4 * i] = hi;
                 L.p_w[(r + 8) * 32 + 4 * i] = lo;
             }
