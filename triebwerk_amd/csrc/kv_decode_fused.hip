@@ -438,9 +438,11 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
 
         PairState<R> S;
         S.reset();
-        // One tile of loads in flight per wave.  (Tried: two tiles, 2 % slower -- the wave is not waiting for memory;
-        // the first tile asked for before the rotations, 0.4 us slower, as with one head per wave; the scores of tile
-        // i + 1 placed beside the P.V of tile i for the scheduler to interleave, 3 % slower.)
+        // One tile of loads in flight per wave.  (Tried: two tiles, 2 % slower; a second register set for K alone, whose
+        // loads otherwise have only the softmax and P.V of one tile to arrive in, 6 % slower -- more requests in flight
+        // make the memory slower here, not faster; the first tile asked for before the rotations, 0.4 us slower, as
+        // with one head per wave; the scores of tile i + 1 placed beside the P.V of tile i for the scheduler to
+        // interleave, 3 % slower.)
         PairTileRegs t;
         rotate_unit();
         set_next(0);
