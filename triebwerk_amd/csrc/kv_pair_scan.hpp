@@ -21,10 +21,12 @@
 //            4 pkg + i and 16 + 4 pkg + i, i = 0..3.  Norms: 4 bytes (the pair's two fp16) of tokens tok0 and tok0 + 16.
 //   scores   MFMA set c: columns 0-7 = tokens 8c .. 8c+7 of the first head, columns 8-15 the same tokens of the second;
 //            the A operand holds
-//            the query heads of both KV heads: row hd * R + r the fp16 value, row + 8 the rounding remainder.
+//            the query heads of both KV heads: row 4 hd + r the fp16 value, row + 8 the rounding remainder.  A lane's
+//            accumulator registers are the rows 4 pkg + i, so the first head's scores arrive in lane groups 0 (values)
+//            and 2 (remainders), the second head's in groups 1 and 3, register r in both: no per-lane choice of a register.
 //   softmax  two permlane32 swaps per query head add value and remainder rows and leave lane (pn, pkg) with the scores
-//            of tokens tok0 = 8 (pkg / 2) + pn % 8 and tok0 + 16 of head hd (R = 4: lane groups of the other parity
-//            hold the other head's rows and own nothing).
+//            of tokens tok0 = 8 (pkg / 2) + pn % 8 and tok0 + 16 of head hd; the lanes whose group holds the other
+//            head's rows (pkg % 2 != hd) own nothing.
 //   P.V      the probabilities times the V norms go through the wave's 1 KB LDS tile into A-operand order (rows as
 //            above); MFMA j: columns 0-7 = dim 16 (pn % 8) + j of the first head, 8-15 of the second.
 // A product of a row with a column of the other head is computed and never used.
@@ -44,8 +46,8 @@ struct PairLane {
     uint32_t lane_rep;      // byte offset of the lane's replica inside a table entry
     bool useful;            // owns two (token, head) pairs of every tile
     int tok0;               // the first of them (the other: tok0 + 16)
-    half_t* p_w;            // where its probabilities go in the wave's P tile (row hd * R, column of tok0); with R = 2
-                            // the lanes that own nothing write their zeros to the spare rows 4-7 and 12-15 instead
+    half_t* p_w;            // where its probabilities go in the wave's P tile (row 4 hd, column of tok0); with R < 4
+                            // the lanes that own nothing write their zeros to the spare rows 4 hd + R + r instead
                             // of being masked off (four exec-mask regions less per tile)
     const uint4* p_r;       // its A operand of the P.V MFMAs
     const char* tab;        // the centroid table
@@ -55,9 +57,9 @@ struct PairLane {
     __device__ __forceinline__ void init(int lane, half_t (*p_tile)[32], const uint32_t* table) {
         pn = lane & 15; pkg = lane >> 4; hd = pn >> 3;
         lane_rep = (uint32_t)lane * 4u;
-        useful = R == 4 ? ((pkg & 1) == hd) : ((pkg & 1) == 0);
+        useful = (pkg & 1) == hd;
         tok0 = 8 * (pkg >> 1) + (pn & 7);
-        p_w = &p_tile[hd * R + ((R == 2 && !useful) ? 4 : 0)][8 * (tok0 >> 2) + (tok0 & 3)];
+        p_w = &p_tile[4 * hd + ((R < 4 && !useful) ? R : 0)][8 * (tok0 >> 2) + (tok0 & 3)];
         p_r = reinterpret_cast<const uint4*>(&p_tile[pn][8 * pkg]);
         tab = reinterpret_cast<const char*>(table);
         koff_rows = (uint32_t)(pn & 7); koff_bytes = 16u * (uint32_t)(4 * hd + pkg);
@@ -100,10 +102,10 @@ struct PairState {
     // q_rot of the pair's query heads: row(i) -> the 128 floats of query head i (i = hd * R + r, 0 <= i < 2 R)
     template <class RowOf>
     __device__ __forceinline__ void load_query(const PairLane<R>& L, RowOf row_of) {
-        const int m = L.pn & 7;
+        const int m = L.pn & 7;                                // operand row m (and m + 8): head m / 4, query head m % 4
         const bool lo_part = (L.pn & 8) != 0;
-        const bool live = m < 2 * R;
-        const float* qr = row_of(live ? m : 0) + 32 * L.pkg;
+        const bool live = (m & 3) < R;
+        const float* qr = row_of(live ? (m >> 2) * R + (m & 3) : 0) + 32 * L.pkg;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             float4 v0 = *reinterpret_cast<const float4*>(qr + 8 * j);
@@ -158,11 +160,10 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
     bool raise = false;
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        // the row of (hd, r): hd * R + r; rows 0-3 sit in lane group 0 (R = 4: the second head's in group 1), their
-        // remainders 32 lanes further on
+        // the row of (hd, r) is 4 hd + r: register r of lane group hd, its remainder 32 lanes further on
         float v[4];
 #pragma unroll
-        for (int c = 0; c < 4; c++) v[c] = R == 4 ? s[c][r] : (L.hd ? s[c][R + r] : s[c][r]);
+        for (int c = 0; c < 4; c++) v[c] = s[c][r];
         uint32x2_t s01 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[1]), false, false);
         uint32x2_t s23 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[2]), __float_as_uint(v[3]), false, false);
         raw[0][r] = (__uint_as_float(s01[0]) + __uint_as_float(s01[1])) * kn[0];    // kernels.cu:1707
@@ -183,12 +184,9 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
             S.l_run[r] *= alpha;
 #pragma unroll
             for (int i = 0; i < 2; i++) x[i][r] = valid[i] ? raw[i][r] - m_new : kNegBig;
-            // accumulator register i of a lane is row 4 pkg + i: query head i % R (of either KV head)
+            // accumulator register r of a lane is row 4 pkg + r: query head r (of either KV head, value or remainder)
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
-#pragma unroll
-                for (int i = r; i < 4; i += R) S.o[j][i] *= alpha;
-            }
+            for (int j = 0; j < 16; j++) S.o[j][r] *= alpha;
         }
     }
 #pragma unroll
@@ -200,7 +198,7 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
             const float pf = pe * vn[i];                            // (s * vn) * centroid, kernels.cu:1765
             const half_t hi = (half_t)pf;
             const half_t lo = (half_t)(pf - (float)hi);
-            if (R == 2 || L.useful) {
+            if (R < 4 || L.useful) {
                 L.p_w[r * 32 + 4 * i] = hi;
                 L.p_w[(r + 8) * 32 + 4 * i] = lo;
             }
@@ -250,14 +248,14 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
 // 1 / alpha applied); all lanes end with l_run summed over the head.
 template <int R, class Sink>
 __device__ __forceinline__ void pair_scan_finish(const PairLane<R>& L, PairState<R>& S, float inv_alpha, Sink sink) {
-    const int khi = R == 4 ? L.hd : 0;                          // lane group that holds the rows of head hd
+    const int khi = L.hd;                                       // lane group that holds the rows of head hd
 #pragma unroll
     for (int r = 0; r < R; r++) {
         S.l_run[r] = L.head_sum(S.l_run[r]);
         float ov[16];
 #pragma unroll
         for (int j = 0; j < 16; j++) {
-            float v = R == 4 ? S.o[j][r] : (L.hd ? S.o[j][R + r] : S.o[j][r]);
+            float v = S.o[j][r];
             ov[j] = (v + __shfl_xor(v, 32, 64)) * inv_alpha;
         }
         if (L.pkg == khi) sink(L.hd, r, ov);
