@@ -43,6 +43,7 @@ constexpr uint32_t kPairRowBytes = 128;      // two 4-bit heads of one token
 template <int R>
 struct PairLane {
     int pn, pkg, hd;
+    uint32_t nshift;        // 16 hd: where this lane's head sits in a dword of two fp16 norms
     uint32_t lane_rep;      // byte offset of the lane's replica inside a table entry
     bool useful;            // owns two (token, head) pairs of every tile
     int tok0;               // the first of them (the other: tok0 + 16)
@@ -56,6 +57,7 @@ struct PairLane {
 
     __device__ __forceinline__ void init(int lane, half_t (*p_tile)[32], const uint32_t* table) {
         pn = lane & 15; pkg = lane >> 4; hd = pn >> 3;
+        nshift = 16u * (uint32_t)hd;
         lane_rep = (uint32_t)lane * 4u;
         useful = (pkg & 1) == hd;
         tok0 = 8 * (pkg >> 1) + (pn & 7);
@@ -151,8 +153,8 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
     float kn[2], vn[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        kn[i] = h2f_bits(L.hd ? (t.n[i][0] >> 16) : (t.n[i][0] & 0xffffu));
-        vn[i] = h2f_bits(L.hd ? (t.n[i][1] >> 16) : (t.n[i][1] & 0xffffu));
+        kn[i] = h2f_bits((t.n[i][0] >> L.nshift) & 0xffffu);
+        vn[i] = h2f_bits((t.n[i][1] >> L.nshift) & 0xffffu);
     }
     after_n();
     const bool valid[2] = {L.useful && (tile + L.tok0 < n), L.useful && (tile + L.tok0 + 16 < n)};
