@@ -346,6 +346,7 @@ def paged_bench(args):
     rc = lib.tw_kv_debug_profile_read(C.byref(total_ms), C.byref(launches))
     lib.tw_kv_debug_profile_attention(0)
     assert rc == 0 and launches.value == Kp * L, (rc, launches.value)
+    scan_kernel_name = lib.tw_kv_debug_last_scan_kernel().decode()       # what those launches ran
     n_tokens_prof = int(sum(int((pos_now + i + 1).sum()) for i in range(Kp)))
     kern_ms = total_ms.value / launches.value
     launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=False) / (Kp * L)
@@ -364,6 +365,7 @@ def paged_bench(args):
         "step_algorithmic_GB": step_bytes * 1e-9, "step_achieved_GBps": step_gbs,
         "step_frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": "paged decode attention (context scan), one launch per layer",
+                     "kernel_name": scan_kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "launch_ms": kern_ms, "launch_algorithmic_MB": launch_bytes * 1e-6, "traffic": None},
     }))
@@ -457,7 +459,7 @@ def compact(r):
     """The figures of one cache width for the per_kv_bits table."""
     return {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "step_achieved_GBps": r["step_achieved_GBps"],
             "step_frac_of_hbm_peak": r["step_frac_of_hbm_peak"], "dtype": r["dtype"], "launches_per_layer": r["config"]["launches_per_layer"],
-            "roofline": {k: r["roofline"][k] for k in ("kernel", "achieved", "frac", "launch_ms", "launch_ms_timed", "launch_algorithmic_MB",
+            "roofline": {k: r["roofline"][k] for k in ("kernel", "kernel_name", "achieved", "frac", "launch_ms", "launch_ms_timed", "launch_algorithmic_MB",
                                                        "traffic", "traffic_source")}}
 
 
@@ -643,6 +645,7 @@ def decode_bench(args, kv_bits, with_probe):
     rc = lib.tw_kv_debug_profile_read(C.byref(total_ms), C.byref(launches))
     lib.tw_kv_debug_profile_attention(0)
     assert rc == 0 and launches.value == Kp * L, (rc, launches.value)
+    scan_kernel_name = lib.tw_kv_debug_last_scan_kernel().decode()       # what those launches ran
     n_tokens_prof = int(sum(int((pos_now + i + 1).sum()) for i in range(Kp)))
     eager_kern_ms = total_ms.value / launches.value
     # which kernel those launches were: the whole layer step in one launch (append included), or the scan of the
@@ -728,6 +731,7 @@ def decode_bench(args, kv_bits, with_probe):
             "bound": "hbm",
             "kernel": ("decode step of a layer in one launch (append, query rotation, context scan, merge, rotate-back)"
                        if one_launch else "decode attention (context scan), one launch per layer"),
+            "kernel_name": scan_kernel_name,
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -180,6 +180,11 @@ void tw_kv_debug_set_decode_fused(int mode);
  * summed duration and the launch count.  Reading waits for the recorded launches and resets the counter. */
 void tw_kv_debug_profile_attention(int enable);
 int tw_kv_debug_profile_read(double* total_ms, int* launches);
+/* Name of the kernel that the last attention call of this process launched (or recorded into a graph) for the
+ * context: "attention_pair_kernel", "attention_mfma_kernel", "attention_mfma2c_kernel", "attention_valu_kernel",
+ * "decode_fused_kernel, two KV heads per wave", "decode_fused_kernel, one KV head per wave", a prefill kernel, or
+ * "none".  A static string; lets a benchmark name the kernel its figures belong to. */
+const char* tw_kv_debug_last_scan_kernel(void);
 
 /* One launch or three for a layer's decode step over the compressed cache, as a pure function of what the host
  * knows (1 = one launch, 0 = three): G sequences,

@@ -59,6 +59,7 @@ SIGNATURES = {
     "tw_kv_debug_set_num_splits": (None, [I]),
     "tw_kv_debug_set_prefill_form": (None, [I]),
     "tw_kv_debug_set_decode_fused": (None, [I]),
+    "tw_kv_debug_last_scan_kernel": (C.c_char_p, []),
     "tw_kv_decode_fused_launches": (LL, []),
     "tw_kv_decode_step_plan": (I, [I, I, I, I, I, I, I]),
     "tw_kv_debug_profile_attention": (None, [I]),

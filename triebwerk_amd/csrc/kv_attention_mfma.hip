@@ -710,6 +710,7 @@ bool launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
     }
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3(grid), b3(ngroups * waves * kWave);
+    note_scan_kernel("attention_mfma_kernel");
 #define TW_LAUNCH(P, RR, BB) launch_scan_kernel(attention_mfma_kernel<P, RR, BB, (BB == 4 ? kDepth4 : kDepth2)>, g3, b3, s, a, items, hgroups, waves)
 #define TW_LAUNCH_R(P, BB) \
     do { if (R == 1) TW_LAUNCH(P, 1, BB); else if (R == 2) TW_LAUNCH(P, 2, BB); else TW_LAUNCH(P, 4, BB); } while (0)

@@ -447,6 +447,7 @@ void launch_attention_mfma2c_scan(const AttnArgs& a, hipStream_t s) {
     }
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3(grid), b3(ngroups * kCoopHeads * kWave);
+    note_scan_kernel("attention_mfma2c_kernel");
 #define TW_LAUNCH_C(P, RR) launch_scan_kernel(attention_mfma2c_kernel<P, RR>, g3, b3, s, a, items)
     if (a.block_table) {
         if (R == 1) TW_LAUNCH_C(true, 1); else if (R == 2) TW_LAUNCH_C(true, 2); else TW_LAUNCH_C(true, 4);

@@ -325,6 +325,7 @@ void launch_attention_pair_scan(const AttnArgs& a, hipStream_t s) {
     }
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3(grid), b3(ngroups * waves * kWave);
+    note_scan_kernel("attention_pair_kernel");
 #define TW_LAUNCH(P, RR) launch_scan_kernel(attention_pair_kernel<P, RR>, g3, b3, s, a, items, hgroups, waves)
 #define TW_LAUNCH_R(P) do { if (R == 1) TW_LAUNCH(P, 1); else if (R == 2) TW_LAUNCH(P, 2); else TW_LAUNCH(P, 4); } while (0)
     if (a.block_table) TW_LAUNCH_R(true); else TW_LAUNCH_R(false);

@@ -340,6 +340,7 @@ static void launch_valu_mode(const AttnArgs& a, hipStream_t s) {
 
 void launch_attention_valu(const AttnArgs& a, hipStream_t s) {
     if (a.G <= 0) return;
+    note_scan_kernel("attention_valu_kernel");
     if (a.bits == 0) launch_valu_mode<0>(a, s);
     else if (a.bits == 4) launch_valu_mode<4>(a, s);
     else launch_valu_mode<2>(a, s);

@@ -24,6 +24,7 @@ static std::atomic<int> g_prefill_form{0};   // test hook, see prefill_form()
 int prefill_form() { return g_prefill_form.load(); }
 static std::atomic<int> g_attention_variant{0};   // tw_kv_debug_set_attention_variant, see attention_variant()
 int attention_variant() { return g_attention_variant.load(); }
+const char* volatile g_last_scan_kernel = "none";
 thread_local hipEvent_t t_scan_start = nullptr;
 thread_local hipEvent_t t_scan_stop = nullptr;
 }  // namespace twkv
@@ -215,6 +216,7 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
     return tokens <= ((bits == 2 && num_kv_heads == 8) ? (256LL << 10) : (1LL << 20)) ? 1 : 0;
 }
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }
+const char* tw_kv_debug_last_scan_kernel(void) { return twkv::g_last_scan_kernel; }
 
 void tw_kv_debug_profile_attention(int enable) {
     g_prof.enabled.store(enable);

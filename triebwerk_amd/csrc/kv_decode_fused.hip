@@ -770,6 +770,7 @@ void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s
     const bool pair = allow_pairs && decode_fused_pairs(a, f.hkw);
     const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw))), b3((pair ? kPairWaves : kFusedWaves) * kWave);
     const bool prod = f.q_weight != nullptr || f.cos_table != nullptr;
+    note_scan_kernel(pair ? "decode_fused_kernel, two KV heads per wave" : "decode_fused_kernel, one KV head per wave");
 #define TW_FUSED(RR, BB, PP) \
     do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true, PP>, g3, b3, s, a, f); \
          else launch_scan_kernel(decode_fused_kernel<RR, BB, false, PP>, g3, b3, s, a, f); } while (0)

@@ -16,6 +16,10 @@ namespace twkv {
 // duration without the gaps an event recorded before and after a launch would add.
 extern thread_local hipEvent_t t_scan_start;
 extern thread_local hipEvent_t t_scan_stop;
+// Name of the kernel the last attention launch of this process used for the context (tw_kv_debug_last_scan_kernel):
+// every launch function below records its own.
+extern const char* volatile g_last_scan_kernel;
+inline void note_scan_kernel(const char* name) { g_last_scan_kernel = name; }
 template <typename... Args, typename F = void (*)(Args...)>
 inline void launch_scan_kernel(F kernel, dim3 grid, dim3 block, hipStream_t s, Args... args) {
     if (t_scan_start) hipExtLaunchKernelGGL(kernel, grid, block, 0, s, t_scan_start, t_scan_stop, 0, args...);

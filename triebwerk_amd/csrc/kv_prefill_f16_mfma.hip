@@ -288,6 +288,7 @@ void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form) {
     const int tpw = 16 * nq * kPfWaves / R;
     const int nblk = (T + tpw - 1) / tpw;
     const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(kPfWaves * kWave);
+    note_scan_kernel("prefill_f16_mfma_kernel");
 #define TW_PF_LAUNCH(RR, NN, MM) launch_scan_kernel(prefill_f16_mfma_kernel<RR, NN, MM>, grid, block, s, a, T)
 #define TW_PF_MODES(RR) \
     do { if (mode == 1) TW_PF_LAUNCH(RR, 1, false); else if (mode == 2) TW_PF_LAUNCH(RR, 1, true); \

@@ -540,6 +540,7 @@ void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s) {
     if (tiles < (long long)grid * ngroups) grid = (int)((tiles + ngroups - 1) / ngroups);
     if (grid < 1) grid = 1;
     const dim3 g3(grid), b3(ngroups * waves * kWave);
+    note_scan_kernel("prefill_mfma_kernel");
 #define TW_LAUNCH_P(RR, BB) launch_scan_kernel(prefill_mfma_kernel<RR, BB>, g3, b3, s, a, waves)
     if (a.bits == 4) {
         if (R == 1) TW_LAUNCH_P(1, 4); else if (R == 2) TW_LAUNCH_P(2, 4); else TW_LAUNCH_P(4, 4);

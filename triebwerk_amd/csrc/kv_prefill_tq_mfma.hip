@@ -413,6 +413,7 @@ void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form) {
     const int tpw = 16 * nq * kPtWaves / R;
     const int nblk = (T + tpw - 1) / tpw;
     const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(kPtWaves * kWave);
+    note_scan_kernel("prefill_tq_mfma_kernel");
 #define TW_PT_LAUNCH(RR, BB, NN, MM) launch_scan_kernel(prefill_tq_mfma_kernel<RR, BB, NN, MM>, grid, block, s, a, T)
 #define TW_PT_MODES(RR, BB) \
     do { if (mode == 1) TW_PT_LAUNCH(RR, BB, 1, false); else if (mode == 2) TW_PT_LAUNCH(RR, BB, 1, true); \
