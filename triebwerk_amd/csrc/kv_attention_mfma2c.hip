@@ -309,6 +309,9 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
                 }
             }
 
+            // (wave priority rises through the tile, as in kv_pair_scan.hpp: 1 % here, where a barrier per tile
+            // keeps the waves closer together anyway)
+            __builtin_amdgcn_s_setprio(1);
             // ---- online softmax (base 2): this lane owns token ln of sub-tile my_sub
             const float kn = h2f_bits(*reinterpret_cast<const uint16_t*>(&nn_s[grp][buf][0][nro]));
             const float vn = h2f_bits(*reinterpret_cast<const uint16_t*>(&nn_s[grp][buf][1][nro]));
@@ -355,6 +358,7 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             __builtin_amdgcn_wave_barrier();
 
+            __builtin_amdgcn_s_setprio(2);
             // ---- O[head][dim 8ln + j] += P[head][token] V[token][dim]
             // Per sub-tile: wa = 16-bit codes of tokens (4kg, 4kg+2), wb = of (4kg+1, 4kg+3) for
             // this lane's 8 dims.  xe/xo: per byte, low nibble = token a dims (d, d+1), high
@@ -386,6 +390,7 @@ attention_mfma2c_kernel(AttnArgs a, int total_items) {
                 o[2 * q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, be.h, o[2 * q], 0, 0, 0);
                 o[2 * q + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, o[2 * q + 1], 0, 0, 0);
             }
+            __builtin_amdgcn_s_setprio(0);
         };
         // One tile: start the loads of the next tile, do the arithmetic of tile `it` from LDS, put the
         // tile that arrived into the other buffer, and meet the other waves.  (Two tiles of loads in

@@ -148,6 +148,10 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
         for (int j = 0; j < 4; j++) s[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(S.aq[j], kv[j].h, s[c], 0, 0, 0);
     }
     after_k();
+    // Wave priority rises as the tile advances (scores 0, softmax 1, P.V 2): of the two waves of a SIMD the one
+    // that is further along issues first, finishes its tile and puts its next loads on the way.  2.5 % at
+    // 64 x 8192 tokens; raising it for the scores, or for scores and P.V alike, gains nothing.
+    __builtin_amdgcn_s_setprio(1);
 
     // ---- online softmax (base 2): this lane owns tokens tok0 and tok0 + 16 of head hd
     float kn[2], vn[2];
@@ -213,6 +217,7 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
+    __builtin_amdgcn_s_setprio(2);
     // ---- O[row][dim 16 (pn % 8) + j of head pn / 8] += P[row][token] V[token][dim]
     uint32_t xe[2][4], xo[2][4];
 #pragma unroll
@@ -243,6 +248,7 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
             S.o[8 * dw + 2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, S.o[8 * dw + 2 * jp + 1], 0, 0, 0);
         }
     }
+    __builtin_amdgcn_s_setprio(0);
 }
 
 // The wave's partial result per (head of the pair, query head): sink(hd, r, dims) is called by the 16 lanes that
