@@ -26,6 +26,7 @@
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
+#include "kv_mfma_util.hpp"
 
 namespace twkv {
 
@@ -33,13 +34,7 @@ constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / kWave;
 // lanes that own one token, and the values of its head each of them holds
 template <int MODE> struct LanesPerToken { static constexpr int value = MODE == 0 ? 8 : 4; };
-constexpr float kNegBig = -1e30f;                // the reference's max init (kernels.cu:1686)
-
-__device__ __forceinline__ int seq_pos(const AttnArgs& a, int g) {
-    if (a.pos_mode == kPosArray) return a.positions[g];
-    if (a.pos_mode == kPosScalar) return a.pos_scalar;
-    return g;
-}
+// (kNegBig, the reference's max init of kernels.cu:1686, and seq_pos come from kv_mfma_util.hpp)
 
 // Dimension owned by element e of lane c of a token's lanes.
 template <int MODE>
@@ -58,9 +53,7 @@ __device__ __forceinline__ void load_vals(const void* __restrict__ base, long lo
         const half_t* p = reinterpret_cast<const half_t*>(base) + (row * num_kv_heads + h) * kHeadDim;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            // the eight lanes of a token take one whole line per instruction: non-temporal
-            half8_t h8 = fresh ? *reinterpret_cast<const half8_t*>(fresh + 64 * j + 8 * c)
-                               : __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(p + 64 * j + 8 * c));
+            half8_t h8 = *reinterpret_cast<const half8_t*>((fresh ? fresh : p) + 64 * j + 8 * c);
 #pragma unroll
             for (int i = 0; i < 8; i++) vals[8 * j + i] = (float)h8[i];
         }
@@ -133,6 +126,36 @@ attention_valu_kernel(AttnArgs a) {
     chunk_range(n, chunk, a.nsplit, t0, t1);
     if (t0 >= t1) return;                       // uniform for the workgroup
 
+    // fp16 rows of a contiguous cache come in through buffer loads with the non-temporal hint (the eight lanes of a
+    // token take one whole 128-byte line per instruction; written as an ordinary load beside the load of the appended
+    // row the compiler folds the two into one load of a selected pointer and the hint is gone): a descriptor over
+    // this sequence's rows of head h up to the chunk's end, 32-bit offsets inside it
+    const uint32_t rowbytes = (uint32_t)a.num_kv_heads * kHeadDim * 2;
+    const bool nt_rows = MODE == 0 && !a.block_table && (long long)t1 * rowbytes < (1LL << 31);
+    __amdgpu_buffer_rsrc_t krs, vrs;
+    if (MODE == 0) {
+        const long long first = ((long long)g * a.seq_stride_rows * a.num_kv_heads + h) * kHeadDim * 2;
+        krs = make_rsrc(reinterpret_cast<const char*>(a.k) + first, nt_rows ? t1 * (int)rowbytes : 0);
+        vrs = make_rsrc(reinterpret_cast<const char*>(a.v) + first, nt_rows ? t1 * (int)rowbytes : 0);
+    }
+    auto load_row_nt = [&](__amdgpu_buffer_rsrc_t rs, int t, const half_t* fresh_row, float* vals) {
+        const uint32_t off = (uint32_t)t * rowbytes + 16u * (uint32_t)c;
+        uint32x4_t w[2];
+        w[0] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, kStreamCodes);
+        w[1] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(off + 128u), 0, kStreamCodes);
+        if (fresh_row) {                               // the token being appended: its row is not in the cache yet
+            w[0] = *reinterpret_cast<const uint32x4_t*>(fresh_row + 8 * c);
+            w[1] = *reinterpret_cast<const uint32x4_t*>(fresh_row + 64 + 8 * c);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            union { uint32x4_t u; half8_t h; } cv;
+            cv.u = w[j];
+#pragma unroll
+            for (int i = 0; i < 8; i++) vals[8 * j + i] = (float)cv.h[i];
+        }
+    };
+
     if (tid < 16) cent_s[tid] = (MODE == 2) ? kCentroids2[tid & 3] : kCentroids4[tid];
     const half_t* k_fresh = nullptr;
     const half_t* v_fresh = nullptr;
@@ -196,7 +219,8 @@ attention_valu_kernel(AttnArgs a) {
         }
         float vals[E];
         const bool fresh = APPEND && tc == n - 1;
-        load_vals<MODE>(a.k, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? k_fresh : nullptr);
+        if (MODE == 0 && nt_rows) load_row_nt(krs, tc, fresh ? k_fresh : nullptr, vals);
+        else load_vals<MODE>(a.k, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? k_fresh : nullptr);
         float s[RT];
 #pragma unroll
         for (int r = 0; r < RT; r++) {
@@ -207,7 +231,8 @@ attention_valu_kernel(AttnArgs a) {
             for (int off = 1; off < LPT; off <<= 1) dot += __shfl_xor(dot, off, 64);
             s[r] = dot * (kn * scale);          // kernels.cu:1707
         }
-        load_vals<MODE>(a.v, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? v_fresh : nullptr);
+        if (MODE == 0 && nt_rows) load_row_nt(vrs, tc, fresh ? v_fresh : nullptr, vals);
+        else load_vals<MODE>(a.v, row, a.num_kv_heads, h, c, cent_s, vals, fresh ? v_fresh : nullptr);
         if (valid) {
 #pragma unroll
             for (int r = 0; r < RT; r++) {
