@@ -161,7 +161,8 @@ const char* tw_kv_build_info(void);
  * while no other thread is inside the library. */
 
 /* Compressed-attention kernel family: 0 = automatic, 1 = fp32 vector-ALU kernels, 2 = MFMA kernels, 3 = MFMA kernels
- * with one KV head per wave also where the 4-bit scan would give a wave two. */
+ * with one KV head per wave also where the scan would give a wave two, 4 = MFMA kernels with the cooperative 2-bit
+ * scan (8 KV heads, rows loaded by the workgroup together) where the default is two KV heads per wave. */
 void tw_kv_debug_set_attention_variant(int variant);
 int tw_kv_debug_get_attention_variant(void);
 /* Split count of decode attention (0 = automatic). */
@@ -190,7 +191,7 @@ const char* tw_kv_debug_last_scan_kernel(void);
  * knows (1 = one launch, 0 = three): G sequences,
  * cache width `bits`, max_seq_len, and the range of positions + 1 (ctx_max = 0: unknown).  One launch when every
  * wave gets at most 8 tiles of 32 tokens, or when the lengths are within 1/8 of each other, the batch gives at
- * least half the CUs a workgroup and the launch stays under ~1M tokens (256k at 2 bit with 8 KV heads).
+ * least half the CUs a workgroup and the launch stays under ~1M tokens (512k at 2 bit).
  * Alignment of the buffers, which the entry point also checks, is not part of it. */
 int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max);
 /* Layer steps that took the one-launch kernel since the library was loaded (launches issued or recorded into a

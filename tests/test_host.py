@@ -101,10 +101,13 @@ def test_decode_step_plan_is_the_documented_rule():
     from triebwerk_amd import _lib
     lib = _lib.load()
     plan = lib.tw_kv_decode_step_plan
-    # the benchmark's target: 64 sequences of 8192 tokens, lengths known and equal -> one launch at 4 bit,
-    # three at 2 bit (the cooperative 2-bit scan streams faster at that size)
+    # the benchmark's target: 64 sequences of 8192 tokens, lengths known and equal -> one launch at 4 bit; at 2 bit
+    # the three-kernel path has caught up at that size (512k tokens per launch; at 4 bit a million)
     assert plan(64, 16, 8, 4, 8448, 8192, 8192) == 1
     assert plan(64, 16, 8, 2, 8448, 8192, 8192) == 0
+    assert plan(64, 16, 8, 2, 8448, 8000, 8000) == 1
+    assert plan(128, 16, 8, 2, 8448, 8192, 8192) == 0
+    assert plan(128, 16, 8, 4, 8448, 8192, 8192) == 1
     # the same batch with nothing known about the lengths, or known to be ragged: three launches
     assert plan(64, 16, 8, 4, 8448, 0, 0) == 0
     assert plan(64, 16, 8, 4, 8448, 512, 8192) == 0

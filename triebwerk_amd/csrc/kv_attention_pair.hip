@@ -1,5 +1,5 @@
-// kv_attention_pair.hip -- the stand-alone context scan of GQA decode attention over the 4-bit compressed cache with
-// two KV heads per wave (gfx950).  Same mathematics, workspace and partials as attention_mfma_kernel
+// kv_attention_pair.hip -- the stand-alone context scan of GQA decode attention over the compressed cache (4 and 2 bit)
+// with two KV heads per wave (gfx950).  Same mathematics, workspace and partials as attention_mfma_kernel
 // (kv_attention_mfma.hip; kernels.cu:1641-1776 of the reference) and the same two ways of cutting the work -- even
 // chunks of every sequence, or the balanced walk over all tiles of a ragged batch -- but the tile is
 // kv_pair_scan.hpp's: a wave reads whole 128-byte lines (two heads) with non-temporal loads, so the waves of a
@@ -15,13 +15,14 @@ namespace twkv {
 
 namespace {
 constexpr int kPairScanWaves = 8;      // waves per workgroup: 256 registers each, one workgroup per CU (64 KB table)
-constexpr uint32_t kHeadBytes4 = 64;   // bytes of one 4-bit head in a cache row
 }  // namespace
 
-template <bool PAGED, int R>
+template <bool PAGED, int R, int BITS>
 __global__ void __launch_bounds__(kPairScanWaves * kWave)
 attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves) {
-    constexpr float kAlpha = kAlpha4;
+    constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
+    constexpr uint32_t kHeadBytes4 = BITS * 16;                      // bytes of one head in a cache row
+    constexpr int kCodesAux = BITS == 4 ? kStreamCodes : 0;          // whole lines per instruction only at 4 bit
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
     __shared__ __attribute__((aligned(16))) half_t p_s[kPairScanWaves][16][32];
     // balanced walk: tiles of the sequences before g, and {tiles per group, total tiles}
@@ -39,7 +40,7 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     const uint32_t kvp = (uint32_t)Hk * kHeadBytes4;   // bytes per cache row (all heads)
     const uint32_t nrow = (uint32_t)Hk * 2u;           // bytes per norm row
 
-    PairLane<R> L;
+    PairLane<R, BITS> L;
     L.init(lane, p_s[wave], tab_s);
     const uint32_t koff = L.koff_rows * kvp + L.koff_bytes;
     const uint32_t voff = L.voff_rows * kvp + L.voff_bytes;
@@ -103,27 +104,35 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     int pages_next = 0;                          // entries of the tile whose loads are issued next in the loop
     // `pages`: paged cache, the tile's two block-table entries; contiguous cache, the rows of the tile that exist
     auto tile_rows = [&](int tile) -> int { return max(min(n - tile, 32), 0); };
-    auto issue_k = [&](PairTileRegs& t, int tile, int pages) {
+    auto load_k = [&](__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        if constexpr (BITS == 4) return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kCodesAux);
+        else return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kCodesAux);
+    };
+    auto load_v = [&](__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        if constexpr (BITS == 4) return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kCodesAux);
+        else return __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, kCodesAux);
+    };
+    auto issue_k = [&](PairTileRegs<BITS>& t, int tile, int pages) {
         if (PAGED) {
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
                 __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + page_row(pages, sub) * kvp, kPageTokens * (int)kvp);
-                t.k[2 * sub] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)koff, 0, kStreamCodes);
-                t.k[2 * sub + 1] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + 8u * kvp), 0, kStreamCodes);
+                t.k[2 * sub] = load_k(r, koff);
+                t.k[2 * sub + 1] = load_k(r, koff + 8u * kvp);
             }
         } else {
             __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (long long)tile * kvp, pages * (int)kvp);
 #pragma unroll
-            for (int c = 0; c < 4; c++) t.k[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kStreamCodes);
+            for (int c = 0; c < 4; c++) t.k[c] = load_k(r, koff + (uint32_t)(8 * c) * kvp);
         }
     };
-    auto issue_v = [&](PairTileRegs& t, int tile, int pages) {
+    auto issue_v = [&](PairTileRegs<BITS>& t, int tile, int pages) {
         if (PAGED) {
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
                 __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + page_row(pages, sub) * kvp, kPageTokens * (int)kvp);
 #pragma unroll
-                for (int j = 0; j < 4; j++) t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)j * kvp), 0, kStreamCodes);
+                for (int j = 0; j < 4; j++) t.v[sub][j] = load_v(r, voff + (uint32_t)j * kvp);
             }
         } else {
             __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (long long)tile * kvp, pages * (int)kvp);
@@ -131,12 +140,12 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
             for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kStreamCodes);
+                    t.v[sub][j] = load_v(r, voff + (uint32_t)(16 * sub + j) * kvp);
             }
         }
     };
     // the pair's two fp16 norms of tokens tok0 and tok0 + 16, K and V
-    auto issue_n = [&](PairTileRegs& t, int tile, int pages) {
+    auto issue_n = [&](PairTileRegs<BITS>& t, int tile, int pages) {
         if (PAGED) {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
@@ -158,7 +167,7 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
 
     // One tile of loads is in flight per wave; each register set is re-issued for the next tile as soon as its
     // contents have been expanded.
-    PairTileRegs t;
+    PairTileRegs<BITS> t;
     auto issue_first = [&]() {
         int pg0 = PAGED ? 0 : tile_rows(t0);
         if (PAGED) {
@@ -216,9 +225,16 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     // ---- dequantization table, once per workgroup: entry e fills 256 bytes with replicas
     for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
         const int e = i >> 6;
-        half2_t pc = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
-        uint32_t w = *reinterpret_cast<uint32_t*>(&pc);
-        *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
+        if constexpr (BITS == 4) {
+            half2_t pc = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
+            uint32_t w = *reinterpret_cast<uint32_t*>(&pc);
+            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
+        } else {                                         // a byte's four centroids in their own order, 32 replicas of 8 bytes
+            half2_t p0 = {(half_t)(kAlpha * kCentroids2[e & 3]), (half_t)(kAlpha * kCentroids2[(e >> 2) & 3])};
+            half2_t p1 = {(half_t)(kAlpha * kCentroids2[(e >> 4) & 3]), (half_t)(kAlpha * kCentroids2[e >> 6])};
+            uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
+            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
+        }
     }
     for (int i = tid; i < kPairScanWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
     __syncthreads();             // the only workgroup-wide barrier; every wave reaches it
@@ -300,10 +316,10 @@ static int pair_scan_waves(const AttnArgs& a) {
 
 bool attention_pair_usable(const AttnArgs& a) {
     const int R = a.num_kv_heads > 0 ? a.num_heads / a.num_kv_heads : 0;
-    if (a.bits != 4 || (a.num_kv_heads & 1) != 0 || (R != 1 && R != 2 && R != 4)) return false;
+    if ((a.bits != 4 && a.bits != 2) || (a.num_kv_heads & 1) != 0 || (R != 1 && R != 2 && R != 4)) return false;
     if (a.pos_mode == kPosIota || !a.ws || !a.qrot) return false;
     auto al = [](const void* p, unsigned m) { return (reinterpret_cast<uintptr_t>(p) & m) == 0; };
-    if (!al(a.k, 15) || !al(a.v, 15) || !al(a.k_norms, 3) || !al(a.v_norms, 3)) return false;
+    if (!al(a.k, a.bits == 4 ? 15 : 7) || !al(a.v, a.bits == 4 ? 15 : 7) || !al(a.k_norms, 3) || !al(a.v_norms, 3)) return false;
     if (!al(a.ws, 15) || (a.ws_stride & 3) != 0) return false;       // 16-byte stores of the partials
     const long long items = (long long)a.G * a.nsplit * (a.num_kv_heads / (2 * pair_scan_waves(a)));
     return items > 0 && items <= 0x7fffffff;
@@ -326,9 +342,10 @@ void launch_attention_pair_scan(const AttnArgs& a, hipStream_t s) {
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3(grid), b3(ngroups * waves * kWave);
     note_scan_kernel("attention_pair_kernel");
-#define TW_LAUNCH(P, RR) launch_scan_kernel(attention_pair_kernel<P, RR>, g3, b3, s, a, items, hgroups, waves)
-#define TW_LAUNCH_R(P) do { if (R == 1) TW_LAUNCH(P, 1); else if (R == 2) TW_LAUNCH(P, 2); else TW_LAUNCH(P, 4); } while (0)
-    if (a.block_table) TW_LAUNCH_R(true); else TW_LAUNCH_R(false);
+#define TW_LAUNCH(P, RR, BB) launch_scan_kernel(attention_pair_kernel<P, RR, BB>, g3, b3, s, a, items, hgroups, waves)
+#define TW_LAUNCH_R(P, BB) do { if (R == 1) TW_LAUNCH(P, 1, BB); else if (R == 2) TW_LAUNCH(P, 2, BB); else TW_LAUNCH(P, 4, BB); } while (0)
+    if (a.bits == 4) { if (a.block_table) TW_LAUNCH_R(true, 4); else TW_LAUNCH_R(false, 4); }
+    else { if (a.block_table) TW_LAUNCH_R(true, 2); else TW_LAUNCH_R(false, 2); }
 #undef TW_LAUNCH_R
 #undef TW_LAUNCH
 }

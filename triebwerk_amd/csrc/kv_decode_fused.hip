@@ -52,7 +52,6 @@ static_assert(8 * (2 + 4) * kStageStride <= kFusedMaxQ * kRowFloats * 4, "staged
 template <int R, int BITS, bool PROD, bool PAIR>
 __global__ void __launch_bounds__((PAIR ? kPairWaves : kFusedWaves) * kWave)
 decode_fused_kernel(AttnArgs a, FusedArgs f) {
-    static_assert(!PAIR || BITS == 4, "two heads per wave: a 128-byte cache line is two 4-bit heads");
     constexpr int NW = PAIR ? kPairWaves : kFusedWaves;        // waves of the workgroup
     constexpr int KW = BITS, VW = BITS;
     constexpr uint32_t kHeadBytes = BITS * 16;
@@ -283,8 +282,11 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
                 uint32_t w = *reinterpret_cast<uint32_t*>(&p);
                 *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
             } else {
-                half2_t p0 = {(half_t)__shfl(cent_lane, e & 3, 64), (half_t)__shfl(cent_lane, (e >> 4) & 3, 64)};
-                half2_t p1 = {(half_t)__shfl(cent_lane, (e >> 2) & 3, 64), (half_t)__shfl(cent_lane, (e >> 6) & 3, 64)};
+                // a byte's four codes in the order 0, 2, 1, 3 (one head per wave: what its lane-pair exchange wants) or
+                // in their own order (two heads per wave)
+                const int f1 = PAIR ? 2 : 4, f2 = PAIR ? 4 : 2;
+                half2_t p0 = {(half_t)__shfl(cent_lane, e & 3, 64), (half_t)__shfl(cent_lane, (e >> f1) & 3, 64)};
+                half2_t p1 = {(half_t)__shfl(cent_lane, (e >> f2) & 3, 64), (half_t)__shfl(cent_lane, (e >> 6) & 3, 64)};
                 uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
                 *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
             }
@@ -391,7 +393,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         // ---- 2 (PAIR). scan of this wave's part, two KV heads per wave (kv_pair_scan.hpp has the tile and why)
         int l2 = lane;
         asm volatile("" : "+v"(l2));
-        PairLane<R> L;
+        PairLane<R, BITS> L;
         L.init(l2, p_s[wave], tab_s);
         const uint32_t kvp = (uint32_t)Hk * kHeadBytes;
         const uint32_t nrow = (uint32_t)Hk * 2u;
@@ -411,23 +413,30 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             next_tile = tile_at(i);
             next_rows = i < ntiles ? max(min(n - next_tile, 32), 0) : 0;
         };
-        auto issue_k = [&](PairTileRegs& t) {
+        // (4 bit: every load instruction covers whole lines, non-temporal; 2 bit: half lines, the ordinary policy)
+        constexpr int kCodesAux = BITS == 4 ? kStreamCodes : 0;
+        auto issue_k = [&](PairTileRegs<BITS>& t) {
             __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + (long long)next_tile * kvp, next_rows * (int)kvp);
 #pragma unroll
-            for (int c = 0; c < 4; c++) t.k[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kStreamCodes);
+            for (int c = 0; c < 4; c++) {
+                if constexpr (BITS == 4) t.k[c] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kCodesAux);
+                else t.k[c] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(koff + (uint32_t)(8 * c) * kvp), 0, kCodesAux);
+            }
         };
-        auto issue_v = [&](PairTileRegs& t) {
+        auto issue_v = [&](PairTileRegs<BITS>& t) {
             __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + (long long)next_tile * kvp, next_rows * (int)kvp);
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kStreamCodes);
+                for (int j = 0; j < 4; j++) {
+                    if constexpr (BITS == 4) t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kCodesAux);
+                    else t.v[sub][j] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)(voff + (uint32_t)(16 * sub + j) * kvp), 0, kCodesAux);
+                }
             }
         };
         // (every lane asks, also those that own no token: they repeat a neighbour's address, which costs nothing, and
         // the loop has no branch here)
-        auto issue_n = [&](PairTileRegs& t) {
+        auto issue_n = [&](PairTileRegs<BITS>& t) {
             __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + (long long)next_tile * nrow, next_rows * (int)nrow);
             __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + (long long)next_tile * nrow, next_rows * (int)nrow);
             t.n[0][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
@@ -443,7 +452,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         // make the memory slower here, not faster; the first tile asked for before the rotations, 0.4 us slower, as
         // with one head per wave; the scores of tile i + 1 placed beside the P.V of tile i for the scheduler to
         // interleave, 3 % slower.)
-        PairTileRegs t;
+        PairTileRegs<BITS> t;
         rotate_unit();
         set_next(0);
         issue_k(t);
@@ -759,7 +768,7 @@ bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
 // vector per 16 threads) and its HKW * R outputs its merge slots (one per 32 threads).
 bool decode_fused_pairs(const AttnArgs& a, int hkw) {
     const int R = a.num_heads / a.num_kv_heads;
-    return a.bits == 4 && (hkw & 1) == 0 && (2 * kPairWaves) % hkw == 0 && hkw * (2 + R) <= 4 * kPairWaves && hkw * R <= 2 * kPairWaves;
+    return (a.bits == 4 || a.bits == 2) && (hkw & 1) == 0 && (2 * kPairWaves) % hkw == 0 && hkw * (2 + R) <= 4 * kPairWaves && hkw * R <= 2 * kPairWaves;
 }
 
 void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s, bool allow_pairs) {
@@ -776,7 +785,7 @@ void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s
          else launch_scan_kernel(decode_fused_kernel<RR, BB, false, PP>, g3, b3, s, a, f); } while (0)
 #define TW_FUSED_R(BB, PP) do { if (R == 1) TW_FUSED(1, BB, PP); else if (R == 2) TW_FUSED(2, BB, PP); else TW_FUSED(4, BB, PP); } while (0)
     if (a.bits == 4) { if (pair) TW_FUSED_R(4, true); else TW_FUSED_R(4, false); }
-    else TW_FUSED_R(2, false);
+    else { if (pair) TW_FUSED_R(2, true); else TW_FUSED_R(2, false); }
 #undef TW_FUSED_R
 #undef TW_FUSED
 }

@@ -30,6 +30,12 @@
 //   P.V      the probabilities times the V norms go through the wave's 1 KB LDS tile into A-operand order (rows as
 //            above); MFMA j: columns 0-7 = dim 16 (pn % 8) + j of the first head, 8-15 of the second.
 // A product of a row with a column of the other head is computed and never used.
+//
+// The 2-bit form (BITS = 2) is the same tile on rows of half the size: a pair of heads is 64 bytes of a token's row,
+// K 4 x 8 bytes per lane (32 dims), V 8 x 4 bytes (16 dims of one token), the table maps a byte to its FOUR
+// centroids (8 bytes, ds_read_b64, 32 replicas).  Half a line per load instruction, so no non-temporal hint.  For P.V
+// the 2-bit fields of four tokens are transposed into bytes that hold one dim of the four (two v_bfi stages, one
+// instruction per look-up), so that a look-up yields four consecutive contraction slots.
 #pragma once
 
 #include "kv_common.hpp"
@@ -37,10 +43,10 @@
 
 namespace twkv {
 
-constexpr uint32_t kPairRowBytes = 128;      // two 4-bit heads of one token
+template <int BITS> struct PairBytes { static constexpr uint32_t head = BITS * 16u; };     // code bytes of one head and token
 
 // What a lane knows about itself (derive once, after any code that would otherwise keep these alive in registers).
-template <int R>
+template <int R, int BITS = 4>
 struct PairLane {
     int pn, pkg, hd;
     uint32_t nshift;        // 16 hd: where this lane's head sits in a dword of two fp16 norms
@@ -58,16 +64,17 @@ struct PairLane {
     __device__ __forceinline__ void init(int lane, half_t (*p_tile)[32], const uint32_t* table) {
         pn = lane & 15; pkg = lane >> 4; hd = pn >> 3;
         nshift = 16u * (uint32_t)hd;
-        lane_rep = (uint32_t)lane * 4u;
+        lane_rep = BITS == 4 ? (uint32_t)lane * 4u : (uint32_t)(lane & 31) * 8u;
         useful = (pkg & 1) == hd;
         tok0 = 8 * (pkg >> 1) + (pn & 7);
         p_w = &p_tile[4 * hd + ((R < 4 && !useful) ? R : 0)][8 * (tok0 >> 2) + (tok0 & 3)];
         p_r = reinterpret_cast<const uint4*>(&p_tile[pn][8 * pkg]);
         tab = reinterpret_cast<const char*>(table);
-        koff_rows = (uint32_t)(pn & 7); koff_bytes = 16u * (uint32_t)(4 * hd + pkg);
-        voff_rows = (uint32_t)(4 * pkg); voff_bytes = 8u * (uint32_t)pn;
+        koff_rows = (uint32_t)(pn & 7); koff_bytes = (BITS == 4 ? 16u : 8u) * (uint32_t)(4 * hd + pkg);
+        voff_rows = (uint32_t)(4 * pkg); voff_bytes = (BITS == 4 ? 8u : 4u) * (uint32_t)pn;
     }
     __device__ __forceinline__ uint32_t lut32(uint32_t addr) const { return *reinterpret_cast<const uint32_t*>(tab + addr); }
+    __device__ __forceinline__ uint2 lut64(uint32_t addr) const { return *reinterpret_cast<const uint2*>(tab + addr); }
     // reductions over the lanes of this lane's head (lane groups of both parities included: those that own nothing
     // contribute the neutral element)
     __device__ __forceinline__ float head_max(float v) const {
@@ -83,9 +90,13 @@ struct PairLane {
 };
 
 // The registers of one tile in flight.
+template <int BITS> struct PairPieces;
+template <> struct PairPieces<4> { typedef uint32x4_t k_t; typedef uint32x2_t v_t; };
+template <> struct PairPieces<2> { typedef uint32x2_t k_t; typedef uint32_t v_t; };
+template <int BITS = 4>
 struct PairTileRegs {
-    uint32x4_t k[4];        // instruction c
-    uint32x2_t v[2][4];     // [sub-tile][i]
+    typename PairPieces<BITS>::k_t k[4];        // instruction c: 32 dims of one token and head
+    typename PairPieces<BITS>::v_t v[2][4];     // [sub-tile][i]: 16 dims of one token and head
     uint32_t n[2][2];       // [token tok0 | tok0 + 16][K | V]: the pair's two fp16 norms
 };
 
@@ -102,8 +113,8 @@ struct PairState {
         for (int r = 0; r < R; r++) { m_run[r] = kNegBig; l_run[r] = 0.0f; }
     }
     // q_rot of the pair's query heads: row(i) -> the 128 floats of query head i (i = hd * R + r, 0 <= i < 2 R)
-    template <class RowOf>
-    __device__ __forceinline__ void load_query(const PairLane<R>& L, RowOf row_of) {
+    template <class Lane, class RowOf>
+    __device__ __forceinline__ void load_query(const Lane& L, RowOf row_of) {
         const int m = L.pn & 7;                                // operand row m (and m + 8): head m / 4, query head m % 4
         const bool lo_part = (L.pn & 8) != 0;
         const bool live = (m & 3) < R;
@@ -126,8 +137,8 @@ struct PairState {
 
 // One tile.  `tile` is its first token, `n` the tokens of the sequence; after_k / after_n / after_v are called as
 // soon as the K, norm and V registers of `t` have been consumed (the caller re-issues them for a later tile there).
-template <int R, class AfterK, class AfterN, class AfterV>
-__device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R>& S, PairTileRegs& t, int tile, int n,
+template <int R, int BITS, class AfterK, class AfterN, class AfterV>
+__device__ __forceinline__ void pair_scan_tile(const PairLane<R, BITS>& L, PairState<R>& S, PairTileRegs<BITS>& t, int tile, int n,
                                                AfterK after_k, AfterN after_n, AfterV after_v) {
     constexpr float kRaise = 5.0f;                     // raise the running max only past 2^5
     // ---- scores: set c = tokens 8c .. 8c+7 of both heads
@@ -137,11 +148,19 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
         union { uint32_t u[4]; half8_t h; } kv[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint32_t w = t.k[c][j];
-            kv[j].u[0] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0400u));
-            kv[j].u[1] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0500u));
-            kv[j].u[2] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0600u));
-            kv[j].u[3] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0700u));
+            if constexpr (BITS == 4) {
+                const uint32_t w = t.k[c][j];
+                kv[j].u[0] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0400u));
+                kv[j].u[1] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0500u));
+                kv[j].u[2] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0600u));
+                kv[j].u[3] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0700u));
+            } else {                                            // bytes 2j and 2j + 1 of the lane's 8: dims 8j .. 8j + 7
+                const uint32_t w = t.k[c][j >> 1];
+                const uint32_t sel = 0x0c0c0400u + ((uint32_t)(2 * (j & 1)) << 8);
+                const uint2 lo = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel));
+                const uint2 hi = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel + 0x100u));
+                kv[j].u[0] = lo.x; kv[j].u[1] = lo.y; kv[j].u[2] = hi.x; kv[j].u[3] = hi.y;
+            }
         }
         s[c] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -219,6 +238,7 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
 
     __builtin_amdgcn_s_setprio(2);
     // ---- O[row][dim 16 (pn % 8) + j of head pn / 8] += P[row][token] V[token][dim]
+    if constexpr (BITS == 4) {
     uint32_t xe[2][4], xo[2][4];
 #pragma unroll
     for (int dw = 0; dw < 2; dw++) {
@@ -248,14 +268,43 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R>& L, PairState<R
             S.o[8 * dw + 2 * jp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bo.h, S.o[8 * dw + 2 * jp + 1], 0, 0, 0);
         }
     }
+    } else {
+    // 2 bit: t.v[sub][i] holds the 16 codes (dims 0..15 of the lane's 16, field j at bit 2j) of token 4 pkg + i of
+    // sub-tile `sub`.  y[sub][m]: bytes k = 0..3, byte k = the codes of the sub-tile's four tokens (token i at bit 2i)
+    // for dim 4k + {0, 2, 1, 3}[m]: one look-up gives the four contraction slots 4 sub .. 4 sub + 3 of that dim.
+    uint32_t y[2][4];
+#pragma unroll
+    for (int sub = 0; sub < 2; sub++) {
+        const uint32_t w0 = t.v[sub][0], w1 = t.v[sub][1], w2 = t.v[sub][2], w3 = t.v[sub][3];
+        // nibble k of xe: tokens (a, b) at dim 2k; of xo: at dim 2k + 1
+        const uint32_t xe01 = (w0 & 0x33333333u) | ((w1 << 2) & 0xccccccccu), xo01 = ((w0 >> 2) & 0x33333333u) | (w1 & 0xccccccccu);
+        const uint32_t xe23 = (w2 & 0x33333333u) | ((w3 << 2) & 0xccccccccu), xo23 = ((w2 >> 2) & 0x33333333u) | (w3 & 0xccccccccu);
+        y[sub][0] = (xe01 & 0x0f0f0f0fu) | ((xe23 << 4) & 0xf0f0f0f0u);        // dims 0, 4, 8, 12
+        y[sub][1] = ((xe01 >> 4) & 0x0f0f0f0fu) | (xe23 & 0xf0f0f0f0u);        // dims 2, 6, 10, 14
+        y[sub][2] = (xo01 & 0x0f0f0f0fu) | ((xo23 << 4) & 0xf0f0f0f0u);        // dims 1, 5, 9, 13
+        y[sub][3] = ((xo01 >> 4) & 0x0f0f0f0fu) | (xo23 & 0xf0f0f0f0u);        // dims 3, 7, 11, 15
+    }
+    after_v();
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        constexpr int kWhich[4] = {0, 2, 1, 3};
+        const int m = kWhich[j & 3];
+        const uint32_t sel = 0x0c0c0400u + ((uint32_t)(j >> 2) << 8);
+        const uint2 a4 = L.lut64(__builtin_amdgcn_perm(y[0][m], L.lane_rep, sel));
+        const uint2 b4 = L.lut64(__builtin_amdgcn_perm(y[1][m], L.lane_rep, sel));
+        union { uint32_t u[4]; half8_t h; } bv;
+        bv.u[0] = a4.x; bv.u[1] = a4.y; bv.u[2] = b4.x; bv.u[3] = b4.y;
+        S.o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bv.h, S.o[j], 0, 0, 0);
+    }
+    }
     __builtin_amdgcn_s_setprio(0);
 }
 
 // The wave's partial result per (head of the pair, query head): sink(hd, r, dims) is called by the 16 lanes that
 // hold the rows of head hd with dims = the lane's 16 values of dim 16 (pn % 8) .. +15 (value + remainder rows added,
 // 1 / alpha applied); all lanes end with l_run summed over the head.
-template <int R, class Sink>
-__device__ __forceinline__ void pair_scan_finish(const PairLane<R>& L, PairState<R>& S, float inv_alpha, Sink sink) {
+template <int R, int BITS, class Sink>
+__device__ __forceinline__ void pair_scan_finish(const PairLane<R, BITS>& L, PairState<R>& S, float inv_alpha, Sink sink) {
     const int khi = L.hd;                                       // lane group that holds the rows of head hd
 #pragma unroll
     for (int r = 0; r < R; r++) {
