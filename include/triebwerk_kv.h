@@ -191,7 +191,7 @@ const char* tw_kv_debug_last_scan_kernel(void);
  * knows (1 = one launch, 0 = three): G sequences,
  * cache width `bits`, max_seq_len, and the range of positions + 1 (ctx_max = 0: unknown).  One launch when every
  * wave gets at most 8 tiles of 32 tokens, or when the lengths are within 1/8 of each other, the batch gives at
- * least half the CUs a workgroup and the launch stays under ~1M tokens (512k at 2 bit).
+ * least half the CUs a workgroup and the launch stays under ~1M tokens (480k at 2 bit).
  * Alignment of the buffers, which the entry point also checks, is not part of it. */
 int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max);
 /* Layer steps that took the one-launch kernel since the library was loaded (launches issued or recorded into a

@@ -213,7 +213,7 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
     if (bound <= 256 * split) return 1;                           // at most 8 tiles of 32 tokens per wave
     if (!known || (long long)(ctx_max - ctx_min) * 8 > ctx_max || units * 2 < compute_units_host()) return 0;
     const long long tokens = (long long)G * ctx_max;
-    return tokens <= (bits == 2 ? (512LL << 10) : (1LL << 20)) ? 1 : 0;
+    return tokens <= (bits == 2 ? (480LL << 10) : (1LL << 20)) ? 1 : 0;
 }
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }
 const char* tw_kv_debug_last_scan_kernel(void) { return twkv::g_last_scan_kernel; }
