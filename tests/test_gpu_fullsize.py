@@ -154,7 +154,7 @@ def test_target_shape_append_and_attention(kv, oracle, rotation_fixture, bits):
                                      kv_dim, bits)
     scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
     outs = {}
-    for variant in (0, 1, 3, 4):
+    for variant in (0, 1, 3):
         kv.set_attention_variant(variant)
         out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
         kv.launch_turbo_gqa_attention_batch(out, dev(q), ck, cv, kn, vn, rot, scratch, dev(pos), msl, G, H, Hk, D,
@@ -258,7 +258,7 @@ def test_ragged_paged_batch64(kv, oracle, rotation_fixture, bits):
     want = np.zeros((G, q_dim), np.float16)
     oracle.turbo_gqa_attention_batch(want, q, ck, cv, kn, vn, rotation_fixture, pos, msl, G, H, Hk, D, q_dim, kv_dim, bits)
     ws = torch.zeros(kv.attention_workspace_floats(G, H, msl), dtype=torch.float32, device="cuda")
-    for variant in (0, 1, 3, 4):
+    for variant in (0, 1, 3):
         kv.set_attention_variant(variant)
         out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
         kv.tw_paged_turbo_gqa_attention_batch(out, dev(q), p_ck, p_cv, p_kn, p_vn, rot, ws, dev(pos), d_bt,
@@ -340,7 +340,7 @@ def test_extremely_ragged_batch(kv, oracle, rotation_fixture, bits):
     oracle.turbo_gqa_attention_batch(want, q, host(ck), host(cv), host(kn), host(vn), rotation_fixture, pos, msl, G, H, Hk,
                                      D, q_dim, kv_dim, bits)
     scratch = torch.full((G * H * msl,), float("nan"), dtype=torch.float32, device="cuda")   # nothing may rely on its content
-    for variant in (0, 1, 3, 4):
+    for variant in (0, 1, 3):
         kv.set_attention_variant(variant)
         out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
         kv.launch_turbo_gqa_attention_batch(out, dev(q), ck, cv, kn, vn, rot, scratch, dev(pos), msl, G, H, Hk, D,

@@ -24,7 +24,6 @@ SOURCES = [
     "kv_append.hip",
     "kv_attention_valu.hip",
     "kv_attention_mfma.hip",
-    "kv_attention_mfma2c.hip",
     "kv_attention_pair.hip",
     "kv_decode_fused.hip",
     "kv_prefill_mfma.hip",
@@ -48,11 +47,9 @@ HIPCC_FLAGS = [
 
 
 # Files whose kernels run faster with another of LLVM's schedulers than with the default one (measured on
-# MI355X): the two prompt kernels with the iterative ILP scheduler, 3-8 %; the 2-bit scan with loads grouped
-# into clauses, 1 %.  The other decode kernels keep the default: with the ILP schedulers the scans get spills
-# inside their loops, and nothing else measured faster.
+# MI355X): the two prompt kernels with the iterative ILP scheduler, 3-8 %.  The decode kernels keep the default:
+# with the ILP schedulers the scans get spills inside their loops, and nothing else measured faster.
 PER_FILE_FLAGS = {
-    "kv_attention_mfma2c.hip": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
     "kv_prefill_f16_mfma.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"],
     "kv_prefill_tq_mfma.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"],
 }

@@ -688,16 +688,8 @@ bool launch_attention_mfma_scan(const AttnArgs& a, hipStream_t s) {
         launch_prefill_mfma_scan(a, s);
         return false;
     }
-    if (attention_variant() == 4 && attention_mfma2c_usable(a)) {    // (the cooperative 2-bit kernel, kept for A/B tests)
-        launch_attention_mfma2c_scan(a, s);
-        return false;
-    }
     if (attention_variant() != 3 && attention_pair_usable(a)) {      // KV heads in pairs: two heads per wave
         launch_attention_pair_scan(a, s);
-        return false;
-    }
-    if (attention_mfma2c_usable(a)) {
-        launch_attention_mfma2c_scan(a, s);
         return false;
     }
     const int waves = scan_waves(a);

@@ -224,8 +224,5 @@ void launch_attention_pair_scan(const AttnArgs& a, hipStream_t s);
 // test hook (tw_kv_debug_set_attention_variant): 0 automatic, 1 vector-ALU kernels, 2 MFMA kernels, 3 MFMA kernels
 // with one KV head per wave also where the 4-bit scan would give a wave two
 int attention_variant();
-// 2-bit decode scan for 8 KV heads whose waves load whole cache rows together (kv_attention_mfma2c.hip)
-bool attention_mfma2c_usable(const AttnArgs& a);
-void launch_attention_mfma2c_scan(const AttnArgs& a, hipStream_t s);
 
 }  // namespace twkv
