@@ -2,8 +2,9 @@
 // with two KV heads per wave (gfx950).  Same mathematics, workspace and partials as attention_mfma_kernel
 // (kv_attention_mfma.hip; kernels.cu:1641-1776 of the reference) and the same two ways of cutting the work -- even
 // chunks of every sequence, or the balanced walk over all tiles of a ragged batch -- but the tile is
-// kv_pair_scan.hpp's: a wave reads whole 128-byte lines (two heads) with non-temporal loads, so the waves of a
-// group (four pairs = 8 KV heads) read whole 512-byte cache rows between them and every byte is fetched once.
+// kv_pair_scan.hpp's: at 4 bit a wave reads whole 128-byte lines (two heads) with non-temporal loads, so the waves of a
+// group (four pairs = 8 KV heads) read whole 512-byte cache rows between them and every byte is fetched once; at 2 bit
+// a pair is half a line and the loads keep the ordinary policy.
 // Contiguous and paged layout; launched between rotate_kernel (q_rot into the workspace) and merge_rotate_kernel.
 
 #include "kv_common.hpp"

@@ -2,12 +2,15 @@
 // append K and V of the new token (turbo_kv_quantize_batch_kernel, kernels.cu:1563-1636), rotate the query
 // (1671-1681), scan the context (1688-1766), merge the parts of the context, normalise and rotate back
 // (1746, 1769-1775).  forward_layer_batch does this with three launches (engine.cpp:1985-2006) and the
-// three-kernel path of this library (rotate_kernel, attention_mfma_kernel, merge_rotate_kernel) does too;
+// three-kernel path of this library (rotate_kernel, attention_pair_kernel or attention_mfma_kernel,
+// merge_rotate_kernel) does too;
 // each of those small launches costs ~4.5 us before it does anything and the scan another ~6 us to start
 // and drain, which is a third of a layer at contexts of a few hundred tokens.
 //
-// A workgroup of 16 waves owns one sequence and HKW of its KV heads (HKW = 1, 2, 4 or 8) together with
-// their query heads, so nothing is handed from one workgroup to another:
+// A workgroup owns one sequence and HKW of its KV heads (HKW = 1, 2, 4 or 8) together with their query heads, so
+// nothing is handed from one workgroup to another.  Two forms: PAIR (HKW even) -- 8 waves, each scanning two KV heads
+// with the tile of kv_pair_scan.hpp (256 registers per wave, two waves per SIMD either way); otherwise 16 waves with
+// one KV head each, described here:
 //   1. all threads stage the unit's vectors (K heads, V heads, query heads of the new token) in LDS and fill
 //      the centroid table; with producers one wave per K or query vector applies RMSNorm and rotary embedding
 //      there (kernels.cu:880-961).  Waves 0-7 (all 16 when the unit has more than 16 vectors) then rotate the
@@ -18,8 +21,9 @@
 //      w / HKW) for head w % HKW with the loop of attention_mfma_kernel (the table look-ups, MFMA tiling,
 //      online softmax are described there).  All its loads are issued after the barrier: the new token's row
 //      was stored by this workgroup (same CU, same L1), which a workgroup-scope barrier makes visible;
-//   3. the partial results meet in LDS: merge (log-sum-exp), "+1e-8" normalisation, and R^T with the MFMA
-//      chain of merge_rotate_kernel; output gate as there.
+//   3. the partial results meet in LDS: merge (log-sum-exp), "+1e-8" normalisation, and R^T on fp16 MFMAs (value +
+//      remainder of the normalised output; the output tolerates a different order of additions, the codes did
+//      not); output gate as in merge_rotate_kernel.
 // The waves in the upper wave slots of a CU run ~5 % slower (see kv_common.hpp: kPairShare), so the parts
 // of the upper eight waves get 31/64 of the tiles.
 //
