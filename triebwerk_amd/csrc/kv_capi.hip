@@ -40,6 +40,7 @@ constexpr int kMaxSplits = 64;
 constexpr long long kPagedBlockFloats = 64 * (long long)kPartialFloats + 128 + 4;  // per (sequence, head): partials + rotated query
 constexpr int kMinChunk = 128;       // tokens
 constexpr int kTargetGroups = 2048;  // workgroups wanted per launch: 8 per CU on 256 CUs
+constexpr int kMinRowChunk = 64;         // tokens: eight per wave
 constexpr int kTargetItems = 512;    // (sequence, chunk) items wanted by the persistent MFMA scan: one per resident workgroup
 
 void set_error(int code, const char* fmt, ...) {
@@ -79,6 +80,8 @@ bool check_bits(const char* fn, int bits) {
     return true;
 }
 
+int compute_units_host();
+
 // Split the context over workgroups.  ctx_bound: upper bound of positions+1
 // known to the host (max_seq_len, or pos+1 for the by-value entry points).
 // ws_floats_per_head: room per (sequence, head) in the caller's workspace.
@@ -88,16 +91,24 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     // workgroups per split: the MFMA scan takes up to 8 KV heads per workgroup,
     // the vector-ALU kernel one (KV head, tile of query heads) each
     long long base_groups;
+    const bool rows = !mfma && attention_rows_usable(a);
     if (mfma) {
         base_groups = (long long)a.G * ((a.num_kv_heads + 7) / 8);
+    } else if (rows) {
+        base_groups = (long long)a.G * attention_rows_groups(a);
     } else {
         const int group = a.num_heads / a.num_kv_heads;
         const int rt = (group % 4 == 0) ? 4 : (group % 2 == 0) ? 2 : 1;
         base_groups = (long long)a.G * a.num_kv_heads * (group / rt);
     }
     int want = g_nsplit_override.load();
-    if (want <= 0) want = (int)(((mfma ? kTargetItems : kTargetGroups) + base_groups - 1) / base_groups);
-    int max_by_ctx = (ctx_bound + kMinChunk - 1) / kMinChunk;
+    if (want <= 0) {
+        // the whole-row fp16 scan runs two workgroups per CU at once: as many chunks as still fit in that one go
+        if (rows) want = (int)std::max<long long>(1, 2LL * compute_units_host() / base_groups);
+        else want = (int)(((mfma ? kTargetItems : kTargetGroups) + base_groups - 1) / base_groups);
+    }
+    const int min_chunk = rows ? kMinRowChunk : kMinChunk;
+    int max_by_ctx = (ctx_bound + min_chunk - 1) / min_chunk;
     // a block holds nsplit partials, then (16-byte aligned) the rotated query
     int max_by_ws = a.ws ? (int)((ws_floats_per_head - kHeadDim - 3) / kPartialFloats) : 0;
     int nsplit = want;
@@ -111,7 +122,7 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     // The MFMA scan may cut a ragged batch into up to max_slots pieces per sequence instead
     // (a long sequence among short ones takes several groups' worth of tiles).
     int slots = nsplit;
-    if (have_ws && mfma && a.pos_mode != kPosScalar) {
+    if (have_ws && (mfma || rows) && a.pos_mode != kPosScalar) {
         slots = 4 * nsplit + 2;
         if (slots > max_by_ws) slots = max_by_ws;
         if (slots > kMaxSplits) slots = kMaxSplits;
@@ -126,6 +137,13 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
         a.ws = nullptr;          // too small to hold anything: single pass, no workspace
         a.ws_stride = 0;
         a.qrot = nullptr;
+    }
+    if (rows) {
+        a.even_chunks = 1;
+        a.slots_from_ws = 1;
+        // ragged batches: cut the work by tokens, not by sequence (decided on the device from the positions)
+        a.balance = (a.pos_mode != kPosScalar && attention_rows_balances(a)) ? 1 : 0;
+        a.force_merge = a.balance;
     }
 }
 

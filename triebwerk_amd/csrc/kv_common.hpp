@@ -101,6 +101,19 @@ __device__ __forceinline__ bool chunk_nonempty(int n, int c, int nsplit) {
     return chunk_boundary(tiles, (unsigned)c + 1u, (unsigned)nsplit) > chunk_boundary(tiles, (unsigned)c, (unsigned)nsplit);
 }
 
+// The same for the fp16 whole-row scan (AttnArgs::even_chunks): units of 8 tokens, one per wave of its workgroups,
+// dealt out evenly with no shares; units * nsplit < 2^32.
+__device__ __forceinline__ void even_chunk_range(int n, int c, int nsplit, int& t0, int& t1) {
+    const unsigned units = (unsigned)(n + 7) >> 3;
+    t0 = 8 * (int)(((unsigned)c * units) / (unsigned)nsplit);
+    const int e = 8 * (int)((((unsigned)c + 1u) * units) / (unsigned)nsplit);
+    t1 = e < n ? e : n;
+}
+__device__ __forceinline__ bool even_chunk_nonempty(int n, int c, int nsplit) {
+    const unsigned units = (unsigned)(n + 7) >> 3;
+    return (((unsigned)c + 1u) * units) / (unsigned)nsplit > ((unsigned)c * units) / (unsigned)nsplit;
+}
+
 // fp32 -> fp16 of a value that must first exist as a rounded fp32 number.  Without the barrier the
 // compiler folds a preceding multiply or fused multiply-add into the conversion (v_fma_mixlo_f16: one
 // rounding instead of two), which changes a result in a few hundred thousand.

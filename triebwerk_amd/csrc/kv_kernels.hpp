@@ -155,6 +155,7 @@ struct AttnArgs {
     int balance;            // MFMA scan: may cut the batch by tiles instead of by sequence (ragged lengths)
     int max_slots;          // partials the workspace holds per (sequence, head): >= nsplit
     int slots_from_ws;      // merge: the spare word of partial 0 holds the number of partials (0: even chunks)
+    int even_chunks;        // the chunks are the fp16 whole-row scan's (even_chunk_range), not chunk_range's
     // optional output gate (gated attention, kernels.cu:2987-2995): out = half(float(half(out)) * sigmoid(gate))
     const half_t* gate;     // row g at gate + g * gate_stride, laid out like a row of out; NULL = none
     long long gate_stride;
@@ -169,6 +170,11 @@ struct AttnArgs {
 constexpr int kPartialFloats = kHeadDim + 4;  // acc[128], running max, running sum, 2 pad (16-byte rows)
 
 void launch_attention_valu(const AttnArgs& a, hipStream_t s);
+// fp16 cache: will launch_attention_valu run the kernel whose waves read whole rows (eight KV heads)?  Its workgroups
+// have eight waves that share one chunk, so the split planner gives it more and smaller chunks.
+bool attention_rows_usable(const AttnArgs& a);
+int attention_rows_groups(const AttnArgs& a);      // workgroups per (sequence, chunk)
+bool attention_rows_balances(const AttnArgs& a);   // may cut a ragged batch by tokens instead (needs max_slots set)
 void launch_attention_merge(const AttnArgs& a, hipStream_t s);
 bool launch_merge_rotate(const AttnArgs& a, hipStream_t s);   // MFMA merge + rotate-back; false = not applicable
 // MFMA path, two steps so that the scan kernel can be timed alone:
