@@ -291,6 +291,95 @@ def test_fp16_attention_single_sequence(kv, oracle):
         assert rel_err(host(out), want) <= TOL
 
 
+ROW_SCAN_LENS = {
+    # ragged: the balanced walk (lengths differ by more than 1/8), pieces cut at sequence ends, every wave of a
+    # workgroup meets the appended token somewhere
+    "ragged": [0, 1, 7, 8, 9, 15, 16, 17, 63, 64, 65, 100, 255, 256, 257, 300, 511, 512, 513, 700, 900, 1021, 1022, 1023],
+    # nearly equal: even chunks in units of 8 tokens
+    "even": [700 + i for i in range(20)],
+    # very short: most even chunks hold no token
+    "short": [0, 1, 2, 3, 5, 8, 9, 11, 13, 16, 17, 19, 21, 24, 25, 27, 30],
+}
+
+
+@pytest.mark.parametrize("append", [False, True])
+@pytest.mark.parametrize("nsplit", [0, 1, 5])
+@pytest.mark.parametrize("lens_kind", ["ragged", "even", "short"])
+@pytest.mark.parametrize("H,Hk", [(16, 8), (8, 8), (32, 8), (32, 16)])
+def test_fp16_whole_row_scan(kv, oracle, H, Hk, lens_kind, nsplit, append):
+    """fp16 cache with KV heads in blocks of eight and 16 or more sequences: the scan whose waves read whole cache
+    rows (groups of 1, 2 and 4 query heads per KV head, one and two blocks of KV heads), attention alone and with
+    the append inside the launch, == the oracle's attention; the appended rows are the oracle's row copy."""
+    import torch
+    r = gen.rng(230 + H + Hk + nsplit)
+    lens = ROW_SCAN_LENS[lens_kind]
+    G, msl = len(lens), 1024
+    kv_dim, q_dim = Hk * D, H * D
+    ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+    pos = np.array(lens, np.int32)
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    if append:
+        for g in range(G):
+            ck[g, pos[g]:] = 0; cv[g, pos[g]:] = 0
+    d_ck, d_cv = dev(ck), dev(cv)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.set_num_splits(nsplit)
+    try:
+        if append:
+            kv.tw_append_attention_batch(out, dev(q), dev(k), dev(v), d_ck, d_cv, scratch, dev(pos), msl, G, H, Hk, D,
+                                         q_dim, kv_dim)
+        else:
+            kv.launch_gqa_attention_batch(out, dev(q), d_ck, d_cv, scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim)
+    finally:
+        kv.set_num_splits(0)
+    assert kv.last_scan_kernel() == "attention_rows_kernel"
+    if append:
+        oracle.kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    assert_bytes_equal(host(d_ck), ck, "K rows"); assert_bytes_equal(host(d_cv), cv, "V rows")
+    assert rel_err(host(out), want) <= TOL
+
+
+def test_fp16_whole_row_scan_without_workspace_and_paged(kv, oracle):
+    """The same kernel where the caller's scratch is too small for partials (every workgroup walks a whole
+    sequence and writes the output itself), and over 16-token pages in shuffled order."""
+    import torch
+    r = gen.rng(236)
+    G, H, Hk = 18, 16, 8
+    kv_dim, q_dim = Hk * D, H * D
+    pages_per_seq = 12
+    msl = pages_per_seq * 16                       # 192 floats per (sequence, head): no room for a partial and q_rot
+    ck, cv = build_fp16_cache(r, G, msl, kv_dim)
+    pos = np.array([0, 1, 15, 16, 17, 31, 32, 33, 47, 64, 100, 127, 128, 150, 170, 189, 190, 191], np.int32)
+    q = gen.normal_f16(r, (G, q_dim))
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.launch_gqa_attention_batch(out, dev(q), dev(ck), dev(cv), scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim)
+    assert kv.last_scan_kernel() == "attention_rows_kernel"
+    assert rel_err(host(out), want) <= TOL
+
+    bt = gen.shuffled_block_table(r, G, pages_per_seq)
+    pool_k = np.zeros((G * pages_per_seq, 16, kv_dim), np.float16); pool_v = np.zeros_like(pool_k)
+    for g in range(G):
+        for i in range(pages_per_seq):
+            pool_k[bt[g, i]] = ck[g, 16 * i:16 * (i + 1)]; pool_v[bt[g, i]] = cv[g, 16 * i:16 * (i + 1)]
+    for nsplit in (0, 1, 3):
+        out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+        ws = torch.zeros(kv.attention_workspace_floats(G, H, msl), dtype=torch.float32, device="cuda")
+        kv.set_num_splits(nsplit)
+        try:
+            kv.tw_paged_gqa_attention_batch(out, dev(q), dev(pool_k), dev(pool_v), ws, dev(pos), dev(bt), pages_per_seq, msl,
+                                            G, H, Hk, D, q_dim, kv_dim)
+        finally:
+            kv.set_num_splits(0)
+        assert kv.last_scan_kernel() == "attention_rows_kernel"
+        assert rel_err(host(out), want) <= TOL, nsplit
+
+
 def test_fp16_prefill_attention(kv, oracle):
     r = gen.rng(204)
     T, H, Hk, msl = 70, 4, 2, 96
@@ -992,17 +1081,16 @@ def test_sigmoid_gate_batch(kv, oracle):
     assert np.mean(host(d_data).view(np.uint16) == data.view(np.uint16)) > 0.999
 
 
-@pytest.mark.parametrize("kv_bits,nsplit", [(4, 0), (2, 0), (0, 0), (0, 1), (4, 1)])
-def test_layer_attention_step_with_gate(kv, oracle, rotation_fixture, kv_bits, nsplit):
+@pytest.mark.parametrize("kv_bits,nsplit,G", [(4, 0, 6), (2, 0, 6), (0, 0, 6), (0, 1, 6), (4, 1, 6), (0, 0, 18)])
+def test_layer_attention_step_with_gate(kv, oracle, rotation_fixture, kv_bits, nsplit, G):
     """Producers + append + attention + sigmoid gate through one call, with the gate in the second half of
     the q rows (gated q projection: row stride 2*H*D) == the oracle's six steps."""
     import torch
     r = gen.rng(760 + kv_bits + nsplit)
-    G, H, Hk, msl = 6, 16, 8, 160
+    H, Hk, msl = 16, 8, 160
     kv_dim, q_dim = Hk * D, 2 * H * D
-    lens = np.array([1, 2, 17, 64, 100, 159])
+    lens = np.resize(np.array([1, 2, 17, 64, 100, 159]), G)     # 18 sequences: the fp16 scan that reads whole rows
     pos = lens.astype(np.int32)
-    pos[5] = 159
     q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
     qw = (1.0 + 0.2 * r.standard_normal(D)).astype(np.float16); kw = (1.0 + 0.2 * r.standard_normal(D)).astype(np.float16)
     ct, st = rope_tables(msl, D)

@@ -280,6 +280,11 @@ def set_decode_fused(mode: int) -> None:
     _lib.load().tw_kv_debug_set_decode_fused(int(mode))
 
 
+def last_scan_kernel() -> str:
+    """Name of the kernel that the last decode-attention call launched for the context scan (a test hook)."""
+    return _lib.load().tw_kv_debug_last_scan_kernel().decode()
+
+
 def set_num_splits(nsplit: int) -> None:
     _lib.load().tw_kv_debug_set_num_splits(int(nsplit))
 
