@@ -30,6 +30,12 @@
 // One sequence is one workgroup's work whatever its length: right for batches of similar lengths (a
 // rollout's decode steps) and for short contexts; the three-kernel path with its balanced walk stays the
 // choice for ragged long contexts, and the only one for the paged layout.
+// (Tried at batch 64: workgroups of all 8 KV heads, four per sequence with a quarter of the context each, so that a
+// workgroup's waves read whole cache rows side by side -- a plain read of the cache in that pattern runs at 6.8
+// instead of 6.4 TB/s -- and the quarters' sums meeting in a workspace, finished by whichever workgroup takes the
+// last arrival ticket.  The agent-scope release and acquire fences around that hand-over, each a write-back or an
+// invalidation of the XCD's L2, cost 34 us per launch; with no fence at all, which is not correct, the launch took
+// 99 us against 97: the scan is not held up by the access pattern.)
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
