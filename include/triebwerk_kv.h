@@ -161,7 +161,8 @@ const char* tw_kv_build_info(void);
  * while no other thread is inside the library. */
 
 /* Compressed-attention kernel family: 0 = automatic, 1 = fp32 vector-ALU kernels, 2 = MFMA kernels, 3 = MFMA kernels
- * with one KV head per wave also where the scan would give a wave two. */
+ * with one KV head per wave also where the scan would give a wave two; 3 also keeps the fp16 cache on the kernel whose
+ * workgroups scan one KV head where the one whose waves read whole rows of eight heads would run. */
 void tw_kv_debug_set_attention_variant(int variant);
 int tw_kv_debug_get_attention_variant(void);
 /* Split count of decode attention (0 = automatic). */
@@ -181,7 +182,7 @@ void tw_kv_debug_set_decode_fused(int mode);
 void tw_kv_debug_profile_attention(int enable);
 int tw_kv_debug_profile_read(double* total_ms, int* launches);
 /* Name of the kernel that the last attention call of this process launched (or recorded into a graph) for the
- * context: "attention_pair_kernel", "attention_mfma_kernel", "attention_valu_kernel",
+ * context: "attention_pair_kernel", "attention_mfma_kernel", "attention_rows_kernel", "attention_valu_kernel",
  * "decode_fused_kernel, two KV heads per wave", "decode_fused_kernel, one KV head per wave", a prefill kernel, or
  * "none".  A static string; lets a benchmark name the kernel its figures belong to. */
 const char* tw_kv_debug_last_scan_kernel(void);
