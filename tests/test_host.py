@@ -102,12 +102,12 @@ def test_decode_step_plan_is_the_documented_rule():
     lib = _lib.load()
     plan = lib.tw_kv_decode_step_plan
     # the benchmark's target: 64 sequences of 8192 tokens, lengths known and equal -> one launch at 4 bit; at 2 bit
-    # the three-kernel path has caught up at that size (from 480k tokens per launch on; at 4 bit from a million on)
+    # the three-kernel path has caught up at that size
     assert plan(64, 16, 8, 4, 8448, 8192, 8192) == 1
     assert plan(64, 16, 8, 2, 8448, 8192, 8192) == 0
-    assert plan(64, 16, 8, 2, 8448, 7000, 7000) == 1
+    assert plan(64, 16, 8, 2, 8448, 6000, 6000) == 1
     assert plan(128, 16, 8, 2, 8448, 8192, 8192) == 0
-    assert plan(128, 16, 8, 4, 8448, 8192, 8192) == 1
+    assert plan(128, 16, 8, 4, 8448, 4096, 4096) == 1
     # the same batch with nothing known about the lengths, or known to be ragged: three launches
     assert plan(64, 16, 8, 4, 8448, 0, 0) == 0
     assert plan(64, 16, 8, 4, 8448, 512, 8192) == 0
@@ -117,12 +117,20 @@ def test_decode_step_plan_is_the_documented_rule():
     # a rollout: 128 sequences a few hundred tokens long, at either width
     assert plan(128, 16, 8, 4, 1536, 300, 300) == 1
     assert plan(128, 16, 8, 2, 1536, 300, 300) == 1
-    # small batches: one head per workgroup, 16 parts; long contexts of few sequences do not fill the GPU
+    # small batches: one head per workgroup, 16 parts; long contexts of few sequences do not fill the GPU with one
+    # workgroup per (sequence, head) -- 63 us per layer against 45 at batch 16, 8192 tokens -- shorter ones do
     assert plan(4, 16, 8, 4, 640, 0, 0) == 1
     assert plan(4, 16, 8, 4, 16384, 16000, 16000) == 0
+    assert plan(16, 16, 8, 4, 8448, 8192, 8192) == 0
+    assert plan(32, 16, 8, 4, 8448, 8192, 8192) == 0
+    assert plan(16, 16, 8, 4, 8448, 2048, 2048) == 1
     assert plan(16, 32, 8, 2, 4352, 4097, 4097) == 1          # 2 bit, GQA 4, 65k tokens
-    # beyond a million tokens per launch the three-kernel path has caught up
+    # batches that fill three quarters of the CUs with two or four heads per workgroup
+    assert plan(48, 16, 8, 4, 8448, 8192, 8192) == 1
+    assert plan(96, 16, 8, 4, 8448, 4096, 4096) == 1
+    # large launches: the three-kernel path has caught up
     assert plan(256, 16, 8, 4, 8448, 8192, 8192) == 0
+    assert plan(128, 16, 8, 4, 8448, 8192, 8192) == 0
     # shapes the one-launch kernel does not take
     assert plan(64, 64, 8, 4, 1024, 0, 0) == 0                # GQA group 8
     assert plan(64, 16, 8, 3, 1024, 0, 0) == 0

@@ -4,7 +4,9 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -103,9 +105,12 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     }
     int want = g_nsplit_override.load();
     if (want <= 0) {
-        // the whole-row fp16 scan runs two workgroups per CU at once: as many chunks as still fit in that one go
+        // the whole-row fp16 scan runs two workgroups per CU at once and the MFMA scans kTargetItems items: as many
+        // chunks as still fit in that one go (one more would leave a second round for a few items: batch 48 took
+        // 112 us with 11 chunks per sequence, 528 items)
         if (rows) want = (int)std::max<long long>(1, 2LL * compute_units_host() / base_groups);
-        else want = (int)(((mfma ? kTargetItems : kTargetGroups) + base_groups - 1) / base_groups);
+        else if (mfma) want = (int)std::max<long long>(1, kTargetItems / base_groups);
+        else want = (int)((kTargetGroups + base_groups - 1) / base_groups);
     }
     const int min_chunk = rows ? kMinRowChunk : kMinChunk;
     int max_by_ctx = (ctx_bound + min_chunk - 1) / min_chunk;
@@ -223,15 +228,20 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
     if (G <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || (bits != 2 && bits != 4)) return 0;
     const int group = num_heads / num_kv_heads;
     if (group != 1 && group != 2 && group != 4) return 0;
-    const int hkw = decode_fused_heads_per_workgroup(G, num_kv_heads);
+    const bool allow_pairs = g_decode_fused.load() != 3;
+    const int hkw = decode_fused_heads_per_workgroup(G, num_heads, num_kv_heads, bits, allow_pairs);
     const int split = 16 / hkw;                                   // parts of the context per head: waves / heads
-    const long long units = (long long)G * (num_kv_heads / hkw);  // workgroups
     const bool known = ctx_max > 0;
     const int bound = known ? ctx_max : max_seq_len;
     if (bound <= 256 * split) return 1;                           // at most 8 tiles of 32 tokens per wave
-    if (!known || (long long)(ctx_max - ctx_min) * 8 > ctx_max || units * 2 < compute_units_host()) return 0;
-    const long long tokens = (long long)G * ctx_max;
-    return tokens <= (bits == 2 ? (480LL << 10) : (1LL << 20)) ? 1 : 0;
+    if (!known || (long long)(ctx_max - ctx_min) * 8 > ctx_max) return 0;   // lengths unknown or ragged: the balanced walk
+    // Equal lengths: the cheaper of the two by estimates fitted to launches measured on MI355X (microseconds per
+    // layer): one launch as decode_fused_estimate_us counts it; three launches: 27 us of launches, query rotation and
+    // merge, and the scan at its rate.
+    const double bpt = bits == 4 ? 132.0 : 68.0;                  // bytes per token and KV head: K and V codes and norms
+    const double one = decode_fused_estimate_us(G, num_heads, num_kv_heads, bits, allow_pairs, hkw, ctx_max);
+    const double three = 27.0 + (double)G * num_kv_heads * bpt * ctx_max / (bits == 4 ? 7.4e6 : 5.8e6);
+    return one <= three ? 1 : 0;
 }
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }
 const char* tw_kv_debug_last_scan_kernel(void) { return twkv::g_last_scan_kernel; }

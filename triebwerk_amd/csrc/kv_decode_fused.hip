@@ -37,6 +37,8 @@
 // invalidation of the XCD's L2, cost 34 us per launch; with no fence at all, which is not correct, the launch took
 // 99 us against 97: the scan is not held up by the access pattern.)
 
+#include <cmath>
+
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
 #include "kv_mfma_util.hpp"
@@ -746,14 +748,45 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     }
 }
 
-// KV heads per workgroup: as many (of 8, 4, 2, 1) as still give every CU a workgroup -- the more heads, the
-// longer the contiguous piece of a cache row one workgroup reads -- and one when the batch is too small for that.
-int decode_fused_heads_per_workgroup(int G, int Hk) {
-    const long long cus = compute_units();
-    for (int c = 8; c > 1; c >>= 1) {
-        if (Hk % c == 0 && (long long)G * (Hk / c) >= cus) return c;
+// Two KV heads per wave (PAIR) when the workgroup's heads come in pairs: eight waves, every cache line of the 4-bit
+// cache fetched by one instruction.  The workgroup's HKW * (2 + R) vectors must fit its staging slots (a vector per
+// 16 threads) and its HKW * R outputs its merge slots (one per 32 threads).
+static bool pairs_fit(int bits, int R, int hkw) {
+    return (bits == 4 || bits == 2) && (hkw & 1) == 0 && (2 * kPairWaves) % hkw == 0 && hkw * (2 + R) <= 4 * kPairWaves && hkw * R <= 2 * kPairWaves;
+}
+bool decode_fused_pairs(const AttnArgs& a, int hkw) { return pairs_fit(a.bits, a.num_heads / a.num_kv_heads, hkw); }
+
+// Microseconds one launch takes for G sequences of ctx tokens with hkw KV heads per workgroup, by a count fitted to
+// launches measured on MI355X at batches 16 to 256 and contexts 1k to 8k (it reproduces them within 5 %): the
+// workgroups run in rounds of one per CU; a round costs 13 us of prologue and epilogue and, per token of context, the
+// cube-root sum of what one CU sustains for the workgroup's heads (a workgroup whose waves scan one head each moves
+// its bytes at about half the rate of one whose waves scan two) and of the whole chip's rate for all the workgroups
+// of the round.
+double decode_fused_estimate_us(int G, int num_heads, int Hk, int bits, bool allow_pairs, int hkw, double ctx) {
+    const double cus = compute_units();
+    const int R = Hk > 0 ? num_heads / Hk : 1;
+    const double bpt = bits == 4 ? 132.0 : 68.0;                  // bytes per token and KV head: K and V codes and norms
+    const double units = (double)G * (Hk / hkw);
+    const double rounds = std::ceil(units / cus), active = units < cus ? units : cus;
+    const bool pair = allow_pairs && pairs_fit(bits, R, hkw);
+    const double per_head_ns = pair ? (bits == 4 ? 3.08 : 2.88) : (bits == 4 ? 5.95 : 4.68);
+    const double k_cu = hkw * per_head_ns, k_bw = active * hkw * bpt / (bits == 4 ? 7200.0 : 5240.0);   // ns per token
+    return rounds * (13.0 + ctx * 1e-3 * std::cbrt(k_cu * k_cu * k_cu + k_bw * k_bw * k_bw));
+}
+
+// KV heads per workgroup (8, 4, 2 or 1): the choice with the smallest estimate at a context of 4096 tokens (the order
+// hardly depends on the context); among equals the larger number, whose workgroups read longer contiguous pieces of a
+// cache row.  (Batch 64 with 8 KV heads: 2, one round of 256 workgroups; batch 48: 2 again, 192 workgroups in one
+// round, where two rounds of 384 single-head workgroups took 119 us against 85; batch 96: 4.)
+int decode_fused_heads_per_workgroup(int G, int num_heads, int Hk, int bits, bool allow_pairs) {
+    int best = 1;
+    double best_us = 0.0;
+    for (int c = 1; c <= 8; c <<= 1) {
+        if (Hk % c != 0) continue;
+        const double us = decode_fused_estimate_us(G, num_heads, Hk, bits, allow_pairs, c, 4096.0);
+        if (c == 1 || us <= best_us) { best = c; best_us = us; }
     }
-    return 1;
+    return best;
 }
 
 bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
@@ -773,17 +806,9 @@ bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
     return true;
 }
 
-// Two KV heads per wave (PAIR) when the cache is 4 bit and the workgroup's heads come in pairs: eight waves, every
-// cache line fetched by one instruction.  The workgroup's HKW * (2 + R) vectors must fit its staging slots (a
-// vector per 16 threads) and its HKW * R outputs its merge slots (one per 32 threads).
-bool decode_fused_pairs(const AttnArgs& a, int hkw) {
-    const int R = a.num_heads / a.num_kv_heads;
-    return (a.bits == 4 || a.bits == 2) && (hkw & 1) == 0 && (2 * kPairWaves) % hkw == 0 && hkw * (2 + R) <= 4 * kPairWaves && hkw * R <= 2 * kPairWaves;
-}
-
 void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s, bool allow_pairs) {
     FusedArgs f = f_in;
-    f.hkw = decode_fused_heads_per_workgroup(a.G, a.num_kv_heads);
+    f.hkw = decode_fused_heads_per_workgroup(a.G, a.num_heads, a.num_kv_heads, a.bits, allow_pairs);
     f.q_scale = attention_mfma_q_scale(a.bits);
     const int R = a.num_heads / a.num_kv_heads;
     const bool pair = allow_pairs && decode_fused_pairs(a, f.hkw);

@@ -205,7 +205,9 @@ struct FusedArgs {
     int rope_dim;            // 128, or a multiple of 16 up to 64
 };
 bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f);
-int decode_fused_heads_per_workgroup(int G, int num_kv_heads);   // 8, 4, 2 or 1; a workgroup has 16 waves
+int decode_fused_heads_per_workgroup(int G, int num_heads, int num_kv_heads, int bits, bool allow_pairs);   // 8, 4, 2 or 1
+// estimated microseconds of one launch with hkw KV heads per workgroup, all sequences at ctx tokens
+double decode_fused_estimate_us(int G, int num_heads, int num_kv_heads, int bits, bool allow_pairs, int hkw, double ctx);
 // allow_pairs: the 4-bit kernel whose waves scan two KV heads each, where the shape admits it (false: one head per wave)
 void launch_decode_fused(const AttnArgs& a, const FusedArgs& f, hipStream_t s, bool allow_pairs);
 // causal prefill with blocks of query tokens per wave (kv_prefill_mfma.hip); same workspace and merge
