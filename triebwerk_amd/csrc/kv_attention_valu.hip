@@ -627,31 +627,47 @@ attention_rows_kernel(AttnArgs a, int total_items, int hgroups) {
     }
 }
 
-// Log-sum-exp merge of the split partials, normalisation, rotate-back, store.
+// Log-sum-exp merge of the split partials, normalisation, rotate-back, store.  Thread c first takes partial c's
+// maximum and sum (at most kMergeSlots partials), so that the weights of all partials are known after one round trip
+// to memory; the sums over the partials then run over loads that do not depend on each other.
+constexpr int kMergeSlots = 64;
 __global__ void __launch_bounds__(kHeadDim)
 attention_merge_kernel(AttnArgs a) {
     __shared__ float o_s[kHeadDim];
+    __shared__ float w_s[kMergeSlots];
+    __shared__ float red_s[2][2];
     const int head = blockIdx.x, g = blockIdx.y, d = threadIdx.x;
     const int n = seq_pos(a, g) + 1;
     const float* part = a.ws + ((long long)g * a.num_heads + head) * a.ws_stride;
-    // which slots were written: the first nseg (balanced MFMA scan) or the non-empty even chunks
+    // which slots were written: the first nseg (balanced walk) or the non-empty even chunks
     const int nseg = a.slots_from_ws ? reinterpret_cast<const int*>(part)[kHeadDim + 2] : 0;
     auto live = [&](int c) -> bool {
         if (nseg > 0) return c < nseg;
         return a.even_chunks ? even_chunk_nonempty(n, c, a.nsplit) : chunk_nonempty(n, c, a.nsplit);
     };
-    const int nslots = nseg > 0 ? nseg : a.nsplit;
-    float mg = kNegBig;
-    for (int cidx = 0; cidx < nslots; cidx++) {
-        if (live(cidx)) mg = fmaxf(mg, part[(long long)cidx * kPartialFloats + kHeadDim]);
+    const int nslots = min(nseg > 0 ? nseg : a.nsplit, kMergeSlots);
+    const bool mine = d < nslots && live(d);                // no workgroup wrote the other slots
+    float m_c = kNegBig, l_c = 0.0f;
+    if (mine) {
+        m_c = part[(long long)d * kPartialFloats + kHeadDim];
+        l_c = part[(long long)d * kPartialFloats + kHeadDim + 1];
     }
-    float lsum = 0.0f, av = 0.0f;
+    const float mw = wave_max(m_c);
+    if ((d & 63) == 0) red_s[0][d >> 6] = mw;
+    __syncthreads();
+    const float mg = fmaxf(red_s[0][0], red_s[0][1]);
+    const float w = mine ? (a.m_log2 ? __builtin_amdgcn_exp2f(m_c - mg) : __expf(m_c - mg)) : 0.0f;
+    if (d < kMergeSlots) w_s[d] = w;
+    const float lw = wave_sum(l_c * w);
+    if ((d & 63) == 0) red_s[1][d >> 6] = lw;
+    __syncthreads();
+    const float lsum = red_s[1][0] + red_s[1][1];
+    float av = 0.0f;
+#pragma unroll 8
     for (int cidx = 0; cidx < nslots; cidx++) {
-        if (!live(cidx)) continue;                          // no workgroup wrote this slot
-        const float* pc = part + (long long)cidx * kPartialFloats;
-        float f = a.m_log2 ? __builtin_amdgcn_exp2f(pc[kHeadDim] - mg) : __expf(pc[kHeadDim] - mg);
-        lsum = __builtin_fmaf(pc[kHeadDim + 1], f, lsum);
-        av = __builtin_fmaf(pc[d], f, av);
+        const float wc = w_s[cidx];
+        const float v = part[(long long)cidx * kPartialFloats + d];     // a slot nobody wrote: inside the block, not used
+        av = wc != 0.0f ? __builtin_fmaf(v, wc, av) : av;
     }
     o_s[d] = av * (1.0f / (lsum + 1e-8f));
     __syncthreads();
@@ -675,15 +691,15 @@ static void launch_valu_mode(const AttnArgs& a, hipStream_t s) {
     else launch_scan_kernel(attention_valu_kernel<MODE, 1, false>, grid, block, s, a);
 }
 
-// The whole-row kernel: fp16 cache, KV heads in blocks of eight, 16-byte aligned rows, and a batch large enough that
-// at most 64 chunks per sequence fill the chip.
+// The whole-row kernel: fp16 cache, KV heads in blocks of eight, 16-byte aligned rows.  (Whether the batch is large
+// enough for it is the split planner's question: it knows the bound of the context.)
 bool attention_rows_usable(const AttnArgs& a) {
     if (a.bits != 0 || a.num_kv_heads <= 0 || a.num_kv_heads % kRowHeads != 0 || attention_variant() == 3) return false;
     auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     if (!al(a.k) || !al(a.v) || !al(a.q) || !al(a.out) || (a.q_stride & 7) != 0) return false;
     if (a.gate && (!al(a.gate) || (a.gate_stride & 7) != 0)) return false;
     if (a.k_new && (!al(a.k_new) || !al(a.v_new) || (a.kv_new_stride & 7) != 0)) return false;
-    return (long long)a.G * attention_rows_groups(a) >= 16;
+    return true;
 }
 
 // blocks of 8 KV heads times tiles of query heads: the workgroups one chunk of one sequence takes
@@ -725,7 +741,7 @@ static void launch_attention_rows(const AttnArgs& a, hipStream_t s) {
 
 void launch_attention_valu(const AttnArgs& a, hipStream_t s) {
     if (a.G <= 0) return;
-    if (attention_rows_usable(a)) { launch_attention_rows(a, s); return; }
+    if (a.even_chunks) { launch_attention_rows(a, s); return; }     // the split planner chose the whole-row kernel
     note_scan_kernel("attention_valu_kernel");
     if (a.bits == 0) launch_valu_mode<0>(a, s);
     else if (a.bits == 4) launch_valu_mode<4>(a, s);

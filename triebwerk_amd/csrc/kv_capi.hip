@@ -93,7 +93,15 @@ void plan_splits(AttnArgs& a, int ctx_bound, long long ws_floats_per_head) {
     // workgroups per split: the MFMA scan takes up to 8 KV heads per workgroup,
     // the vector-ALU kernel one (KV head, tile of query heads) each
     long long base_groups;
-    const bool rows = !mfma && attention_rows_usable(a);
+    // fp16 whole-row scan: 16 or more (sequence, head block) pairs, or fewer with a context long enough that its
+    // chunks (at most kMaxSplits of at least kMinRowChunk tokens) still make 256 workgroups -- below that the kernel
+    // with a workgroup per (sequence, KV head, chunk) has more of them in flight
+    bool rows = !mfma && attention_rows_usable(a);
+    if (rows) {
+        const long long pairs = (long long)a.G * attention_rows_groups(a);
+        const long long chunks = std::min<long long>(kMaxSplits, (ctx_bound + kMinRowChunk - 1) / kMinRowChunk);
+        rows = pairs >= 16 || pairs * chunks >= 256;
+    }
     if (mfma) {
         base_groups = (long long)a.G * ((a.num_kv_heads + 7) / 8);
     } else if (rows) {
