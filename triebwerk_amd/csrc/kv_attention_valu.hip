@@ -699,6 +699,7 @@ bool attention_rows_usable(const AttnArgs& a) {
     if (!al(a.k) || !al(a.v) || !al(a.q) || !al(a.out) || (a.q_stride & 7) != 0) return false;
     if (a.gate && (!al(a.gate) || (a.gate_stride & 7) != 0)) return false;
     if (a.k_new && (!al(a.k_new) || !al(a.v_new) || (a.kv_new_stride & 7) != 0)) return false;
+    if (a.ws && !al(a.ws)) return false;                         // 16-byte stores of the partials
     return true;
 }
 
