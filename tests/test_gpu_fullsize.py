@@ -216,6 +216,33 @@ def test_target_shape_fp16_cache(kv, oracle):
     print(f"fp16 cache, batch 64 x 8192: max rel err {worst:.2e}")
 
 
+@pytest.mark.parametrize("lens", [[8191, 8190, 8189, 8191, 8188], [8191, 7000, 4099, 100, 1]])
+def test_fp16_small_batch_long_context(kv, oracle, lens):
+    """Five sequences of up to 8192 tokens over the fp16 cache: the whole-row scan with its 64 chunks per sequence
+    (equal lengths) or its balanced walk (ragged), and the merge over up to 64 partials per head, with the append
+    inside the launch."""
+    import torch
+    G, H, Hk, msl = len(lens), 16, 8, 8192
+    kv_dim, q_dim = Hk * D, H * D
+    r = gen.rng(960 + lens[1] % 7)
+    ck, cv = gen.normal_f16(r, (G, msl, kv_dim)), gen.normal_f16(r, (G, msl, kv_dim))
+    pos = np.array(lens, np.int32)
+    for g in range(G):
+        ck[g, pos[g]:] = 0; cv[g, pos[g]:] = 0
+    q = gen.normal_f16(r, (G, q_dim)); k = gen.normal_f16(r, (G, kv_dim)); v = gen.normal_f16(r, (G, kv_dim))
+    d_ck, d_cv = dev(ck), dev(cv)
+    out = torch.zeros((G, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(G * H * msl, dtype=torch.float32, device="cuda")
+    kv.tw_append_attention_batch(out, dev(q), dev(k), dev(v), d_ck, d_cv, scratch, dev(pos), msl, G, H, Hk, D, q_dim, kv_dim)
+    assert kv.last_scan_kernel() == "attention_rows_kernel"
+    oracle.kv_cache_write_batch(ck, cv, k, v, pos, msl, G, kv_dim)
+    want = np.zeros((G, q_dim), np.float16)
+    oracle.gqa_attention_batch(want, q, ck, cv, pos, msl, G, H, Hk, D, q_dim, kv_dim)
+    assert np.array_equal(host(d_ck).view(np.uint16), ck.view(np.uint16)) and np.array_equal(host(d_cv).view(np.uint16), cv.view(np.uint16))
+    err = rel_err_rows(host(out), want)
+    assert err.max() <= TOL, f"max rel err {err.max():.3e} (per sequence {err})"
+
+
 @pytest.mark.parametrize("bits", [4, 2])
 def test_ragged_paged_batch64(kv, oracle, rotation_fixture, bits):
     """Contexts uniform in [512, 8192], 16-token pages in random order."""
