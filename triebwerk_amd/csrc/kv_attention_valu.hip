@@ -23,6 +23,9 @@
 //     goes to memory; V is accumulated in registers in the rotated basis and
 //     rotated back once per (sequence, head) (kernels.cu:1769-1775).
 // Arithmetic is fp32 throughout like the reference; only summation order differs.
+// The file holds two scan kernels -- attention_valu_kernel, which the list above describes, and attention_rows_kernel
+// for the fp16 cache with KV heads in eights (its waves read whole cache rows; described where it is defined) -- and
+// attention_merge_kernel, the log-sum-exp merge of either one's partial results.
 
 #include <algorithm>
 
