@@ -622,8 +622,10 @@ static FusedArgs fused_args(const tw_half* k_buf, const tw_half* v_buf, int kv_d
     return f;
 }
 
-static bool try_decode_fused(const AttnArgs& a, const FusedArgs& f, int msl, hipStream_t s, const char* fn) {
+static bool try_decode_fused(const AttnArgs& a, const FusedArgs& f_in, int msl, hipStream_t s, const char* fn) {
     const int mode = g_decode_fused.load();
+    FusedArgs f = f_in;
+    f.ctx_bound = t_ctx_max > 0 ? (t_ctx_max < msl ? t_ctx_max : msl) : msl;
     if (mode == 2 || g_variant.load() == 1) return false;
     if (!decode_fused_usable(a, f)) return false;
     if (mode != 1 && mode != 3 && !tw_kv_decode_step_plan(a.G, a.num_heads, a.num_kv_heads, a.bits, msl, t_ctx_min, t_ctx_max)) return false;

@@ -61,7 +61,10 @@ static_assert(8 * (2 + 4) * kStageStride <= kFusedMaxQ * kRowFloats * 4, "staged
 
 }  // namespace
 
-template <int R, int BITS, bool PROD, bool PAIR>
+// EARLY (PAIR only): waves ask for their first tile in the middle of the prologue; for launches whose waves have few
+// tiles (the host decides from what it knows of the context lengths).  A template parameter because the mere presence
+// of that path, never taken, made the long-context launch 2 us slower.
+template <int R, int BITS, bool PROD, bool PAIR, bool EARLY>
 __global__ void __launch_bounds__((PAIR ? kPairWaves : kFusedWaves) * kWave)
 decode_fused_kernel(AttnArgs a, FusedArgs f) {
     constexpr int NW = PAIR ? kPairWaves : kFusedWaves;        // waves of the workgroup
@@ -274,33 +277,49 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     uint32_t kreg[2][KW];
     uint32_t vreg[2][VW];
     uint32_t nreg = 0;
-    // (Tiles are only requested after the rotations.  Asking for the first one up front, without the row this
-    // workgroup is about to store, made launches 0.4 to 0.9 us slower at every context length, also with R
+    // (One head per wave: tiles are only requested after the rotations.  Asking for the first one up front, without the
+    // row this workgroup is about to store, made launches 0.4 to 0.9 us slower at every context length, also with R
     // arriving in 4 coalesced pieces per lane, and no faster when only the waves without a rotation to do ask;
     // pulling further tiles towards the caches during the prologue cost 2 us per tile: what the prologue waits
     // for then queues behind them.)
 
     // ---- 1. rotations of the unit's vectors
-    auto rotate_unit = [&]() {
+    // early(): called once the staged vectors and R are in LDS, before the rotations -- where the scan asks for its
+    // first tile when that tile lies wholly before the new token
+    auto rotate_unit = [&](auto early) {
         const int i16 = ln, kk = kg;
         const int dblk = rot_dblk;
-        // the centroid table while the loads are under way: entry e fills 256 bytes with replicas.  The centroids
-        // come out of a register by wave shuffle (lane c holds centroid c): indexing the constant array with a
-        // per-lane index is a dependent memory load per look-up, several microseconds for this loop.
-        for (int i = tid * 4; i < kTableWords; i += NW * kWave * 4) {
-            const int e = i >> 6;
-            if constexpr (BITS == 4) {
-                half2_t p = {(half_t)__shfl(cent_lane, e & 15, 64), (half_t)__shfl(cent_lane, e >> 4, 64)};
-                uint32_t w = *reinterpret_cast<uint32_t*>(&p);
-                *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
-            } else {
-                // a byte's four codes in the order 0, 2, 1, 3 (one head per wave: what its lane-pair exchange wants) or
-                // in their own order (two heads per wave)
-                const int f1 = PAIR ? 2 : 4, f2 = PAIR ? 4 : 2;
-                half2_t p0 = {(half_t)__shfl(cent_lane, e & 3, 64), (half_t)__shfl(cent_lane, (e >> f1) & 3, 64)};
-                half2_t p1 = {(half_t)__shfl(cent_lane, (e >> f2) & 3, 64), (half_t)__shfl(cent_lane, (e >> 6) & 3, 64)};
-                uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
-                *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
+        // the centroid table while the loads are under way: entry e fills 256 bytes with replicas.  A thread writes
+        // entries e0 + 4 NW k, k = 0, 1, ...: the low four bits of e are the thread's own in every round (their
+        // centroids come out of a register by wave shuffle, once: lane c holds centroid c; indexing the constant array
+        // with a per-lane index is a dependent memory load per look-up, several microseconds for this loop), the
+        // upper four are the same for the whole wave (v_readlane).
+        constexpr int kStep = NW * kWave * 4, kRounds = kTableWords / kStep;
+        static_assert(kRounds * kStep == kTableWords && kStep % 1024 == 0, "a round advances e by a multiple of 16");
+        const int e0 = tid >> 4, hi0 = uniform(tid >> 8);
+        auto cent_of = [&](int c) -> float {                // c uniform over the wave
+            return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cent_lane), c));
+        };
+        if constexpr (BITS == 4) {
+            const half_t lo = (half_t)__shfl(cent_lane, e0 & 15, 64);
+#pragma unroll
+            for (int k = 0; k < kRounds; k++) {
+                half2_t p = {lo, (half_t)cent_of(hi0 + (NW / 4) * k)};
+                const uint32_t w = *reinterpret_cast<uint32_t*>(&p);
+                *reinterpret_cast<uint4*>(&tab_s[tid * 4 + k * kStep]) = uint4{w, w, w, w};
+            }
+        } else {
+            // a byte's four codes in the order 0, 2, 1, 3 (one head per wave: what its lane-pair exchange wants) or
+            // in their own order (two heads per wave)
+            const half_t c0 = (half_t)__shfl(cent_lane, e0 & 3, 64), c1 = (half_t)__shfl(cent_lane, (e0 >> 2) & 3, 64);
+#pragma unroll
+            for (int k = 0; k < kRounds; k++) {
+                const int hi = hi0 + (NW / 4) * k;          // e >> 4
+                const half_t c2 = (half_t)cent_of(hi & 3), c3 = (half_t)cent_of(hi >> 2);
+                half2_t p0 = {c0, PAIR ? c1 : c2};
+                half2_t p1 = {PAIR ? c2 : c1, c3};
+                const uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
+                *reinterpret_cast<uint4*>(&tab_s[tid * 4 + k * kStep]) = uint4{w0, w1, w0, w1};
             }
         }
 
@@ -311,6 +330,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         if (PROD && prod_live) *reinterpret_cast<uint4*>(&prod_s[prod_row][8 * prod_piece]) = prod;
         if (wave < 8) stage_operand_tile(rot_s + wave * kOperandTileDwords, rraw, lane);
         lds_barrier();
+        early();
         float rv[32];                                      // R[16 * rot_dblk + ln][4s + kg]
         if (rotating) read_operand_tile(rot_s + rot_dblk * kOperandTileDwords, lane, rv);
         if (PROD) {
@@ -465,11 +485,22 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         // with one head per wave; the scores of tile i + 1 placed beside the P.V of tile i for the scheduler to
         // interleave, 3 % slower.)
         PairTileRegs<BITS> t;
-        rotate_unit();
-        set_next(0);
-        issue_k(t);
-        issue_n(t);
-        issue_v(t);
+        // EARLY: a wave asks for its first tile in the middle of the prologue, behind the prologue's own loads
+        // and ahead of the rotations, when all of its rows are older than the token this launch appends (the launch's
+        // own row only exists after the barrier that ends the rotations).  Rollouts of a few hundred tokens gain
+        // 4.5 % (128 sequences at 257..768 tokens: 21.6 against 22.6 us per launch); with 8 tiles per wave it makes no
+        // difference, and with 16 and more the launch gets slower (64 x 4096 tokens: + 0.6 us, x 8192: + 2.2 us), as
+        // with every other way of putting more requests in flight at the start that was tried.
+        const bool first_early = EARLY && ntiles > 0 && tile_at(0) + 32 <= pos;      // uniform over the wave
+        rotate_unit([&]() {
+            if (first_early) { set_next(0); issue_k(t); issue_n(t); issue_v(t); }
+        });
+        if (!first_early) {
+            set_next(0);
+            issue_k(t);
+            issue_n(t);
+            issue_v(t);
+        }
         load_rb();              // behind the first tile's loads; the registers are there, and the epilogue need not wait
         if (ntiles > 0) {
             S.load_query(L, [&](int i) -> const float* { return &qrot_s[hk_local * R + i][0]; });
@@ -487,7 +518,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             if ((L.pn & 7) == 0) { pr[kHeadDim] = S.m_run[r]; pr[kHeadDim + 1] = S.l_run[r]; }
         });
     } else {
-        rotate_unit();
+        rotate_unit([]() {});
         {
             int l2 = lane;
             asm volatile("" : "+v"(l2));
@@ -814,15 +845,20 @@ void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s
     const bool pair = allow_pairs && decode_fused_pairs(a, f.hkw);
     const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw))), b3((pair ? kPairWaves : kFusedWaves) * kWave);
     const bool prod = f.q_weight != nullptr || f.cos_table != nullptr;
+    // first tile in the middle of the prologue: when no wave gets more than 8 tiles of 32 tokens by the caller's bound
+    // of the context (two heads per wave: 16 / hkw parts per head)
+    const bool early = pair && f.ctx_bound > 0 && f.ctx_bound <= 8 * 32 * (2 * kPairWaves / f.hkw);
     note_scan_kernel(pair ? "decode_fused_kernel, two KV heads per wave" : "decode_fused_kernel, one KV head per wave");
-#define TW_FUSED(RR, BB, PP) \
-    do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true, PP>, g3, b3, s, a, f); \
-         else launch_scan_kernel(decode_fused_kernel<RR, BB, false, PP>, g3, b3, s, a, f); } while (0)
+#define TW_FUSED_E(RR, BB, PP, EE) \
+    do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true, PP, EE>, g3, b3, s, a, f); \
+         else launch_scan_kernel(decode_fused_kernel<RR, BB, false, PP, EE>, g3, b3, s, a, f); } while (0)
+#define TW_FUSED(RR, BB, PP) do { if (PP && early) TW_FUSED_E(RR, BB, PP, PP); else TW_FUSED_E(RR, BB, PP, false); } while (0)
 #define TW_FUSED_R(BB, PP) do { if (R == 1) TW_FUSED(1, BB, PP); else if (R == 2) TW_FUSED(2, BB, PP); else TW_FUSED(4, BB, PP); } while (0)
     if (a.bits == 4) { if (pair) TW_FUSED_R(4, true); else TW_FUSED_R(4, false); }
     else { if (pair) TW_FUSED_R(2, true); else TW_FUSED_R(2, false); }
 #undef TW_FUSED_R
 #undef TW_FUSED
+#undef TW_FUSED_E
 }
 
 }  // namespace twkv

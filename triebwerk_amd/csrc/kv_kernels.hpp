@@ -193,6 +193,7 @@ struct FusedArgs {
     uint8_t* v_codes;
     half_t* k_norms;
     half_t* v_norms;
+    int ctx_bound;          // in: upper bound of positions + 1 that the host knows (0: none)
     int hkw;                // KV heads per workgroup (launch_decode_fused fills this in)
     float q_scale;          // likewise
     // optional producers of q and k applied on the way in, as RotArgs has them (V rows stay as they are)
