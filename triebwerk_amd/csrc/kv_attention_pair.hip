@@ -225,20 +225,8 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
         issue_first();
         ready = true;
     }
-    // ---- dequantization table, once per workgroup: entry e fills 256 bytes with replicas
-    for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
-        const int e = i >> 6;
-        if constexpr (BITS == 4) {
-            half2_t pc = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
-            uint32_t w = *reinterpret_cast<uint32_t*>(&pc);
-            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
-        } else {                                         // a byte's four centroids in their own order, 32 replicas of 8 bytes
-            half2_t p0 = {(half_t)(kAlpha * kCentroids2[e & 3]), (half_t)(kAlpha * kCentroids2[(e >> 2) & 3])};
-            half2_t p1 = {(half_t)(kAlpha * kCentroids2[(e >> 4) & 3]), (half_t)(kAlpha * kCentroids2[e >> 6])};
-            uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
-            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
-        }
-    }
+    // ---- dequantization table, once per workgroup
+    build_centroid_table<BITS, true>(tab_s, kAlpha, tid, nthreads);
     for (int i = tid; i < kPairScanWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
     __syncthreads();             // the only workgroup-wide barrier; every wave reaches it
 

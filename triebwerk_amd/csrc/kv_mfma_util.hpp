@@ -60,4 +60,31 @@ constexpr int kStreamNorms = 0;
 // compute units of the current device (cached; kv_attention_mfma.hip)
 int compute_units();
 
+// The dequantization table of the MFMA scans, built by the nthreads threads of a workgroup: entry e (a cache byte)
+// fills 256 bytes with replicas of its centroids as fp16 -- 4 bit: 64 replicas of (low code, high code); 2 bit: 32
+// replicas of the byte's four codes, in their own order (NATURAL) or as 0, 2, 1, 3.  The centroids come out of a
+// register by wave shuffle (lane c holds centroid c, scaled): indexing the constant arrays with a per-lane index is a
+// dependent memory load per look-up, microseconds for this loop.  Lower lanes run at least as many rounds as higher
+// ones, so the lanes the shuffles read (0..15) are active whenever any lane is.
+template <int BITS, bool NATURAL>
+__device__ __forceinline__ void build_centroid_table(uint32_t* tab_s, float alpha, int tid, int nthreads) {
+    const int lane = tid & 63;
+    const float cent_lane = alpha * (BITS == 4 ? kCentroids4[lane & 15] : kCentroids2[lane & 3]);
+    auto cent = [&](int c) -> half_t { return (half_t)__shfl(cent_lane, c, 64); };
+    for (int i = tid * 4; i < kTableWords; i += nthreads * 4) {
+        const int e = i >> 6;
+        if constexpr (BITS == 4) {
+            half2_t p = {cent(e & 15), cent(e >> 4)};
+            const uint32_t w = *reinterpret_cast<uint32_t*>(&p);
+            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w, w, w, w};
+        } else {
+            constexpr int f1 = NATURAL ? 2 : 4, f2 = NATURAL ? 4 : 2;
+            half2_t p0 = {cent(e & 3), cent((e >> f1) & 3)};
+            half2_t p1 = {cent((e >> f2) & 3), cent((e >> 6) & 3)};
+            const uint32_t w0 = *reinterpret_cast<uint32_t*>(&p0), w1 = *reinterpret_cast<uint32_t*>(&p1);
+            *reinterpret_cast<uint4*>(&tab_s[i]) = uint4{w0, w1, w0, w1};
+        }
+    }
+}
+
 }  // namespace twkv
