@@ -216,13 +216,15 @@ def test_target_shape_fp16_cache(kv, oracle):
     print(f"fp16 cache, batch 64 x 8192: max rel err {worst:.2e}")
 
 
+@pytest.mark.parametrize("H,Hk", [(16, 8), (32, 16)])
 @pytest.mark.parametrize("lens", [[8191, 8190, 8189, 8191, 8188], [8191, 7000, 4099, 100, 1]])
-def test_fp16_small_batch_long_context(kv, oracle, lens):
+def test_fp16_small_batch_long_context(kv, oracle, lens, H, Hk):
     """Five sequences of up to 8192 tokens over the fp16 cache: the whole-row scan with its 64 chunks per sequence
     (equal lengths) or its balanced walk (ragged), and the merge over up to 64 partials per head, with the append
-    inside the launch."""
+    inside the launch.  With 16 KV heads a sequence's chunks are two workgroups' work each, more items than the grid
+    holds at once, and there is no balanced walk."""
     import torch
-    G, H, Hk, msl = len(lens), 16, 8, 8192
+    G, msl = len(lens), 8192
     kv_dim, q_dim = Hk * D, H * D
     r = gen.rng(960 + lens[1] % 7)
     ck, cv = gen.normal_f16(r, (G, msl, kv_dim)), gen.normal_f16(r, (G, msl, kv_dim))
