@@ -33,29 +33,19 @@ static const float kCentroids4Host[16] = {
     -0.24155f, -0.18293f, -0.14304f, -0.11099f, -0.08330f, -0.05806f, -0.03432f, -0.01135f,
     0.01135f,  0.03432f,  0.05806f,  0.08330f,  0.11099f,  0.14304f,  0.18293f,  0.24155f};
 
-// turbo_quantize of the reference (kernels.cu:1448-1473) with the boundaries as
-// immediates: strict `<` for 4 bits (a value on a boundary goes up, NaN -> 15),
-// a count of `>=` for 2 bits (NaN -> 0).
+// turbo_quantize of the reference (kernels.cu:1448-1473) with the boundaries as immediates.  The reference walks a
+// tree of strict `<` comparisons for 4 bits (a value on a boundary goes up, NaN -> 15) and counts `>=` for 2 bits
+// (NaN -> 0).  The tree's answer is the number of boundaries b, in their sorted order, with !(val < b) -- the values
+// below a boundary form a lower set -- and that count is what is computed here: 15 compare-and-add pairs without a
+// branch, where the tree as written costs a wave whose lanes disagree every one of its 15 nodes with the branching
+// around them (2 us per decode launch for the four values per lane of a rotation).
 __device__ __forceinline__ int turbo_quantize(float val, int bits) {
     if (bits == 4) {
-        int idx;
-        if (val < 0.00000f) {
-            if (val < -0.09715f) {
-                if (val < -0.16299f) idx = val < -0.21224f ? 0 : 1;
-                else idx = val < -0.12701f ? 2 : 3;
-            } else {
-                if (val < -0.04619f) idx = val < -0.07068f ? 4 : 5;
-                else idx = val < -0.02284f ? 6 : 7;
-            }
-        } else {
-            if (val < 0.09715f) {
-                if (val < 0.04619f) idx = val < 0.02284f ? 8 : 9;
-                else idx = val < 0.07068f ? 10 : 11;
-            } else {
-                if (val < 0.16299f) idx = val < 0.12701f ? 12 : 13;
-                else idx = val < 0.21224f ? 14 : 15;
-            }
-        }
+        constexpr float kB[15] = {-0.21224f, -0.16299f, -0.12701f, -0.09715f, -0.07068f, -0.04619f, -0.02284f, 0.00000f,
+                                  0.02284f,  0.04619f,  0.07068f,  0.09715f,  0.12701f,  0.16299f,  0.21224f};
+        int idx = 0;
+#pragma unroll
+        for (int i = 0; i < 15; i++) idx += !(val < kB[i]) ? 1 : 0;
         return idx;
     }
     return (int)(val >= -0.08677f) + (int)(val >= 0.0f) + (int)(val >= 0.08677f);
