@@ -248,7 +248,7 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
     // merge, and the scan at its rate.
     const double bpt = bits == 4 ? 132.0 : 68.0;                  // bytes per token and KV head: K and V codes and norms
     const double one = decode_fused_estimate_us(G, num_heads, num_kv_heads, bits, allow_pairs, hkw, ctx_max);
-    const double three = 27.0 + (double)G * num_kv_heads * bpt * ctx_max / (bits == 4 ? 7.4e6 : 5.8e6);
+    const double three = 27.0 + (double)G * num_kv_heads * bpt * ctx_max / (bits == 4 ? 7.2e6 : 5.8e6);
     return one <= three ? 1 : 0;
 }
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }

@@ -789,7 +789,7 @@ bool decode_fused_pairs(const AttnArgs& a, int hkw) { return pairs_fit(a.bits, a
 
 // Microseconds one launch takes for G sequences of ctx tokens with hkw KV heads per workgroup, by a count fitted to
 // launches measured on MI355X at batches 16 to 256 and contexts 1k to 8k (it reproduces them within 5 %): the
-// workgroups run in rounds of one per CU; a round costs 13 us of prologue and epilogue and, per token of context, the
+// workgroups run in rounds of one per CU; a round costs 12 us of prologue and epilogue and, per token of context, the
 // cube-root sum of what one CU sustains for the workgroup's heads (a workgroup whose waves scan one head each moves
 // its bytes at about half the rate of one whose waves scan two) and of the whole chip's rate for all the workgroups
 // of the round.
@@ -802,7 +802,7 @@ double decode_fused_estimate_us(int G, int num_heads, int Hk, int bits, bool all
     const bool pair = allow_pairs && pairs_fit(bits, R, hkw);
     const double per_head_ns = pair ? (bits == 4 ? 3.08 : 2.88) : (bits == 4 ? 5.95 : 4.68);
     const double k_cu = hkw * per_head_ns, k_bw = active * hkw * bpt / (bits == 4 ? 7200.0 : 5240.0);   // ns per token
-    return rounds * (13.0 + ctx * 1e-3 * std::cbrt(k_cu * k_cu * k_cu + k_bw * k_bw * k_bw));
+    return rounds * (12.0 + ctx * 1e-3 * std::cbrt(k_cu * k_cu * k_cu + k_bw * k_bw * k_bw));
 }
 
 // KV heads per workgroup (8, 4, 2 or 1): the choice with the smallest estimate at a context of 4096 tokens (the order
