@@ -194,8 +194,8 @@ const char* tw_kv_debug_last_scan_kernel(void);
  * cheaper of the two by estimates fitted to measured launches (one launch: rounds of one workgroup per CU, each the
  * time a workgroup needs for its heads of one sequence; three launches: their fixed cost plus the scan at its rate).
  * At 8 KV heads of 128 and a context of 8192 that is one launch for batches of about 40 to 64 sequences and again at
- * 128 (whole rounds of one workgroup per CU) at 4 bit, and three for smaller ones, which leave CUs idle, and for those
- * in between; at 4096 tokens one launch up to batch 128.
+ * 128 (whole rounds of one workgroup per CU) at 4 bit, at batches 64 and 128 at 2 bit, and three for smaller ones,
+ * which leave CUs idle, and for those in between; at 4096 tokens one launch up to batch 128 at both widths.
  * Alignment of the buffers, which the entry point also checks, is not part of it. */
 int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max);
 /* Layer steps that took the one-launch kernel since the library was loaded (launches issued or recorded into a

@@ -97,7 +97,11 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     // rather than skipped by a branch).  Paged cache: a tile is two 16-token pages, each with its own descriptor; the
     // two block-table entries of a tile are fetched one tile ahead (even lanes the first page, odd lanes the second),
     // before the loads of the tile in between, so they have returned, in order, by the time they are needed.  Past
-    // the end the last page is re-read (its tokens are masked).
+    // the end the last page is re-read (its tokens are masked).  After a chunk's last tile the loads are still issued,
+    // through descriptors of no bytes (`live` false: zeros, no traffic), and the block table is read again at the
+    // chunk's last entry: with every load of the loop unconditional the compiler knows how many are in flight when
+    // the entries are needed and waits for exactly those before them -- with the loads under `if (more)` it waited
+    // for all of them, the next tile's included, at the end of every tile (9 % of the 2-bit paged scan, 2 % at 4 bit).
     auto fetch_pages = [&](int ts) -> int { return bt[min(ts + 16 * (lane & 1), t1 - 1) >> 4]; };
     auto page_row = [&](int pages, int sub) -> long long {
         return (long long)__builtin_amdgcn_readlane(pages, sub) * kPageTokens;
@@ -113,11 +117,11 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
         if constexpr (BITS == 4) return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kCodesAux);
         else return __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, kCodesAux);
     };
-    auto issue_k = [&](PairTileRegs<BITS>& t, int tile, int pages) {
+    auto issue_k = [&](PairTileRegs<BITS>& t, int tile, int pages, bool live = true) {
         if (PAGED) {
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
-                __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + page_row(pages, sub) * kvp, kPageTokens * (int)kvp);
+                __amdgpu_buffer_rsrc_t r = make_rsrc(kpair + page_row(pages, sub) * kvp, live ? kPageTokens * (int)kvp : 0);
                 t.k[2 * sub] = load_k(r, koff);
                 t.k[2 * sub + 1] = load_k(r, koff + 8u * kvp);
             }
@@ -127,11 +131,11 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
             for (int c = 0; c < 4; c++) t.k[c] = load_k(r, koff + (uint32_t)(8 * c) * kvp);
         }
     };
-    auto issue_v = [&](PairTileRegs<BITS>& t, int tile, int pages) {
+    auto issue_v = [&](PairTileRegs<BITS>& t, int tile, int pages, bool live = true) {
         if (PAGED) {
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
-                __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + page_row(pages, sub) * kvp, kPageTokens * (int)kvp);
+                __amdgpu_buffer_rsrc_t r = make_rsrc(vpair + page_row(pages, sub) * kvp, live ? kPageTokens * (int)kvp : 0);
 #pragma unroll
                 for (int j = 0; j < 4; j++) t.v[sub][j] = load_v(r, voff + (uint32_t)j * kvp);
             }
@@ -146,12 +150,12 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
         }
     };
     // the pair's two fp16 norms of tokens tok0 and tok0 + 16, K and V
-    auto issue_n = [&](PairTileRegs<BITS>& t, int tile, int pages) {
+    auto issue_n = [&](PairTileRegs<BITS>& t, int tile, int pages, bool live = true) {
         if (PAGED) {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + page_row(pages, i) * nrow, kPageTokens * (int)nrow);
-                __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + page_row(pages, i) * nrow, kPageTokens * (int)nrow);
+                __amdgpu_buffer_rsrc_t rk = make_rsrc(knpair + page_row(pages, i) * nrow, live ? kPageTokens * (int)nrow : 0);
+                __amdgpu_buffer_rsrc_t rv = make_rsrc(vnpair + page_row(pages, i) * nrow, live ? kPageTokens * (int)nrow : 0);
                 t.n[i][0] = __builtin_amdgcn_raw_buffer_load_b32(rk, (int)noff, 0, kStreamNorms);
                 t.n[i][1] = __builtin_amdgcn_raw_buffer_load_b32(rv, (int)noff, 0, kStreamNorms);
             }
@@ -268,11 +272,11 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
             int pages = 0;
             if (PAGED) {
                 pages = pages_next;                                  // the next tile's pages, already here
-                if (more) pages_next = fetch_pages(tile + 64);       // and the one after: before the next tile's loads
+                pages_next = fetch_pages(tile + 64);                 // and the one after: before the next tile's loads
             }
             if (PAGED) {
-                pair_scan_tile<R>(L, S, t, tile, n, [&]() { if (more) issue_k(t, tile + 32, pages); },
-                                  [&]() { if (more) issue_n(t, tile + 32, pages); }, [&]() { if (more) issue_v(t, tile + 32, pages); });
+                pair_scan_tile<R>(L, S, t, tile, n, [&]() { issue_k(t, tile + 32, pages, more); },
+                                  [&]() { issue_n(t, tile + 32, pages, more); }, [&]() { issue_v(t, tile + 32, pages, more); });
             } else {
                 const int rows = more ? tile_rows(tile + 32) : 0;
                 pair_scan_tile<R>(L, S, t, tile, n, [&]() { issue_k(t, tile + 32, rows); }, [&]() { issue_n(t, tile + 32, rows); },

@@ -244,11 +244,11 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
     if (bound <= 256 * split) return 1;                           // at most 8 tiles of 32 tokens per wave
     if (!known || (long long)(ctx_max - ctx_min) * 8 > ctx_max) return 0;   // lengths unknown or ragged: the balanced walk
     // Equal lengths: the cheaper of the two by estimates fitted to launches measured on MI355X (microseconds per
-    // layer): one launch as decode_fused_estimate_us counts it; three launches: 27 us of launches, query rotation and
-    // merge, and the scan at its rate.
+    // layer): one launch as decode_fused_estimate_us counts it; three launches: 27 us (25 at 2 bit) of launches, query
+    // rotation and merge, and the scan at its rate.
     const double bpt = bits == 4 ? 132.0 : 68.0;                  // bytes per token and KV head: K and V codes and norms
     const double one = decode_fused_estimate_us(G, num_heads, num_kv_heads, bits, allow_pairs, hkw, ctx_max);
-    const double three = 27.0 + (double)G * num_kv_heads * bpt * ctx_max / (bits == 4 ? 7.2e6 : 5.8e6);
+    const double three = (bits == 4 ? 27.0 : 25.0) + (double)G * num_kv_heads * bpt * ctx_max / (bits == 4 ? 7.2e6 : 5.4e6);
     return one <= three ? 1 : 0;
 }
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }

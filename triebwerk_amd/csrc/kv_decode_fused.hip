@@ -800,8 +800,8 @@ double decode_fused_estimate_us(int G, int num_heads, int Hk, int bits, bool all
     const double units = (double)G * (Hk / hkw);
     const double rounds = std::ceil(units / cus), active = units < cus ? units : cus;
     const bool pair = allow_pairs && pairs_fit(bits, R, hkw);
-    const double per_head_ns = pair ? (bits == 4 ? 3.08 : 2.88) : (bits == 4 ? 5.95 : 4.68);
-    const double k_cu = hkw * per_head_ns, k_bw = active * hkw * bpt / (bits == 4 ? 7200.0 : 5240.0);   // ns per token
+    const double per_head_ns = pair ? (bits == 4 ? 3.08 : hkw >= 4 ? 2.45 : 2.72) : (bits == 4 ? 5.95 : 4.68);
+    const double k_cu = hkw * per_head_ns, k_bw = active * hkw * bpt / (bits == 4 ? 7200.0 : 5500.0);   // ns per token
     return rounds * (12.0 + ctx * 1e-3 * std::cbrt(k_cu * k_cu * k_cu + k_bw * k_bw * k_bw));
 }
 

@@ -143,28 +143,44 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R, BITS>& L, PairS
     constexpr float kRaise = 5.0f;                     // raise the running max only past 2^5
     // ---- scores: set c = tokens 8c .. 8c+7 of both heads
     float4_t s[4];
+    if constexpr (BITS == 2) {
+        // operand i = 4 c + j: bytes 2 (j % 2) and + 1 of dword j / 2 of the lane's 8 bytes of set c, dims 8j .. 8j + 7.
+        // The look-ups run kAheadK operands ahead of the MFMAs (see the P.V loop below).
+        constexpr int kAheadK = 4;
+        uint2 klo[kAheadK], khi[kAheadK];
+        auto look = [&](int i, uint2& lo, uint2& hi) {
+            const uint32_t w = t.k[i >> 2][(i & 3) >> 1];
+            const uint32_t sel = 0x0c0c0400u + ((uint32_t)(2 * (i & 1)) << 8);
+            lo = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel));
+            hi = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel + 0x100u));
+        };
+#pragma unroll
+        for (int i = 0; i < kAheadK; i++) look(i, klo[i], khi[i]);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            union { uint32_t u[4]; half8_t h; } kv;
+            kv.u[0] = klo[i % kAheadK].x; kv.u[1] = klo[i % kAheadK].y; kv.u[2] = khi[i % kAheadK].x; kv.u[3] = khi[i % kAheadK].y;
+            if (i + kAheadK < 16) look(i + kAheadK, klo[i % kAheadK], khi[i % kAheadK]);
+            asm volatile("" ::: "memory");
+            if ((i & 3) == 0) s[i >> 2] = float4_t{0.f, 0.f, 0.f, 0.f};
+            s[i >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(S.aq[i & 3], kv.h, s[i >> 2], 0, 0, 0);
+        }
+    } else {
 #pragma unroll
     for (int c = 0; c < 4; c++) {
         union { uint32_t u[4]; half8_t h; } kv[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            if constexpr (BITS == 4) {
-                const uint32_t w = t.k[c][j];
-                kv[j].u[0] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0400u));
-                kv[j].u[1] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0500u));
-                kv[j].u[2] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0600u));
-                kv[j].u[3] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0700u));
-            } else {                                            // bytes 2j and 2j + 1 of the lane's 8: dims 8j .. 8j + 7
-                const uint32_t w = t.k[c][j >> 1];
-                const uint32_t sel = 0x0c0c0400u + ((uint32_t)(2 * (j & 1)) << 8);
-                const uint2 lo = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel));
-                const uint2 hi = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel + 0x100u));
-                kv[j].u[0] = lo.x; kv[j].u[1] = lo.y; kv[j].u[2] = hi.x; kv[j].u[3] = hi.y;
-            }
+            const uint32_t w = t.k[c][j];
+            kv[j].u[0] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0400u));
+            kv[j].u[1] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0500u));
+            kv[j].u[2] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0600u));
+            kv[j].u[3] = L.lut32(__builtin_amdgcn_perm(w, L.lane_rep, 0x0c0c0700u));
         }
         s[c] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 4; j++) s[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(S.aq[j], kv[j].h, s[c], 0, 0, 0);
+    }
     }
     after_k();
     // Wave priority rises as the tile advances (scores 0, softmax 1, P.V 2): of the two waves of a SIMD the one
@@ -285,15 +301,26 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R, BITS>& L, PairS
         y[sub][3] = ((xo01 >> 4) & 0x0f0f0f0fu) | (xo23 & 0xf0f0f0f0u);        // dims 3, 7, 11, 15
     }
     after_v();
-#pragma unroll
-    for (int j = 0; j < 16; j++) {
+    // The look-ups run kAhead operands ahead of the MFMAs, held there by an empty asm statement the scheduler does not
+    // move LDS reads across: left alone it sinks every look-up next to its MFMA and the wave waits out the LDS
+    // latency sixteen times per tile.
+    constexpr int kAhead = 4;
+    uint2 qa[kAhead], qb[kAhead];
+    auto look = [&](int j, uint2& a4, uint2& b4) {
         constexpr int kWhich[4] = {0, 2, 1, 3};
         const int m = kWhich[j & 3];
         const uint32_t sel = 0x0c0c0400u + ((uint32_t)(j >> 2) << 8);
-        const uint2 a4 = L.lut64(__builtin_amdgcn_perm(y[0][m], L.lane_rep, sel));
-        const uint2 b4 = L.lut64(__builtin_amdgcn_perm(y[1][m], L.lane_rep, sel));
+        a4 = L.lut64(__builtin_amdgcn_perm(y[0][m], L.lane_rep, sel));
+        b4 = L.lut64(__builtin_amdgcn_perm(y[1][m], L.lane_rep, sel));
+    };
+#pragma unroll
+    for (int j = 0; j < kAhead; j++) look(j, qa[j], qb[j]);
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
         union { uint32_t u[4]; half8_t h; } bv;
-        bv.u[0] = a4.x; bv.u[1] = a4.y; bv.u[2] = b4.x; bv.u[3] = b4.y;
+        bv.u[0] = qa[j % kAhead].x; bv.u[1] = qa[j % kAhead].y; bv.u[2] = qb[j % kAhead].x; bv.u[3] = qb[j % kAhead].y;
+        if (j + kAhead < 16) look(j + kAhead, qa[j % kAhead], qb[j % kAhead]);
+        asm volatile("" ::: "memory");
         S.o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa.h, bv.h, S.o[j], 0, 0, 0);
     }
     }
