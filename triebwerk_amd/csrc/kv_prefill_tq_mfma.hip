@@ -99,7 +99,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
     // (64 contiguous bytes, all banks different); with the K mapping they would hit rows 8 apart, 8 to a bank
     const int vr_ = tid & 15, vc_ = tid >> 4;
     constexpr int kPiece = BITS;                           // bytes of codes of 8 coordinates
-    struct Staged { uint32_t k[2], v[2]; float nrm; };
+    struct Staged { uint32_t k[2], v[2], nb; };            // codes, and the fp16 bits of a norm as loaded
     // Buffer loads: descriptors over the T rows of the cache (rows past the last token read as zeros and are
     // masked anyway), per-thread byte offsets fixed for the whole kernel, the tile's row offset in a scalar.
     const __amdgpu_buffer_rsrc_t krs = make_rsrc(kbase, T * row_bytes - kvh * kHeadBytes);
@@ -110,6 +110,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
     const int koff0 = sr * row_bytes + kPiece * sc, koff1 = koff0 + 16 * row_bytes;
     const int voff0 = 2 * vr_ * row_bytes + kPiece * vc_, voff1 = voff0 + row_bytes;
     const int noff = (tid & 31) * nrow_bytes;
+    const __amdgpu_buffer_rsrc_t nrs = (wave & 1) ? vnrs : knrs;     // wave-uniform: a scalar choice
     auto load_codes = [&](__amdgpu_buffer_rsrc_t rs, int voff, int soff) -> uint32_t {
         if constexpr (BITS == 4) return __builtin_amdgcn_raw_buffer_load_b32(rs, voff, soff, 0);
         else return __builtin_amdgcn_raw_buffer_load_b16(rs, voff, soff, 0);
@@ -120,8 +121,11 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         st.k[1] = load_codes(krs, koff1, toff);
         st.v[0] = load_codes(vrs, voff0, toff);
         st.v[1] = load_codes(vrs, voff1, toff);
-        if (tid < 32) st.nrm = h2f_bits(__builtin_amdgcn_raw_buffer_load_b16(knrs, noff, tile * nrow_bytes, 0));
-        else if (tid < 64) st.nrm = h2f_bits(__builtin_amdgcn_raw_buffer_load_b16(vnrs, noff, tile * nrow_bytes, 0));
+        // Every thread asks for a norm of row tid % 32 -- even waves K's, odd waves V's; lanes 0..31 of waves 0 and 1
+        // are the ones that keep it -- and holds the bits as they come: a load under a per-lane condition with a
+        // descriptor that depends on the lane becomes a loop over the descriptors, and a value computed from a load
+        // at the place of the load is a wait for every load in flight, here the tile that was just asked for.
+        st.nb = __builtin_amdgcn_raw_buffer_load_b16(nrs, noff, tile * nrow_bytes, 0);
     };
     const int vcol = 2 * vt_slot(2 * vr_);                  // byte column of the token pair in a V^T row
     auto stash = [&](int buf, int vbuf, const Staged& st) {
@@ -139,7 +143,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
             *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x07060302u);
         }
-        if (tid < 64) n_s[vbuf][tid >> 5][tid & 31] = st.nrm;
+        if (tid < 2 * kWave && (tid & 32) == 0) n_s[vbuf][tid >> 6][tid & 31] = h2f_bits(st.nb);
     };
     __syncthreads();                                       // the table is there
 
