@@ -267,7 +267,7 @@ def paged_bench(args):
     L, H, Hk, G, D = w["L"], w["H"], w["Hk"], w["G"], 128
     K, W = args.steps, args.warmup
     kv_dim, q_dim, kvp = Hk * D, H * D, Hk * D * kv_bits // 8
-    total_steps = W + K + K + 2
+    total_steps = W + K + max(1, min(K, 4096 // L, args.profile_steps or K)) + 2
     msl = (w["ctx"] + total_steps + 255) // 256 * 256
     pages_per_seq, n_pages = msl // 16, G * msl // 16
     lib = _lib.load()
@@ -338,7 +338,7 @@ def paged_bench(args):
     step_bytes = algorithmic_bytes(n_tokens_timed, G * K, L, H, Hk, kv_bits, with_append=True) / K
     step_gbs = step_bytes / (elapsed / K) * 1e-9
 
-    Kp = max(1, min(K, 4096 // L))
+    Kp = max(1, min(K, 4096 // L, args.profile_steps or K))
     lib.tw_kv_debug_profile_attention(1)
     with torch.cuda.stream(stream):
         for _ in range(Kp):
@@ -353,7 +353,9 @@ def paged_bench(args):
     kern_ms = total_ms.value / launches.value
     launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=False) / (Kp * L)
     achieved = launch_bytes / (kern_ms * 1e-3) * 1e-9
-    print(json.dumps({
+    del pools, q, k, v, ws
+    torch.cuda.empty_cache()
+    return {
         "metric": "decode-attn tokens/s", "value": G * K / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": K,
         "warmup": W, "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": DTYPE[kv_bits], "data": "synthetic",
@@ -361,6 +363,7 @@ def paged_bench(args):
                    "kv_bits": kv_bits, "layers": L, "num_heads": H, "num_kv_heads": Hk, "head_dim": D, "batch": G,
                    "pages": n_pages, "context_first_timed_step": [int(ctx0.min()), int(ctx0.max())],
                    "tokens_attended_per_step": n_tokens_timed / K, "hipgraph": use_graph,
+                   "launches_per_layer": 4 if args.launchers == "reference" else 3,
                    "step": ("paged append K,V + paged decode attention for every layer (two calls, four launches), positions += 1"
                             if args.launchers == "reference" else
                             "tw_paged_turbo_append_attention_batch for every layer (three launches), positions += 1")},
@@ -370,7 +373,7 @@ def paged_bench(args):
                      "kernel_name": scan_kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "launch_ms": kern_ms, "launch_algorithmic_MB": launch_bytes * 1e-6, "traffic": None},
-    }))
+    }
 
 
 def main():
@@ -411,6 +414,12 @@ def main():
                     help="with --prefill: 0 time the attention launch alone, 1 the whole layer over the prompt through "
                          "tw_layer_prompt_step (QK norm, RoPE, T-token append, attention), 2 the same as the reference's "
                          "sequence of launchers")
+    ap.add_argument("--profile-steps", type=int, default=None,
+                    help="eager steps after the timed region whose scan launches are timed one by one with HIP events "
+                         "(default: as many as --steps, at most 4096 launches)")
+    ap.add_argument("--per-config", action="store_true",
+                    help="also measure the BASELINE configs 1-5 (and the reference's launchers at the target shape) with "
+                         "few steps each and report them under per_config; the default run does this")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="instead of the decode step, time causal prefill attention over a T-token prompt of one "
                          "sequence (one layer's launch, the workload's head counts, --kv-bits cache) and exit")
@@ -436,7 +445,7 @@ def main():
               "inside the path, and is not implemented. Use --gpus 1.", file=sys.stderr)
         sys.exit(2)
     if args.paged:
-        paged_bench(args)
+        print(json.dumps(paged_bench(args)))
         return
 
     headline_bits = WORKLOADS[args.workload]["kv_bits"] if args.kv_bits is None else args.kv_bits
@@ -452,6 +461,8 @@ def main():
             if bits != headline_bits:
                 per[str(bits if bits else 16)] = compact(decode_bench(args, bits, with_probe=False))
         result["per_kv_bits"] = {k: per[k] for k in ("16", "4", "2") if k in per}
+    if default_run or args.per_config:
+        result["per_config"] = per_config(args)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(workload_of(args), headline_bits)
     print(json.dumps(result))
@@ -461,8 +472,44 @@ def compact(r):
     """The figures of one cache width for the per_kv_bits table."""
     return {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "step_achieved_GBps": r["step_achieved_GBps"],
             "step_frac_of_hbm_peak": r["step_frac_of_hbm_peak"], "dtype": r["dtype"], "launches_per_layer": r["config"]["launches_per_layer"],
-            "roofline": {k: r["roofline"][k] for k in ("kernel", "kernel_name", "achieved", "frac", "launch_ms", "launch_ms_timed", "launch_algorithmic_MB",
-                                                       "traffic", "traffic_source")}}
+            "roofline": {k: r["roofline"][k] for k in ("kernel", "kernel_name", "achieved", "frac", "frac_timed_region", "frac_eager_kernel_events",
+                                                       "launch_ms", "launch_ms_timed", "launch_algorithmic_MB", "traffic", "traffic_source")}}
+
+
+# The BASELINE configs beside the headline: (key, workload, cache width or None for the workload's own, steps, warm-up,
+# paged, launchers).  Few steps each -- config 5 runs its whole rollout of 512 decode steps, which is what it is --, no
+# CPU leg, no read probe; the scan's launches are timed with events in at most 8 further eager steps.
+PER_CONFIG_LEGS = (
+    ("config1_fp16", "config1", None, 50, 5, False, "engine"),
+    ("config2_tq4", "config2", None, 30, 5, False, "engine"),
+    ("config3_tq4_contiguous", "config3", None, 10, 3, False, "engine"),
+    ("config3_tq4_paged", "config3", None, 10, 3, True, "engine"),
+    ("config3_tq2_paged", "config3", 2, 10, 3, True, "engine"),
+    ("config4_tq2", "config4", None, 20, 3, False, "engine"),
+    ("config5_rollout_tq4", "config5", 4, 512, 3, False, "engine"),
+    ("config5_rollout_fp16", "config5", 0, 512, 3, False, "engine"),
+    ("target_tq4_reference_launchers", "target", 4, 10, 3, False, "reference"),
+)
+
+
+def per_config(args):
+    """Every leg of PER_CONFIG_LEGS as {ms_per_step, tokens_per_s, step_frac_of_hbm_peak, kernel_name, launch_ms, ...}."""
+    import copy
+    out = {}
+    for key, workload, bits, steps, warmup, paged, launchers in PER_CONFIG_LEGS:
+        a = copy.copy(args)
+        a.workload, a.kv_bits, a.steps, a.warmup, a.paged, a.launchers = workload, bits, steps, warmup, paged, launchers
+        a.ctx = a.batch = a.layers = a.max_seq_len = None
+        a.profile_steps = 8
+        kv_bits = WORKLOADS[workload]["kv_bits"] if bits is None else bits
+        r = paged_bench(a) if paged else decode_bench(a, kv_bits, with_probe=False)
+        out[key] = {"workload": r["config"]["workload"], "kv_bits": kv_bits if kv_bits else 16, "steps": r["steps"],
+                    "ms_per_step": r["ms_per_step"], "tokens_per_s": r["value"],
+                    "step_algorithmic_GB": r["step_algorithmic_GB"], "step_frac_of_hbm_peak": r["step_frac_of_hbm_peak"],
+                    "launches_per_layer": r["config"]["launches_per_layer"],
+                    "kernel_name": r["roofline"]["kernel_name"], "launch_ms": r["roofline"]["launch_ms"],
+                    "launch_algorithmic_MB": r["roofline"]["launch_algorithmic_MB"], "launch_frac_of_hbm_peak": r["roofline"]["frac"]}
+    return out
 
 
 def workload_of(args):
@@ -488,7 +535,8 @@ def decode_bench(args, kv_bits, with_probe):
     L, H, Hk, G, D = w["L"], w["H"], w["Hk"], w["G"], 128
     K, W = args.steps, args.warmup
     kv_dim, q_dim = Hk * D, H * D
-    total_steps = W + K + K + 2          # warm-up, graph-timed, kernel-timed (eager), slack
+    Kp = max(1, min(K, 4096 // L, args.profile_steps or K))   # eager steps whose scan launches are timed one by one
+    total_steps = W + K + Kp + 2         # warm-up, graph-timed, kernel-timed (eager), slack
     msl = (w["ctx"] + total_steps + 255) // 256 * 256   # the engine's max_seq_len: context + room for the steps, rounded up
     if args.max_seq_len is not None:
         if args.max_seq_len < w["ctx"] + total_steps:
@@ -636,7 +684,6 @@ def decode_bench(args, kv_bits, with_probe):
     # ---- dominant kernel alone: a pair of HIP events attached to every launch of the context-scanning
     # kernel on its stream (hipExtLaunchKernelGGL: start = the kernel begins, stop = it ends), in eager
     # steps that continue the same decode; the library holds 4096 event pairs
-    Kp = max(1, min(K, 4096 // L))
     fused_before = lib.tw_kv_decode_fused_launches()
     lib.tw_kv_debug_profile_attention(1)
     with torch.cuda.stream(stream):
@@ -654,6 +701,7 @@ def decode_bench(args, kv_bits, with_probe):
     # three-kernel path
     one_launch = lib.tw_kv_decode_fused_launches() - fused_before == Kp * L
     launch_bytes = algorithmic_bytes(n_tokens_prof, G * Kp, L, H, Hk, kv_bits, with_append=one_launch) / (Kp * L)
+    frac_eager = launch_bytes / (eager_kern_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS     # per-launch events, eager steps
     if one_launch and use_graph:
         # The layer step is this one kernel, so the timed region itself is K * L launches of it (plus K one-block
         # position increments): its average duration there, the launches `value` is made of, is the events' time
@@ -738,6 +786,11 @@ def decode_bench(args, kv_bits, with_probe):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
+            # the two readings of the same kernel, side by side: `frac` above is frac_timed_region where the layer is one
+            # launch and the step is graph-replayed (the launches `value` is made of, back to back), else
+            # frac_eager_kernel_events (a pair of events on each launch of eager steps)
+            "frac_timed_region": (achieved / HBM_PEAK_GBS) if (one_launch and use_graph) else None,
+            "frac_eager_kernel_events": frac_eager,
             "launch_ms": kern_ms,
             "launch_ms_timed": timed,
             "launch_ms_eager_events": eager_kern_ms,

@@ -382,7 +382,9 @@ void tw_paged_turbo_append_attention_batch(tw_half* out, const tw_half* q, const
  * Limit: G * num_heads <= TW_NOALLOC_MAX_HEAD_VECTORS, else nothing is launched and an error is returned.
  * All calls on one GPU share that GPU's array, which keeps the last call's contents (nothing in it needs to
  * start at zero: a call reads only what it wrote itself): calls that overlap on one GPU race -- run them on one
- * stream, or order them.  Returns 0, or non-zero with the message in tw_kv_last_error_string(). */
+ * stream, or order them.  Returns 0, or non-zero with the message in tw_kv_last_error_string().  The return value
+ * is this call's own outcome: an error an earlier call left uncleared on the thread does not make it fail (it is
+ * still there afterwards when this call succeeds, and is replaced by this call's message when it fails). */
 #define TW_NOALLOC_SCRATCH_BYTES (32u << 20)
 #define TW_NOALLOC_MAX_HEAD_VECTORS 16384
 int tw_turbo_gqa_attention_batch_noalloc(tw_half* out, const tw_half* q, const uint8_t* ck_q, const uint8_t* cv_q,
@@ -476,6 +478,17 @@ int tw_engine_prompt_layer(tw_engine* e, int layer, int seq, const tw_half* q, c
  * tw_engine_set_positions). */
 int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, const tw_half* v,
                           tw_half* out, int use_graph, hipStream_t s);
+/* When the capture or the instantiation of the step's graph fails, the step is run without a graph, one line goes
+ * to stderr, and so are all later steps with the same buffers (engine.cpp:2396-2410); the next change of buffers,
+ * batch, arena or producers tries again.  graph_state tells what the latest decode step did: 0 run eagerly as asked,
+ * 1 graph replayed, 2 run eagerly after a failed capture.  debug_fail_captures (test hook): the next n captures
+ * are treated as failed after they have been recorded. */
+int tw_engine_graph_state(const tw_engine* e);
+void tw_engine_debug_fail_captures(tw_engine* e, int n);
+/* roctx ranges (tw_engine_decode_step, tw_engine_prompt_layer, tw_engine_single_step) for a profiler's timeline,
+ * where the reference prints std::chrono timings (engine.cpp:2305-2311, 2537-2544).  on != 0 looks the roctx
+ * library up (dlopen; nothing is linked) and switches the ranges on: 0, or -1 when there is none.  Process-wide. */
+int tw_kv_set_trace_ranges(int on);
 
 /* Prefix sharing, engine.cpp:2173-2214: copy rows [0,T) of sequence `src` to
  * every sequence in [dst_begin, dst_end). */
@@ -483,13 +496,35 @@ int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end
                                hipStream_t s);
 
 /* sleep() / wake(), engine.cpp:922-1022: sleep hands the cache memory back (frees an arena the engine
- * allocated, forgets one the caller owns), drops the captured step and the generation bookkeeping;
- * wake is intentionally empty: the reference's wake re-allocates the single-sequence caches it freed in sleep
- * (engine.cpp:985-1022), state this engine object does not own, and the batch state is re-created, zeroed, by the
- * next tw_engine_alloc_batch (or tw_engine_set_arena + tw_engine_alloc_batch), as in the reference. */
+ * allocated, forgets one the caller owns, frees the single-sequence caches), drops the captured step and the
+ * generation bookkeeping; wake re-allocates the single-sequence caches when the engine had them before the sleep
+ * (zeroed, current_pos = 0); the batch state is re-created, zeroed, by the next tw_engine_alloc_batch (or
+ * tw_engine_set_arena + tw_engine_alloc_batch), as in the reference. */
 int tw_engine_sleep(tw_engine* e);
 int tw_engine_wake(tw_engine* e);
 int tw_engine_is_allocated(const tw_engine* e);
+
+/* The single-sequence state of the reference's generate() / decode_token() path (model.h:195-204): per layer a key
+ * and a value array of max_seq_len rows (compressed: codes and norms), each an allocation of its own as in
+ * allocate_buffers (engine.cpp:322-331, 394-404), the attention scratch (num_heads * max_seq_len floats), the
+ * rotation and current_pos.  alloc_single allocates and zeroes them for the shape and max_seq_len the engine has
+ * (0 on success; a later tw_engine_set_shape frees them); tw_engine_reset zeroes them and sets current_pos to 0
+ * (engine.cpp:893-916).  single_cache_ptr: which as in tw_engine_cache_ptr, rows (max_seq_len, ...). */
+int tw_engine_alloc_single(tw_engine* e);
+int tw_engine_single_is_allocated(const tw_engine* e);
+void* tw_engine_single_cache_ptr(tw_engine* e, int layer, int which);
+const tw_half* tw_engine_single_rotation(tw_engine* e);   /* device, NULL when kv_bits==0 */
+int tw_engine_single_pos(const tw_engine* e);             /* state_.current_pos */
+int tw_engine_single_set_pos(tw_engine* e, int pos);      /* 0 <= pos < max_seq_len; waits for the steps in flight */
+/* forward_layer steps 4-5 for `layer` (engine.cpp:1069-1108): K and V of the token into row current_pos, attention
+ * over rows 0 .. current_pos.  q/out: num_heads*head_dim halves, k/v: kv_dim halves, device.  Nothing is allocated
+ * per call (the reference allocates and frees a device word per layer and token for the compressed append,
+ * engine.cpp:1078-1092).  -8: current_pos has reached max_seq_len.  Stream 0 means the engine's own stream (the
+ * reference runs this path on the legacy default stream). */
+int tw_engine_single_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, const tw_half* v, tw_half* out,
+                          hipStream_t s);
+/* current_pos += 1 after the last layer of a token (decode_token), host and device, in stream order. */
+int tw_engine_single_advance(tw_engine* e, hipStream_t s);
 
 /* The tail of generate_batch's decode loop (engine.cpp:2350, 2496-2534), for the caller that owns the
  * sampling: begin_generation sizes a (max_new_tokens, G) token history on the device; record_tokens

@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 
 import gen
+import parity_log
 
 pytestmark = pytest.mark.gpu
 
@@ -41,7 +42,9 @@ def host(t):
 def rel_err(got, want):
     got = got.astype(np.float64).reshape(-1, D)
     want = want.astype(np.float64).reshape(-1, D)
-    return float(np.max(np.max(np.abs(got - want), axis=1) / np.max(np.abs(want), axis=1)))
+    err = float(np.max(np.max(np.abs(got - want), axis=1) / np.max(np.abs(want), axis=1)))
+    parity_log.record(err)
+    return err
 
 
 def assert_bytes_equal(got, want, what, margin=None):

@@ -104,15 +104,18 @@ def test_rollout_loop_against_the_oracle(oracle, kv_bits):
 
 @pytest.mark.parametrize("kv_bits", [0, 4])
 def test_rollout_loop_full_size_by_properties(kv_bits):
-    """16 prompts x 8 = 128 sequences, 28 layers, a 256-token prefix per group, 64 graph-replayed steps.  Without
-    the oracle: positions = 256 + steps; the prefix rows of every group member equal its source's bytes, before
-    and after the steps (decode never touches them); outputs finite; two members of a group that are fed the same
-    q, k and v rows produce the same output bits and the same appended cache bytes, members fed different rows do
-    not; the step after a reset of the positions reproduces the first step's output bit for bit."""
+    """BASELINE config 5 as it is: 16 prompts x 8 = 128 sequences, 28 layers, a 256-token prefix per group, all 512
+    graph-replayed decode steps (contexts 257 .. 768, max_seq_len 776).  Without the oracle: positions = 768 at the
+    end; the prefix rows of every group member equal its source's bytes, before and after the steps (decode never
+    touches them); outputs finite; two members of a group that are fed the same q, k and v rows produce the same
+    output bits and the same appended cache bytes, members fed different rows do not; the step after a reset of the
+    positions reproduces the first step's output bit for bit.  (The choice of kernels does not change inside this
+    rollout: tw_kv_decode_step_plan answers "one launch" for 128 sequences up to contexts of several thousand tokens;
+    test_gpu_engine_single.py crosses a change of plan at BASELINE config 4's size.)"""
     import torch
-    from triebwerk_amd import Engine
-    L, H, Hk, groups, members, T, steps = 28, 16, 8, 16, 8, 256, 64
-    G, msl = groups * members, 384
+    from triebwerk_amd import Engine, _lib
+    L, H, Hk, groups, members, T, steps = 28, 16, 8, 16, 8, 256, 512
+    G, msl = groups * members, 776
     kv_dim, q_dim = Hk * D, H * D
     eng = Engine(max_seq_len=msl, kv_bits=kv_bits)
     eng.set_shape(L, H, Hk, D)
@@ -152,14 +155,22 @@ def test_rollout_loop_full_size_by_properties(kv_bits):
     out = torch.zeros((L, G, q_dim), dtype=torch.float16, device="cuda")
     stream = torch.cuda.Stream()
     first = None
+    lib = _lib.load()
+    plans = set()
     with torch.cuda.stream(stream):
         for step in range(steps):
+            if kv_bits:
+                plans.add(lib.tw_kv_decode_step_plan(G, H, Hk, kv_bits, msl, T + step + 1, T + step + 1))
             eng.decode_step(q, k, v, out, use_graph=True, stream=stream)
+            assert eng.graph_state() == 1
             if step == 0:
                 stream.synchronize()
                 first = out.clone()
+            if step % 64 == 63:
+                print(f"rollout kv_bits={kv_bits}: step {step + 1} of {steps}", flush=True)
     stream.synchronize()
-    assert host(eng.positions()).tolist() == [T + steps] * G
+    assert T + steps == 768 and host(eng.positions()).tolist() == [768] * G
+    assert plans <= {1}, "the plan changed inside the rollout: say so in the docstring"
     assert torch.isfinite(out.float()).all()
     ov = out.view(L, groups, members, -1)
     assert torch.equal(ov[:, :, 0], ov[:, :, 1]), "same prefix, same inputs: different output bits"

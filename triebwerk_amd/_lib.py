@@ -111,6 +111,17 @@ SIGNATURES = {
     "tw_engine_prompt_layer": (I, [P, I, I, P, P, P, P, P, I, P]),
     "tw_engine_decode_step": (I, [P, P, P, P, P, I, P]),
     "tw_engine_broadcast_prefix": (I, [P, I, I, I, I, P]),
+    "tw_engine_graph_state": (I, [P]),
+    "tw_engine_debug_fail_captures": (None, [P, I]),
+    "tw_kv_set_trace_ranges": (I, [I]),
+    "tw_engine_alloc_single": (I, [P]),
+    "tw_engine_single_is_allocated": (I, [P]),
+    "tw_engine_single_cache_ptr": (P, [P, I, I]),
+    "tw_engine_single_rotation": (P, [P]),
+    "tw_engine_single_pos": (I, [P]),
+    "tw_engine_single_set_pos": (I, [P, I]),
+    "tw_engine_single_step": (I, [P, I, P, P, P, P, P]),
+    "tw_engine_single_advance": (I, [P, P]),
 }
 
 _lib = None

@@ -1027,6 +1027,14 @@ int tw_turbo_gqa_attention_batch_noalloc(tw_half* out, const tw_half* q, const u
                                          const int* pos, int msl, int G, int num_heads, int num_kv_heads, int head_dim,
                                          int q_dim, int kv_dim, int bits, hipStream_t s) {
     const char* fn = "tw_turbo_gqa_attention_batch_noalloc";
+    // The return value is this call's own outcome, whatever an earlier call left in the thread's sticky error: that
+    // one is set aside while the call runs and put back when the call succeeds; when the call fails, its own message
+    // is the one tw_kv_last_error_string() returns afterwards.
+    struct StickyAside {
+        int code; char msg[sizeof(g_err_msg)];
+        StickyAside() : code(g_err) { memcpy(msg, g_err_msg, sizeof(msg)); g_err = 0; g_err_msg[0] = 0; }
+        ~StickyAside() { if (g_err == 0 && code != 0) { g_err = code; memcpy(g_err_msg, msg, sizeof(msg)); } }
+    } aside;
     if (!check_shape(fn, num_heads, num_kv_heads, head_dim) || !check_bits(fn, bits)) return 1;
     if (kv_dim != num_kv_heads * head_dim) {
         set_error(1, "%s: kv_dim=%d != num_kv_heads*head_dim", fn, kv_dim);
@@ -1047,9 +1055,8 @@ int tw_turbo_gqa_attention_batch_noalloc(tw_half* out, const tw_half* q, const u
     // then both make the same plan and the same bits
     const long long room = (long long)(TW_NOALLOC_SCRATCH_BYTES / sizeof(float)) / ((long long)G * num_heads);
     plan_splits(a, msl, room < msl ? room : msl);
-    const int before = g_err;
     run_attention(a, s, fn, /*query_done=*/false, /*may_profile=*/false);
-    return (before == 0 && g_err != 0) ? 3 : 0;
+    return g_err != 0 ? 3 : 0;
 }
 
 void tw_paged_gqa_attention_batch(tw_half* out, const tw_half* q, const tw_half* ck,

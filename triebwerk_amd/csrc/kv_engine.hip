@@ -9,11 +9,14 @@
 //   append -> attention per layer ...... engine.cpp:1979-2006
 //   decode-step graph .................. engine.cpp:2369-2412, 2472-2480
 //   prefix broadcast ................... engine.cpp:2173-2214
+//   single-sequence caches ............. engine.cpp:322-331, 394-404 (allocation), 893-916 (reset),
+//                                        922-1022 (sleep / wake), 1069-1108 (append -> attention of a layer)
 //
 // Everything else the reference engine owns (weights, GEMMs, sampling) is not
 // part of this library.
 
 #include <hip/hip_runtime.h>
+#include <dlfcn.h>
 
 #include <cstdio>
 #include <cstring>
@@ -46,6 +49,19 @@ struct tw_engine {
 
     hipStream_t stream = nullptr;     // engine_stream_, engine.cpp:309
 
+    // single-sequence state (InferenceState / KVCache, model.h:195-204): per-layer caches of max_seq_len rows, each
+    // an allocation of its own as in allocate_buffers (engine.cpp:322-331, 394-404), the attention scratch of
+    // num_heads * max_seq_len floats, the rotation, and current_pos -- on the host and, for the launchers that take
+    // positions from device memory, in one device word that lives as long as the caches (the reference allocates and
+    // frees such a word per layer and token, engine.cpp:1078-1092)
+    void* single[kMaxLayers][4] = {};
+    float* single_scores = nullptr;
+    tw_half* single_rotation = nullptr;
+    int* single_d_pos = nullptr;
+    int single_pos = 0;
+    bool single_allocated = false;
+    bool single_wanted = false;       // wake() re-allocates what sleep() freed (engine.cpp:985-1022)
+
     // producers of q and k run with the step (forward_layer_batch step 3, engine.cpp:1972-1977);
     // caller-owned device memory: weights (num_layers, head_dim), tables (positions, rope_dim / 2)
     int producers = 0;                // 0 none, 1 fused into the append, 2 as launches of their own
@@ -63,6 +79,12 @@ struct tw_engine {
     const void* graph_key[4] = {};
     int graph_G = 0;
     int graph_plan = 0;               // tw_kv_decode_step_plan's answer the captured launches were chosen under
+    // generate_batch goes on without a graph when capture or instantiation fails (engine.cpp:2396-2410): so does
+    // tw_engine_decode_step, until the buffers, the batch or the producers change
+    bool graph_failed = false;
+    const void* graph_failed_key[4] = {};
+    int graph_state = 0;              // of the latest decode step: 0 eager as asked, 1 graph replayed, 2 eager after a failed capture
+    int fail_next_captures = 0;       // test hook: treat this many coming captures as failed
 
     // The stream of the latest step: reset, set_positions and everything that lets go of the arena wait for it
     // first (a caller's stream has no implicit order with the engine's own stream or with the null stream).
@@ -106,7 +128,11 @@ struct tw_engine {
         graph_G = 0;
     }
     void drop_arena() {
-        wait_for_steps();
+        // the arena may be freed below: wait for everything on the device, not only for the stream of the latest step
+        // (steps issued earlier on other streams may still be reading it)
+        if (arena) (void)hipDeviceSynchronize();
+        steps_in_flight = false;
+        graph_failed = false;
         drop_graph();  // the capture holds arena addresses, engine.cpp:1440-1442
         drop_generation();
         if (arena && arena_owned) hipFree(arena);
@@ -170,6 +196,47 @@ int carve(tw_engine* e, int G, int msl) {
 }
 
 hipStream_t pick(tw_engine* e, hipStream_t s) { return s ? s : e->stream; }
+
+// ---- trace ranges (the reference prints std::chrono timings around these phases, engine.cpp:2305-2311, 2537-2544;
+// here they are roctx ranges a profiler can show).  Off until tw_kv_set_trace_ranges(1) finds the roctx library.
+typedef int (*roctx_push_fn)(const char*);
+typedef int (*roctx_pop_fn)();
+roctx_push_fn g_range_push = nullptr;
+roctx_pop_fn g_range_pop = nullptr;
+bool g_ranges_on = false;
+struct TraceRange {
+    bool on;
+    explicit TraceRange(const char* name) : on(g_ranges_on && g_range_push && g_range_pop) { if (on) g_range_push(name); }
+    ~TraceRange() { if (on) g_range_pop(); }
+};
+
+// per-array row bytes of a cache: keys, values, key norms, value norms (0: the array does not exist)
+size_t cache_row_bytes(const tw_engine* e, int which) {
+    if (e->kv_bits == 0) return which < 2 ? (size_t)e->kv_dim() * 2 : 0;
+    return which < 2 ? e->kv_dim_packed() : (size_t)e->shape.num_kv_heads * 2;
+}
+
+void free_single(tw_engine* e) {
+    if (!e->single_allocated) return;
+    (void)hipDeviceSynchronize();
+    for (int i = 0; i < kMaxLayers; i++)
+        for (int w = 0; w < 4; w++)
+            if (e->single[i][w]) { hipFree(e->single[i][w]); e->single[i][w] = nullptr; }
+    if (e->single_scores) { hipFree(e->single_scores); e->single_scores = nullptr; }
+    if (e->single_rotation) { hipFree(e->single_rotation); e->single_rotation = nullptr; }
+    if (e->single_d_pos) { hipFree(e->single_d_pos); e->single_d_pos = nullptr; }
+    e->single_allocated = false;
+}
+
+int zero_single(tw_engine* e) {
+    const size_t rows = (size_t)e->max_seq_len;
+    for (int i = 0; i < e->shape.num_layers; i++)
+        for (int w = 0; w < 4; w++)
+            if (e->single[i][w] && hipMemset(e->single[i][w], 0, rows * cache_row_bytes(e, w)) != hipSuccess) return -1;
+    if (hipMemset(e->single_d_pos, 0, sizeof(int)) != hipSuccess) return -1;
+    e->single_pos = 0;
+    return 0;
+}
 
 // A step appends at positions[g]: once the furthest sequence the host knows of has used its last row there is no
 // row left, and the append would land in the next sequence's rows (or past the array).
@@ -245,6 +312,7 @@ tw_engine* tw_engine_create(int max_seq_len, int kv_bits) {
 void tw_engine_destroy(tw_engine* e) {
     if (!e) return;
     e->drop_arena();
+    free_single(e);
     if (e->stream) hipStreamDestroy(e->stream);
     delete e;
 }
@@ -257,6 +325,7 @@ int tw_engine_set_shape(tw_engine* e, const tw_model_shape* shape) {
         shape->num_kv_heads < 1 || shape->num_heads % shape->num_kv_heads != 0)
         return -1;
     e->drop_arena();
+    free_single(e);                   // sized by the shape; tw_engine_alloc_single makes them anew
     e->shape = *shape;
     return 0;
 }
@@ -282,7 +351,10 @@ int tw_engine_alloc_batch(tw_engine* e, int G, int max_seq_len) {
         e->arena_cap = need;
         e->arena_owned = true;
     } else {
-        e->wait_for_steps();
+        // the rows are about to be re-carved and zeroed: as in drop_arena, wait for the whole device
+        (void)hipDeviceSynchronize();
+        e->steps_in_flight = false;
+        e->graph_failed = false;
         e->drop_graph();
         e->drop_generation();
     }
@@ -301,21 +373,17 @@ int tw_engine_set_arena(tw_engine* e, void* device_ptr, size_t bytes) {
 }
 
 int tw_engine_reset(tw_engine* e) {
+    if (e->single_allocated) {                 // reset(), engine.cpp:893-916: the single-sequence caches, current_pos = 0
+        e->wait_for_steps();
+        if (zero_single(e) != 0) return -1;
+    }
     if (!e->arena || e->G == 0) return 0;
     e->wait_for_steps();
     hipStream_t s = e->stream;
     const size_t rows = (size_t)e->G * e->batch_msl;
-    for (int i = 0; i < e->shape.num_layers; i++) {
-        if (e->kv_bits == 0) {
-            hipMemsetAsync(e->cache[i][0], 0, rows * e->kv_dim() * 2, s);
-            hipMemsetAsync(e->cache[i][1], 0, rows * e->kv_dim() * 2, s);
-        } else {
-            hipMemsetAsync(e->cache[i][0], 0, rows * e->kv_dim_packed(), s);
-            hipMemsetAsync(e->cache[i][1], 0, rows * e->kv_dim_packed(), s);
-            hipMemsetAsync(e->cache[i][2], 0, rows * e->shape.num_kv_heads * 2, s);
-            hipMemsetAsync(e->cache[i][3], 0, rows * e->shape.num_kv_heads * 2, s);
-        }
-    }
+    for (int i = 0; i < e->shape.num_layers; i++)
+        for (int w = 0; w < 4; w++)
+            if (e->cache[i][w]) hipMemsetAsync(e->cache[i][w], 0, rows * cache_row_bytes(e, w), s);
     hipMemsetAsync(e->d_positions, 0, (size_t)e->G * sizeof(int), s);
     e->pos_known = true;
     e->pos_min = e->pos_max = 0;
@@ -353,24 +421,116 @@ int tw_engine_set_producers(tw_engine* e, int mode, const tw_half* q_norm, const
     if ((q_norm == nullptr) != (k_norm == nullptr) || (rope_cos == nullptr) != (rope_sin == nullptr)) return -1;
     if (rope_cos && !(rope_dim == 128 || (rope_dim >= 16 && rope_dim <= 64 && rope_dim % 16 == 0))) return -1;
     e->drop_graph();                  // a captured step holds the old sequence of launches
+    e->graph_failed = false;
     e->producers = (q_norm || rope_cos) ? mode : 0;
     e->q_norm = q_norm; e->k_norm = k_norm; e->norm_eps = eps; e->norm_biased = biased ? 1 : 0;
     e->rope_cos = rope_cos; e->rope_sin = rope_sin; e->rope_dim = rope_dim;
     return 0;
 }
 
-// sleep(), engine.cpp:922-983: give the device memory back (the arena when the engine allocated it; a
-// caller's arena is only forgotten) and drop everything that points into it.  wake(), engine.cpp:985-1022,
-// has nothing to restore for the batch path: alloc_batch re-creates it on the next use.
+// sleep(), engine.cpp:922-983: give the device memory back -- the arena when the engine allocated it (a caller's
+// arena is only forgotten) and the single-sequence caches -- and drop everything that points into it.
+// wake(), engine.cpp:985-1022: re-allocate the single-sequence caches that sleep freed (zeroed, current_pos = 0:
+// the reference leaves them as cudaMalloc returns them and relies on the reset() in front of every generate);
+// the batch state comes back with the next alloc_batch, as in the reference.
 int tw_engine_sleep(tw_engine* e) {
     if (e->stream) hipStreamSynchronize(e->stream);
     e->drop_arena();
+    free_single(e);
     return 0;
 }
 
 int tw_engine_wake(tw_engine* e) {
-    (void)e;
+    if (e->single_wanted && !e->single_allocated) return tw_engine_alloc_single(e);
     return 0;
+}
+
+// allocate_buffers' share for this path, engine.cpp:322-331 (fp16) and 394-404 (compressed): per layer a key and a
+// value array of max_seq_len rows (and the two norm arrays), each an allocation of its own.
+int tw_engine_alloc_single(tw_engine* e) {
+    e->single_wanted = true;
+    if (e->single_allocated) return 0;
+    if (!e->stream && hipStreamCreate(&e->stream) != hipSuccess) return -3;
+    const size_t rows = (size_t)e->max_seq_len;
+    if (rows < 1) return -1;
+    bool ok = true;
+    e->single_allocated = true;               // from here on free_single lets go of whatever was obtained
+    for (int i = 0; i < e->shape.num_layers && ok; i++)
+        for (int w = 0; w < 4 && ok; w++) {
+            const size_t rb = cache_row_bytes(e, w);
+            if (rb) ok = hipMalloc(&e->single[i][w], rows * rb) == hipSuccess;
+        }
+    ok = ok && hipMalloc((void**)&e->single_scores, (size_t)e->shape.num_heads * rows * sizeof(float)) == hipSuccess;
+    ok = ok && hipMalloc((void**)&e->single_d_pos, sizeof(int)) == hipSuccess;
+    if (ok && e->kv_bits > 0) {
+        const size_t n = (size_t)e->shape.head_dim * e->shape.head_dim;
+        ok = hipMalloc((void**)&e->single_rotation, n * 2) == hipSuccess;
+        if (ok) {
+            std::vector<tw_half> rot(n);
+            tw_make_rotation_host(rot.data(), e->shape.head_dim, 42u);
+            ok = hipMemcpy(e->single_rotation, rot.data(), n * 2, hipMemcpyHostToDevice) == hipSuccess;
+        }
+    }
+    if (ok) ok = zero_single(e) == 0;
+    if (!ok) { (void)hipGetLastError(); free_single(e); return -2; }
+    return 0;
+}
+
+int tw_engine_single_is_allocated(const tw_engine* e) { return e->single_allocated ? 1 : 0; }
+int tw_engine_single_pos(const tw_engine* e) { return e->single_pos; }
+void* tw_engine_single_cache_ptr(tw_engine* e, int layer, int which) {
+    if (layer < 0 || layer >= e->shape.num_layers || which < 0 || which > 3) return nullptr;
+    return e->single[layer][which];
+}
+const tw_half* tw_engine_single_rotation(tw_engine* e) { return e->kv_bits > 0 ? e->single_rotation : nullptr; }
+
+int tw_engine_single_set_pos(tw_engine* e, int pos) {
+    if (!e->single_allocated) return -1;
+    if (pos < 0 || pos >= e->max_seq_len) return -2;
+    e->wait_for_steps();
+    if (hipMemcpy(e->single_d_pos, &pos, sizeof(int), hipMemcpyHostToDevice) != hipSuccess) return -3;
+    e->single_pos = pos;
+    return 0;
+}
+
+// forward_layer steps 4-5 (engine.cpp:1069-1108) at current_pos: K and V of the token into row current_pos of the
+// layer's cache, attention over rows 0 .. current_pos.  One call of the layer step of the batch path with a batch
+// of one, so the single sequence gets the same kernels (the append inside the attention launch for the fp16 cache,
+// the whole step in one launch for the compressed one); nothing is allocated per token.
+int tw_engine_single_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, const tw_half* v, tw_half* out,
+                          hipStream_t s) {
+    if (!e->single_allocated || layer < 0 || layer >= e->shape.num_layers) return -1;
+    if (e->single_pos >= e->max_seq_len) return -8;
+    TraceRange range("tw_engine_single_step");
+    s = pick(e, s);
+    e->note_step(s);
+    tw_kv_clear_error();
+    const tw_model_shape& m = e->shape;
+    tw_layer_step_args p;
+    memset(&p, 0, sizeof(p));
+    p.out = out; p.q = const_cast<tw_half*>(q); p.k = const_cast<tw_half*>(k); p.v = v;
+    p.G = 1; p.num_heads = m.num_heads; p.num_kv_heads = m.num_kv_heads; p.head_dim = m.head_dim;
+    p.q_dim = e->q_dim(); p.kv_dim = e->kv_dim();
+    p.positions = e->single_d_pos; p.max_seq_len = e->max_seq_len;
+    p.kv_bits = e->kv_bits;
+    p.cache_k = e->single[layer][0]; p.cache_v = e->single[layer][1];
+    p.k_norms = (tw_half*)e->single[layer][2]; p.v_norms = (tw_half*)e->single[layer][3];
+    p.rotation = e->single_rotation; p.scratch = e->single_scores;
+    p.ctx_min = p.ctx_max = e->single_pos + 1;
+    tw_layer_attention_step(&p, s);
+    return tw_kv_last_error();
+}
+
+// decode_token's `state_.current_pos++` after the last layer: host and device word, in stream order
+int tw_engine_single_advance(tw_engine* e, hipStream_t s) {
+    if (!e->single_allocated) return -1;
+    if (e->single_pos >= e->max_seq_len) return -8;
+    s = pick(e, s);
+    e->note_step(s);
+    tw_kv_clear_error();
+    launch_increment_positions(e->single_d_pos, 1, s);
+    e->single_pos++;
+    return tw_kv_last_error();
 }
 
 int tw_engine_is_allocated(const tw_engine* e) { return e->arena != nullptr && e->G > 0; }
@@ -470,6 +630,7 @@ int tw_engine_prompt_layer(tw_engine* e, int layer, int seq, const tw_half* q, c
         !token_positions)
         return -1;
     if (T == 0) return 0;
+    TraceRange range("tw_engine_prompt_layer");
     s = pick(e, s);
     e->note_step(s);
     tw_kv_clear_error();
@@ -517,15 +678,21 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
                           tw_half* out, int use_graph, hipStream_t s) {
     if (!e->arena) return -1;
     if (cache_full(e)) return -8;          // before any launch or replay: cache and positions stay as they are
+    TraceRange range("tw_engine_decode_step");
     s = pick(e, s);
     e->note_step(s);
     tw_kv_clear_error();
-    if (!use_graph) {
+    const void* key[4] = {q, k, v, out};
+    auto eager = [&](int state) -> int {
         all_layers(e, q, k, v, out, s);
         if (e->pos_known) { e->pos_min++; e->pos_max++; }
+        e->graph_state = state;
         return tw_kv_last_error();
-    }
-    const void* key[4] = {q, k, v, out};
+    };
+    if (!use_graph) return eager(0);
+    // a capture that failed for these buffers is not tried again step after step (engine.cpp:2396-2410 tries once
+    // per generate_batch and decodes eagerly when it fails)
+    if (e->graph_failed && memcmp(key, e->graph_failed_key, sizeof(key)) == 0) return eager(2);
     // The launches in a captured step were chosen from the context lengths at capture; when the lengths have
     // grown (or spread) to where the other kernels are the better choice, the step is captured again.
     const int plan = step_plan(e);
@@ -533,19 +700,27 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
         e->drop_graph();
         // Capture records the launches without running them, so unlike the
         // reference (engine.cpp:2414-2444) nothing has to be re-prefilled.
-        if (hipStreamBeginCapture(s, hipStreamCaptureModeRelaxed) != hipSuccess) return -4;
-        all_layers(e, q, k, v, out, s);
+        int why = 0;                       // -4 begin, -5 end of capture or a launcher's error, -6 instantiation
         hipGraph_t g = nullptr;
-        hipError_t err = hipStreamEndCapture(s, &g);
-        if (err != hipSuccess || !g || tw_kv_last_error() != 0) {
-            if (g) hipGraphDestroy(g);
-            (void)hipGetLastError();
-            return -5;
+        hipError_t err = hipStreamBeginCapture(s, hipStreamCaptureModeRelaxed);
+        if (err != hipSuccess) {
+            why = -4;
+        } else {
+            all_layers(e, q, k, v, out, s);
+            err = hipStreamEndCapture(s, &g);
+            if (err != hipSuccess || !g || tw_kv_last_error() != 0) why = -5;
+            else if (e->fail_next_captures > 0) { e->fail_next_captures--; why = -6; err = hipErrorUnknown; }
+            else if ((err = hipGraphInstantiate(&e->graph_exec, g, nullptr, nullptr, 0)) != hipSuccess) why = -6;
         }
-        if (hipGraphInstantiate(&e->graph_exec, g, nullptr, nullptr, 0) != hipSuccess) {
-            hipGraphDestroy(g);
+        if (why != 0) {
+            if (g) hipGraphDestroy(g);
             e->graph_exec = nullptr;
-            return -6;
+            (void)hipGetLastError();
+            fprintf(stderr, "  hipGraph capture FAILED (step %d, err=%d): decoding without a graph\n", why, (int)err);
+            tw_kv_clear_error();
+            e->graph_failed = true;
+            memcpy(e->graph_failed_key, key, sizeof(key));
+            return eager(2);               // the recorded launches never ran: run the step now
         }
         e->graph = g;
         e->graph_G = e->G;
@@ -554,7 +729,27 @@ int tw_engine_decode_step(tw_engine* e, const tw_half* q, const tw_half* k, cons
     }
     if (hipGraphLaunch(e->graph_exec, s) != hipSuccess) return -7;
     if (e->pos_known) { e->pos_min++; e->pos_max++; }
+    e->graph_state = 1;
     return 0;
+}
+
+int tw_engine_graph_state(const tw_engine* e) { return e->graph_state; }
+void tw_engine_debug_fail_captures(tw_engine* e, int n) { e->fail_next_captures = n > 0 ? n : 0; }
+
+int tw_kv_set_trace_ranges(int on) {
+    if (!on) { g_ranges_on = false; return 0; }
+    if (!g_range_push || !g_range_pop) {
+        for (const char* name : {"librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4", "libroctx64.so"}) {
+            void* h = dlopen(name, RTLD_NOW | RTLD_GLOBAL);
+            if (!h) continue;
+            g_range_push = reinterpret_cast<roctx_push_fn>(dlsym(h, "roctxRangePushA"));
+            g_range_pop = reinterpret_cast<roctx_pop_fn>(dlsym(h, "roctxRangePop"));
+            if (g_range_push && g_range_pop) break;
+            g_range_push = nullptr; g_range_pop = nullptr;
+        }
+    }
+    g_ranges_on = g_range_push && g_range_pop;
+    return g_ranges_on ? 0 : -1;
 }
 
 int tw_engine_broadcast_prefix(tw_engine* e, int src, int dst_begin, int dst_end, int T, hipStream_t s) {

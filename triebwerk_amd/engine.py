@@ -166,16 +166,93 @@ class Engine:
         if rc != 0:
             raise RuntimeError(f"broadcast_prefix failed ({rc})")
 
+    def graph_state(self) -> int:
+        """What the latest decode_step did: 0 eager as asked, 1 graph replayed, 2 eager after a failed capture
+        (generate_batch decodes without a graph when the capture fails, engine.cpp:2396-2410)."""
+        return self._lib.tw_engine_graph_state(self._h)
+
+    # ---- the single-sequence state of generate() / decode_token() (engine.cpp:322-331, 394-404, 1069-1108)
+    def alloc_single(self) -> None:
+        """Per-layer caches of max_seq_len rows for one sequence, each an allocation of its own as in the reference."""
+        rc = self._lib.tw_engine_alloc_single(self._h)
+        if rc != 0:
+            raise RuntimeError(f"alloc_single failed ({rc})")
+
+    def single_is_allocated(self) -> bool:
+        return bool(self._lib.tw_engine_single_is_allocated(self._h))
+
+    def single_pos(self) -> int:
+        return self._lib.tw_engine_single_pos(self._h)
+
+    def single_set_pos(self, pos: int) -> None:
+        rc = self._lib.tw_engine_single_set_pos(self._h, int(pos))
+        if rc != 0:
+            raise ValueError(f"single_set_pos failed ({rc})")
+
+    @staticmethod
+    def _wrap(ptr: int, nbytes: int, dtype, shape):
+        """A torch view of device memory the engine owns (valid until the engine frees it)."""
+        class _Mem:
+            __cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (int(ptr), False), "version": 2}
+        return torch.as_tensor(_Mem(), device="cuda").view(dtype).view(shape)
+
+    def single_cache(self, layer: int):
+        """Torch views of one layer's single-sequence cache: (keys, values, key_norms, value_norms), rows
+        (max_seq_len, ...); valid until sleep, set_shape or the engine's end."""
+        L, H, Hk, D = self._shape
+        msl, bits = self.max_seq_len(), self.kv_bits()
+        ptrs = [self._lib.tw_engine_single_cache_ptr(self._h, layer, w) for w in range(4)]
+        if not ptrs[0]:
+            raise RuntimeError("single-sequence caches are not allocated")
+        if bits == 0:
+            n = msl * Hk * D * 2
+            return (self._wrap(ptrs[0], n, torch.float16, (msl, Hk * D)),
+                    self._wrap(ptrs[1], n, torch.float16, (msl, Hk * D)), None, None)
+        kvp = Hk * D * bits // 8
+        return (self._wrap(ptrs[0], msl * kvp, torch.uint8, (msl, kvp)), self._wrap(ptrs[1], msl * kvp, torch.uint8, (msl, kvp)),
+                self._wrap(ptrs[2], msl * Hk * 2, torch.float16, (msl, Hk)), self._wrap(ptrs[3], msl * Hk * 2, torch.float16, (msl, Hk)))
+
+    def single_rotation(self):
+        p = self._lib.tw_engine_single_rotation(self._h)
+        if not p:
+            return None
+        D = self._shape[3]
+        return self._wrap(p, D * D * 2, torch.float16, (D, D))
+
+    def single_step(self, layer, q, k, v, out, stream=None) -> None:
+        """forward_layer's append + attention for `layer` at current_pos (engine.cpp:1069-1108).
+        q/out: (H*D,), k/v: (Hk*D,)."""
+        L, H, Hk, D = self._shape
+        for name, t, n in (("q", q, H * D), ("out", out, H * D), ("k", k, Hk * D), ("v", v, Hk * D)):
+            if t.numel() != n:
+                raise ValueError(f"{name}: {t.numel()} elements, expected {n}")
+        rc = self._lib.tw_engine_single_step(self._h, layer, _ptr(q, "f16", "q"), _ptr(k, "f16", "k"), _ptr(v, "f16", "v"),
+                                             _ptr(out, "f16", "out"), _stream(stream))
+        if rc != 0:
+            _lib.check(self._lib)
+            raise RuntimeError(f"single_step failed ({rc})")
+
+    def single_advance(self, stream=None) -> None:
+        """current_pos += 1 (decode_token, after the last layer)."""
+        rc = self._lib.tw_engine_single_advance(self._h, _stream(stream))
+        if rc != 0:
+            _lib.check(self._lib)
+            raise RuntimeError(f"single_advance failed ({rc})")
+
     # ---- memory lifecycle (engine.cpp:922-1022)
     def sleep(self) -> None:
-        """Give the cache memory back (the torch arena is released) and drop the captured step."""
+        """Give the cache memory back (the torch arena is released, the single-sequence caches are freed) and drop
+        the captured step."""
         self._lib.tw_engine_sleep(self._h)
         self._arena = None
         self._G = self._msl = 0
 
     def wake(self) -> None:
-        """Nothing to restore for the batch path: call alloc_batch again."""
-        self._lib.tw_engine_wake(self._h)
+        """Re-allocate the single-sequence caches if the engine had them before sleep (engine.cpp:985-1022); the
+        batch comes back with the next alloc_batch."""
+        rc = self._lib.tw_engine_wake(self._h)
+        if rc != 0:
+            raise RuntimeError(f"wake failed ({rc})")
 
     def is_allocated(self) -> bool:
         return bool(self._lib.tw_engine_is_allocated(self._h))
