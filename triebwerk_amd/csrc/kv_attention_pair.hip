@@ -18,16 +18,14 @@ namespace {
 constexpr int kPairScanWaves = 8;      // waves per workgroup: 256 registers each, one workgroup per CU (64 KB table)
 }  // namespace
 
-// TILES: 32-token tiles per step of the loop -- 2 for the contiguous 2-bit cache (pair_scan_tile_x2), else 1.
-template <bool PAGED, int R, int BITS, int TILES = 1>
+template <bool PAGED, int R, int BITS>
 __global__ void __launch_bounds__(kPairScanWaves * kWave)
 attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves) {
-    static_assert(TILES == 1 || (TILES == 2 && BITS == 2 && !PAGED), "two tiles per step: contiguous 2-bit cache only");
     constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
     constexpr uint32_t kHeadBytes4 = BITS * 16;                      // bytes of one head in a cache row
     constexpr int kCodesAux = BITS == 4 ? kStreamCodes : 0;          // whole lines per instruction only at 4 bit
     __shared__ __attribute__((aligned(16))) uint32_t tab_s[kTableWords];
-    __shared__ __attribute__((aligned(16))) half_t p_s[kPairScanWaves][TILES * 16][32];
+    __shared__ __attribute__((aligned(16))) half_t p_s[kPairScanWaves][16][32];
     // balanced walk: tiles of the sequences before g, and {tiles per group, total tiles}
     __shared__ int pre_s[kMaxBalanceSeqs + 1];
     __shared__ int bal_s[2];
@@ -175,20 +173,12 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     // One tile of loads is in flight per wave; each register set is re-issued for the next tile as soon as its
     // contents have been expanded.  (A second set of registers with the tile after next in flight, the loop unrolled
     // over the two sets: 3 % slower at 2 bit, where the waves spend 45 % of their time waiting for loads and the set
-    // costs 20 registers, on even and on ragged batches -- as at 4 bit, more requests in flight do not arrive sooner.)
+    // costs 20 registers, on even and on ragged batches -- as at 4 bit, more requests in flight do not arrive sooner.
+    // Two 2-bit tiles as ONE step of the loop -- both tiles' loads in flight, one pass of the online softmax over the
+    // lane's four tokens, one decision about the maximum and one hand-over of the probabilities per 64 tokens, 203-237
+    // registers: 71.6-72.1 against 67.3-67.8 us at 64 x 8192 tokens, 51.3 against 47.3 us on the ragged batch.)
     PairTileRegs<BITS> t;
-    PairTileRegs<BITS> t2[TILES == 2 ? 2 : 1];                 // TILES == 2: the two tiles of a step
-    auto chunk_rows = [&](int tile) -> int { return max(min(t1 - tile, 32), 0); };   // rows of a tile inside the chunk
     auto issue_first = [&]() {
-        if constexpr (TILES == 2) {
-#pragma unroll
-            for (int u = 0; u < 2; u++) issue_k(t2[u], t0 + 32 * u, chunk_rows(t0 + 32 * u));
-#pragma unroll
-            for (int u = 0; u < 2; u++) issue_n(t2[u], t0 + 32 * u, chunk_rows(t0 + 32 * u));
-#pragma unroll
-            for (int u = 0; u < 2; u++) issue_v(t2[u], t0 + 32 * u, chunk_rows(t0 + 32 * u));
-            return;
-        }
         int pg0 = PAGED ? 0 : tile_rows(t0);
         if (PAGED) {
             pg0 = fetch_pages(t0);
@@ -244,7 +234,7 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
     }
     // ---- dequantization table, once per workgroup
     build_centroid_table<BITS, true>(tab_s, kAlpha, tid, nthreads);
-    for (int i = tid; i < kPairScanWaves * TILES * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
+    for (int i = tid; i < kPairScanWaves * 16 * 32 / 2; i += nthreads) reinterpret_cast<uint32_t*>(p_s)[i] = 0u;
     __syncthreads();             // the only workgroup-wide barrier; every wave reaches it
 
     if (balanced) {
@@ -280,18 +270,6 @@ attention_pair_kernel(AttnArgs a, int total_items, int hgroups, int group_waves)
             return a.qrot + ((long long)g * a.num_heads + (long long)h * R + i) * a.ws_stride;
         });
 
-        if constexpr (TILES == 2) {
-            // a chunk ends on a tile boundary or with the sequence (t1 <= n): the second tile of the last step may lie
-            // past it, then its loads are of no rows and its tokens are masked by the limit t1
-            for (int tile = t0; tile < t1; tile += 64) {
-                const int tl[2] = {tile, tile + 32};
-                const int r0 = chunk_rows(tile + 64), r1 = chunk_rows(tile + 96);
-                pair_scan_tile_x2<R>(L, S, t2, tl, t1,
-                                     [&]() { issue_k(t2[0], tile + 64, r0); issue_k(t2[1], tile + 96, r1); },
-                                     [&]() { issue_n(t2[0], tile + 64, r0); issue_n(t2[1], tile + 96, r1); },
-                                     [&]() { issue_v(t2[0], tile + 64, r0); issue_v(t2[1], tile + 96, r1); });
-            }
-        } else
         for (int tile = t0; tile < t1; tile += 32) {
             const bool more = tile + 32 < t1;
             int pages = 0;
@@ -362,13 +340,10 @@ void launch_attention_pair_scan(const AttnArgs& a, hipStream_t s) {
     const int R = a.num_heads / a.num_kv_heads;
     const dim3 g3(grid), b3(ngroups * waves * kWave);
     note_scan_kernel("attention_pair_kernel");
-#ifndef TW_PAIR_X2
-#define TW_PAIR_X2 1
-#endif
-#define TW_LAUNCH(P, RR, BB, TT) launch_scan_kernel(attention_pair_kernel<P, RR, BB, TT>, g3, b3, s, a, items, hgroups, waves)
-#define TW_LAUNCH_R(P, BB, TT) do { if (R == 1) TW_LAUNCH(P, 1, BB, TT); else if (R == 2) TW_LAUNCH(P, 2, BB, TT); else TW_LAUNCH(P, 4, BB, TT); } while (0)
-    if (a.bits == 4) { if (a.block_table) TW_LAUNCH_R(true, 4, 1); else TW_LAUNCH_R(false, 4, 1); }
-    else { if (a.block_table) TW_LAUNCH_R(true, 2, 1); else TW_LAUNCH_R(false, 2, TW_PAIR_X2 ? 2 : 1); }
+#define TW_LAUNCH(P, RR, BB) launch_scan_kernel(attention_pair_kernel<P, RR, BB>, g3, b3, s, a, items, hgroups, waves)
+#define TW_LAUNCH_R(P, BB) do { if (R == 1) TW_LAUNCH(P, 1, BB); else if (R == 2) TW_LAUNCH(P, 2, BB); else TW_LAUNCH(P, 4, BB); } while (0)
+    if (a.bits == 4) { if (a.block_table) TW_LAUNCH_R(true, 4); else TW_LAUNCH_R(false, 4); }
+    else { if (a.block_table) TW_LAUNCH_R(true, 2); else TW_LAUNCH_R(false, 2); }
 #undef TW_LAUNCH_R
 #undef TW_LAUNCH
 }

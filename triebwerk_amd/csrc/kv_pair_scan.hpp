@@ -327,160 +327,6 @@ __device__ __forceinline__ void pair_scan_tile(const PairLane<R, BITS>& L, PairS
     __builtin_amdgcn_s_setprio(0);
 }
 
-// Two tiles of the 2-bit cache as ONE step of the loop (first tokens tile[0] and tile[1], registers t[0] and t[1]): the
-// scores of both, one pass of the online softmax over the lane's four (token, head) pairs -- one decision about the
-// running maximum, one rescale, one fence and one hand-over of the probabilities through the wave's P tile (two
-// 16 x 32 sub-tiles, 2 KB) -- then both P.V products.  A 2-bit tile is half the bytes of a 4-bit one for the same
-// bookkeeping per tile; this form pays that bookkeeping once per 64 tokens and keeps two tiles of loads in flight.
-// `n`: tokens at or past it are masked (the end of the sequence or of the caller's chunk).
-template <int R, class AfterK, class AfterN, class AfterV>
-__device__ __forceinline__ void pair_scan_tile_x2(const PairLane<R, 2>& L, PairState<R>& S, PairTileRegs<2> (&t)[2],
-                                                  const int (&tile)[2], int n, AfterK after_k, AfterN after_n, AfterV after_v) {
-    constexpr float kRaise = 5.0f;
-    constexpr int kAhead = 4;
-    // ---- scores
-    float4_t s[2][4];
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        uint2 klo[kAhead], khi[kAhead];
-        auto look = [&](int i, uint2& lo, uint2& hi) {
-            const uint32_t w = t[u].k[i >> 2][(i & 3) >> 1];
-            const uint32_t sel = 0x0c0c0400u + ((uint32_t)(2 * (i & 1)) << 8);
-            lo = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel));
-            hi = L.lut64(__builtin_amdgcn_perm(w, L.lane_rep, sel + 0x100u));
-        };
-#pragma unroll
-        for (int i = 0; i < kAhead; i++) look(i, klo[i], khi[i]);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            union { uint32_t w[4]; half8_t h; } kv;
-            kv.w[0] = klo[i % kAhead].x; kv.w[1] = klo[i % kAhead].y; kv.w[2] = khi[i % kAhead].x; kv.w[3] = khi[i % kAhead].y;
-            if (i + kAhead < 16) look(i + kAhead, klo[i % kAhead], khi[i % kAhead]);
-            asm volatile("" ::: "memory");
-            if ((i & 3) == 0) s[u][i >> 2] = float4_t{0.f, 0.f, 0.f, 0.f};
-            s[u][i >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(S.aq[i & 3], kv.h, s[u][i >> 2], 0, 0, 0);
-        }
-    }
-    after_k();
-    __builtin_amdgcn_s_setprio(1);
-
-    // ---- online softmax over tokens tok0, tok0 + 16 of both tiles
-    float kn[2][2], vn[2][2];
-    bool valid[2][2];
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            kn[u][i] = h2f_bits((t[u].n[i][0] >> L.nshift) & 0xffffu);
-            vn[u][i] = h2f_bits((t[u].n[i][1] >> L.nshift) & 0xffffu);
-            valid[u][i] = L.useful && (tile[u] + L.tok0 + 16 * i < n);
-        }
-    }
-    after_n();
-    float raw[2][2][R], x[2][2][R];
-    bool raise = false;
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            uint32x2_t s01 = __builtin_amdgcn_permlane32_swap(__float_as_uint(s[u][0][r]), __float_as_uint(s[u][1][r]), false, false);
-            uint32x2_t s23 = __builtin_amdgcn_permlane32_swap(__float_as_uint(s[u][2][r]), __float_as_uint(s[u][3][r]), false, false);
-            raw[u][0][r] = (__uint_as_float(s01[0]) + __uint_as_float(s01[1])) * kn[u][0];    // kernels.cu:1707
-            raw[u][1][r] = (__uint_as_float(s23[0]) + __uint_as_float(s23[1])) * kn[u][1];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                x[u][i][r] = valid[u][i] ? raw[u][i][r] - S.m_run[r] : kNegBig;
-                raise = raise || (x[u][i][r] > kRaise);
-            }
-        }
-    }
-    if (__any(raise)) {
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            float mine = kNegBig;
-#pragma unroll
-            for (int u = 0; u < 2; u++)
-#pragma unroll
-                for (int i = 0; i < 2; i++) mine = fmaxf(mine, valid[u][i] ? raw[u][i][r] : kNegBig);
-            const float m_new = fmaxf(S.m_run[r], L.head_max(mine));
-            const float alpha = __builtin_amdgcn_exp2f(S.m_run[r] - m_new);
-            S.m_run[r] = m_new;
-            S.l_run[r] *= alpha;
-#pragma unroll
-            for (int u = 0; u < 2; u++)
-#pragma unroll
-                for (int i = 0; i < 2; i++) x[u][i][r] = valid[u][i] ? raw[u][i][r] - m_new : kNegBig;
-#pragma unroll
-            for (int j = 0; j < 16; j++) S.o[j][r] *= alpha;
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const float pe = __builtin_amdgcn_exp2f(x[u][i][r]);
-                S.l_run[r] += pe;
-                const float pf = pe * vn[u][i];                         // (s * vn) * centroid, kernels.cu:1765
-                const half_t hi = (half_t)pf;
-                const half_t lo = (half_t)(pf - (float)hi);
-                if (R < 4 || L.useful) {
-                    L.p_w[u * 512 + r * 32 + 4 * i] = hi;
-                    L.p_w[u * 512 + (r + 8) * 32 + 4 * i] = lo;
-                }
-            }
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    union { uint4 q; half8_t h; } pa[2];
-    pa[0].q = L.p_r[0];
-    pa[1].q = L.p_r[64];
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-
-    __builtin_amdgcn_s_setprio(2);
-    // ---- P.V of both tiles (the transposition of the 2-bit fields as in pair_scan_tile)
-    uint32_t y[2][2][4];
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++) {
-            const uint32_t w0 = t[u].v[sub][0], w1 = t[u].v[sub][1], w2 = t[u].v[sub][2], w3 = t[u].v[sub][3];
-            const uint32_t xe01 = (w0 & 0x33333333u) | ((w1 << 2) & 0xccccccccu), xo01 = ((w0 >> 2) & 0x33333333u) | (w1 & 0xccccccccu);
-            const uint32_t xe23 = (w2 & 0x33333333u) | ((w3 << 2) & 0xccccccccu), xo23 = ((w2 >> 2) & 0x33333333u) | (w3 & 0xccccccccu);
-            y[u][sub][0] = (xe01 & 0x0f0f0f0fu) | ((xe23 << 4) & 0xf0f0f0f0u);
-            y[u][sub][1] = ((xe01 >> 4) & 0x0f0f0f0fu) | (xe23 & 0xf0f0f0f0u);
-            y[u][sub][2] = (xo01 & 0x0f0f0f0fu) | ((xo23 << 4) & 0xf0f0f0f0u);
-            y[u][sub][3] = ((xo01 >> 4) & 0x0f0f0f0fu) | (xo23 & 0xf0f0f0f0u);
-        }
-    }
-    after_v();
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        uint2 qa[kAhead], qb[kAhead];
-        auto look = [&](int j, uint2& a4, uint2& b4) {
-            constexpr int kWhich[4] = {0, 2, 1, 3};
-            const int m = kWhich[j & 3];
-            const uint32_t sel = 0x0c0c0400u + ((uint32_t)(j >> 2) << 8);
-            a4 = L.lut64(__builtin_amdgcn_perm(y[u][0][m], L.lane_rep, sel));
-            b4 = L.lut64(__builtin_amdgcn_perm(y[u][1][m], L.lane_rep, sel));
-        };
-#pragma unroll
-        for (int j = 0; j < kAhead; j++) look(j, qa[j], qb[j]);
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            union { uint32_t w[4]; half8_t h; } bv;
-            bv.w[0] = qa[j % kAhead].x; bv.w[1] = qa[j % kAhead].y; bv.w[2] = qb[j % kAhead].x; bv.w[3] = qb[j % kAhead].y;
-            if (j + kAhead < 16) look(j + kAhead, qa[j % kAhead], qb[j % kAhead]);
-            asm volatile("" ::: "memory");
-            S.o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[u].h, bv.h, S.o[j], 0, 0, 0);
-        }
-    }
-    __builtin_amdgcn_s_setprio(0);
-}
-
 // The wave's partial result per (head of the pair, query head): sink(hd, r, dims) is called by the 16 lanes that
 // hold the rows of head hd with dims = the lane's 16 values of dim 16 (pn % 8) .. +15 (value + remainder rows added,
 // 1 / alpha applied); all lanes end with l_run summed over the head.
