@@ -388,6 +388,9 @@ def main():
     ap.add_argument("--one-launch", type=int, default=None, choices=[0, 1, 2, 3],
                     help="decode step of a compressed layer as one kernel: 0 by max_seq_len, 1 whenever possible, 2 never "
                          "(default: what the engine picks from the spread of the context lengths)")
+    ap.add_argument("--fused-shape", default=None, metavar="HKW,SHARES",
+                    help="force the one-launch step's KV heads per workgroup and workgroups per (sequence, head group); "
+                         "0 = the library's choice")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--producers", default="none", choices=["none", "fused", "separate"],
@@ -550,6 +553,8 @@ def decode_bench(args, kv_bits, with_probe):
     if args.one_launch is not None:
         kvcache.set_decode_fused(args.one_launch)
     kvcache.set_num_splits(args.nsplit)
+    if args.fused_shape:
+        kvcache.set_fused_shape(*[int(x) for x in args.fused_shape.split(",")])
     eng = Engine(max_seq_len=msl, kv_bits=kv_bits)
     eng.set_shape(L, H, Hk, D)
     eng.alloc_batch(G, msl)

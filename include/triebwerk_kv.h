@@ -198,6 +198,14 @@ const char* tw_kv_debug_last_scan_kernel(void);
  * which leave CUs idle, and for those in between; at 4096 tokens one launch up to batch 128 at both widths.
  * Alignment of the buffers, which the entry point also checks, is not part of it. */
 int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max);
+/* The same for a caller that hands the step tickets (tw_layer_step_args::tickets; can_share != 0): the one launch may
+ * then give a sequence's context to up to eight workgroups where the batch alone leaves compute units idle, which
+ * makes it the choice for small batches of long sequences too (16 sequences of 4096 or 8192 tokens). */
+int tw_kv_decode_step_plan2(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max,
+                            int can_share);
+/* Test hook: KV heads per workgroup (0 = automatic; 1, 2, 4, 8) and workgroups per sequence and head group (0 =
+ * automatic; 1, 2, 4 -- more than 1 only where the call has tickets) of the one-launch decode step. */
+void tw_kv_debug_set_fused_shape(int hkw, int shares);
 /* Layer steps that took the one-launch kernel since the library was loaded (launches issued or recorded into a
  * graph under capture): lets a benchmark say which kernel its figures belong to. */
 long long tw_kv_decode_fused_launches(void);
@@ -315,6 +323,11 @@ typedef struct tw_layer_step_args {
     long long gate_stride;
     int ctx_min, ctx_max;      /* what the host knows of min and max over g of positions[g] + 1; 0, 0 = nothing.
                                 * Only steers the choice between kernels (tw_kv_debug_set_decode_fused), never results. */
+    unsigned* tickets;         /* NULL, or G*num_kv_heads device words that are ZERO before the first call and that
+                                * only these calls touch (every call leaves them zero): with them, the one-launch step
+                                * of a compressed layer may give a sequence's context to two, four or eight workgroups when
+                                * the batch alone leaves compute units idle (their sums meet in `scratch`).  Calls that
+                                * share tickets must not overlap.  Decode step only. */
 } tw_layer_step_args;
 void tw_layer_attention_step(const tw_layer_step_args* args, hipStream_t s);
 

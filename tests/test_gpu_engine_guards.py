@@ -109,10 +109,12 @@ def test_engine_captured_step_follows_the_plan(oracle):
     from triebwerk_amd import Engine, _lib
     lib = _lib.load()
     r = gen.rng(8803)
-    L, H, Hk, G, msl, bits = 2, 16, 8, 2, 4352, 4
+    # (the engine hands the step its tickets, so small batches of long sequences stay on the one launch with their
+    # contexts shared by workgroups: a batch that fills the compute units by itself is what changes over)
+    L, H, Hk, G, msl, bits = 2, 16, 8, 72, 4352, 4
     kv_dim, q_dim = Hk * D, H * D
-    assert lib.tw_kv_decode_step_plan(G, H, Hk, bits, msl, 11, 11) == 1
-    assert lib.tw_kv_decode_step_plan(G, H, Hk, bits, msl, 4201, 4201) == 0
+    assert lib.tw_kv_decode_step_plan2(G, H, Hk, bits, msl, 11, 11, 1) == 1
+    assert lib.tw_kv_decode_step_plan2(G, H, Hk, bits, msl, 4201, 4201, 1) == 0
     eng = Engine(kv_bits=bits)
     eng.set_shape(L, H, Hk, D)
     eng.alloc_batch(G, msl)

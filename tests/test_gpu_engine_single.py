@@ -100,6 +100,45 @@ def test_single_sequence_tokens_against_the_oracle(oracle, rotation_fixture, kv_
                 assert_bytes_equal(host(t), caches[l][i], f"after the hand-set position: layer {l} array {i}")
 
 
+@pytest.mark.parametrize("kv_bits", [4, 2])
+def test_single_sequence_long_context_is_shared_by_workgroups(oracle, kv_bits):
+    """One sequence of a few thousand tokens: the layer step takes the one-launch kernel with the context shared by
+    workgroups (the engine hands its tickets over); random cache bytes, three tokens in a row against the oracle."""
+    import torch
+    from triebwerk_amd import Engine, kvcache
+    L, H, Hk, msl = 2, 16, 8, 4200
+    kv_dim, q_dim = Hk * D, H * D
+    r = gen.rng(9340 + kv_bits)
+    eng = Engine(max_seq_len=msl, kv_bits=kv_bits)
+    eng.set_shape(L, H, Hk, D)
+    eng.alloc_single()
+    rot = host(eng.single_rotation())
+    kvp = kv_dim * kv_bits // 8
+    caches = []
+    for l in range(L):
+        c = [r.integers(0, 256, (msl, kvp), dtype=np.uint8), r.integers(0, 256, (msl, kvp), dtype=np.uint8),
+             (11.3 + 0.7 * r.standard_normal((msl, Hk))).astype(np.float16), (11.3 + 0.7 * r.standard_normal((msl, Hk))).astype(np.float16)]
+        for t, a in zip(eng.single_cache(l), c):
+            t.copy_(dev(a))
+        caches.append(c)
+    start = 4100
+    eng.single_set_pos(start)
+    for tok in range(3):
+        pos = eng.single_pos()
+        print(f"single long context kv_bits={kv_bits} pos={pos}", flush=True)
+        for l in range(L):
+            q = gen.normal_f16(r, (q_dim,)); k = gen.normal_f16(r, (kv_dim,)); v = gen.normal_f16(r, (kv_dim,))
+            out = torch.zeros(q_dim, dtype=torch.float16, device="cuda")
+            eng.single_step(l, dev(q), dev(k), dev(v), out)
+            assert "context shared" in kvcache.last_scan_kernel(), kvcache.last_scan_kernel()
+            want = _oracle_single_layer(oracle, caches[l], q, k, v, rot, pos, msl, H, Hk, kv_bits)
+            assert rel_err(host(out), want) <= TOL, f"token at {pos}, layer {l}"
+        eng.single_advance()
+    for l in range(L):
+        for i, t in enumerate(eng.single_cache(l)):
+            assert_bytes_equal(host(t)[start - 2:start + 5], caches[l][i][start - 2:start + 5], f"layer {l} array {i}")
+
+
 def test_single_state_sleep_wake_and_batch_side_by_side(oracle):
     """sleep frees the single-sequence caches, wake re-allocates them (zeroed, position 0) when the engine had them;
     an engine that never had them gets none from wake; the batch arena and the single-sequence state do not touch
@@ -210,18 +249,18 @@ def test_decode_goes_on_without_a_graph_when_capture_fails(oracle, capfd, kv_bit
 
 
 def test_graph_replay_equals_the_eager_step_across_a_plan_flip_at_full_size():
-    """BASELINE config 4's shape (36 layers, 32 heads over 8 KV heads, 2 bit, 16 sequences) around the context where
-    tw_kv_decode_step_plan changes its answer: an engine that replays a captured step and one that runs every step
-    eagerly take the same plan at every step (both go by the positions the host knows), so their outputs and caches
-    are equal bit for bit before, at and after the flip, and the flip happens inside the run."""
+    """28 layers, 16 heads over 8 KV heads, 2 bit, 80 sequences around the context where tw_kv_decode_step_plan2 changes
+    its answer for a caller with tickets: an engine that replays a captured step and one that runs every step eagerly
+    take the same plan at every step (both go by the positions the host knows), so their outputs and caches are equal
+    bit for bit before, at and after the change, and the change happens inside the run."""
     import torch
     from triebwerk_amd import Engine, _lib
     lib = _lib.load()
-    L, H, Hk, G, bits = 36, 32, 8, 16, 2
+    L, H, Hk, G, bits = 28, 16, 8, 80, 2
     kv_dim, q_dim = Hk * D, H * D
-    msl = 8192
-    flip = next(c for c in range(2, msl) if lib.tw_kv_decode_step_plan(G, H, Hk, bits, msl, c, c) == 0)
-    assert lib.tw_kv_decode_step_plan(G, H, Hk, bits, msl, flip - 1, flip - 1) == 1 and flip + 8 < msl
+    msl = 4352
+    flip = next(c for c in range(2, msl) if lib.tw_kv_decode_step_plan2(G, H, Hk, bits, msl, c, c, 1) == 0)
+    assert lib.tw_kv_decode_step_plan2(G, H, Hk, bits, msl, flip - 1, flip - 1, 1) == 1 and flip + 8 < msl
     start = flip - 5                     # contexts of the steps: start + 1 .. start + 8, the flip among them
     gt = torch.Generator(device="cuda"); gt.manual_seed(97)
     engines = []

@@ -128,6 +128,17 @@ def test_decode_step_plan_is_the_documented_rule():
     assert plan(16, 16, 8, 4, 8448, 8192, 8192) == 0
     assert plan(32, 16, 8, 4, 8448, 8192, 8192) == 0
     assert plan(16, 16, 8, 4, 8448, 2048, 2048) == 1
+    # a caller with tickets (the engine): the one launch may share a sequence's context between workgroups, which makes
+    # it the choice for small batches of long sequences too; nothing changes where the batch fills the GPU or is ragged
+    plan2 = lib.tw_kv_decode_step_plan2
+    assert plan2(16, 32, 8, 2, 4352, 4097, 4097, 1) == 1          # BASELINE config 4
+    assert plan2(4, 16, 8, 4, 16384, 16000, 16000, 1) == 1
+    assert plan2(16, 16, 8, 4, 8448, 8192, 8192, 1) == 1
+    assert plan2(32, 16, 8, 4, 8448, 8192, 8192, 1) == 1
+    assert plan2(16, 16, 8, 4, 8448, 8192, 8192, 0) == 0
+    assert plan2(64, 16, 8, 4, 8448, 8192, 8192, 1) == 1 and plan2(96, 16, 8, 2, 8448, 8192, 8192, 1) == 0
+    assert plan2(64, 16, 8, 4, 8448, 512, 8192, 1) == 0
+    assert plan2(16, 16, 8, 4, 400, 0, 0, 1) == 1                 # too little scratch for shares: as without
     assert plan(16, 32, 8, 2, 4352, 4097, 4097) == 1          # 2 bit, GQA 4, 65k tokens
     # batches that fill three quarters of the CUs with two or four heads per workgroup
     assert plan(48, 16, 8, 4, 8448, 8192, 8192) == 1

@@ -24,7 +24,7 @@ class LayerStepArgs(C.Structure):
                 ("q_weight", P), ("k_weight", P), ("eps", C.c_float), ("biased", I),
                 ("cos_table", P), ("sin_table", P), ("rope_dim", I),
                 ("kv_bits", I), ("cache_k", P), ("cache_v", P), ("k_norms", P), ("v_norms", P), ("rotation", P),
-                ("scratch", P), ("gate", P), ("gate_stride", LL), ("ctx_min", I), ("ctx_max", I)]
+                ("scratch", P), ("gate", P), ("gate_stride", LL), ("ctx_min", I), ("ctx_max", I), ("tickets", P)]
 
 
 class ModelShape(C.Structure):
@@ -62,6 +62,8 @@ SIGNATURES = {
     "tw_kv_debug_last_scan_kernel": (C.c_char_p, []),
     "tw_kv_decode_fused_launches": (LL, []),
     "tw_kv_decode_step_plan": (I, [I, I, I, I, I, I, I]),
+    "tw_kv_decode_step_plan2": (I, [I, I, I, I, I, I, I, I]),
+    "tw_kv_debug_set_fused_shape": (None, [I, I]),
     "tw_kv_debug_profile_attention": (None, [I]),
     "tw_kv_debug_profile_read": (I, [C.POINTER(C.c_double), C.POINTER(I)]),
     "tw_kv_measure_read_bandwidth": (C.c_double, [P, C.c_size_t, I, P]),

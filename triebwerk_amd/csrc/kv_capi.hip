@@ -232,7 +232,15 @@ void tw_kv_debug_set_num_splits(int n) { g_nsplit_override.store(n); }
 void tw_kv_debug_set_prefill_form(int form) { g_prefill_form.store(form); }
 void tw_kv_debug_set_decode_fused(int mode) { g_decode_fused.store(mode); }
 
-int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max) {
+// shares' sums that fit the attention scratch (max_seq_len floats per sequence and head): a power of two up to 8
+static int shares_that_fit(int max_seq_len) {
+    int n = 1;
+    while (n < 8 && 2 * n * kPartialFloats <= max_seq_len) n *= 2;
+    return n;
+}
+
+int tw_kv_decode_step_plan2(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max,
+                            int can_share) {
     if (G <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || (bits != 2 && bits != 4)) return 0;
     const int group = num_heads / num_kv_heads;
     if (group != 1 && group != 2 && group != 4) return 0;
@@ -244,13 +252,19 @@ int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int
     if (bound <= 256 * split) return 1;                           // at most 8 tiles of 32 tokens per wave
     if (!known || (long long)(ctx_max - ctx_min) * 8 > ctx_max) return 0;   // lengths unknown or ragged: the balanced walk
     // Equal lengths: the cheaper of the two by estimates fitted to launches measured on MI355X (microseconds per
-    // layer): one launch as decode_fused_estimate_us counts it; three launches: 27 us (25 at 2 bit) of launches, query
-    // rotation and merge, and the scan at its rate.
+    // layer): one launch as decode_fused_shape counts it (with a sequence's context shared by workgroups where the
+    // caller can hand over tickets and the batch alone leaves compute units idle); three launches: 27 us (25 at 2 bit)
+    // of launches, query rotation and merge, and the scan at its rate.
     const double bpt = bits == 4 ? 132.0 : 68.0;                  // bytes per token and KV head: K and V codes and norms
-    const double one = decode_fused_estimate_us(G, num_heads, num_kv_heads, bits, allow_pairs, hkw, ctx_max);
+    const int max_shares = can_share != 0 ? shares_that_fit(max_seq_len) : 1;
+    const double one = decode_fused_shape(G, num_heads, num_kv_heads, bits, allow_pairs, max_shares, ctx_max).us;
     const double three = (bits == 4 ? 27.0 : 25.0) + (double)G * num_kv_heads * bpt * ctx_max / (bits == 4 ? 7.2e6 : 5.4e6);
     return one <= three ? 1 : 0;
 }
+int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max) {
+    return tw_kv_decode_step_plan2(G, num_heads, num_kv_heads, bits, max_seq_len, ctx_min, ctx_max, 0);
+}
+void tw_kv_debug_set_fused_shape(int hkw, int shares) { decode_fused_force_shape(hkw, shares); }
 long long tw_kv_decode_fused_launches(void) { return g_fused_launches.load(); }
 const char* tw_kv_debug_last_scan_kernel(void) { return twkv::g_last_scan_kernel; }
 
@@ -603,6 +617,9 @@ void launch_turbo_gqa_attention_batch(tw_half* out, const tw_half* q, const uint
 // (0, 0 = unknown), for the call being set up on this thread.
 static thread_local int t_ctx_min = 0;
 static thread_local int t_ctx_max = 0;
+// Its tickets (tw_layer_step_args::tickets): with them the one-launch step may share a sequence's context between
+// workgroups; the shares' sums go to the attention scratch.
+static thread_local unsigned* t_tickets = nullptr;
 
 // The whole step in one launch (kv_decode_fused.hip)?  There one workgroup owns a sequence's heads from the first
 // token to the last: it saves two launches and the scan's ramp (~10 us of a layer) and loses to the three-kernel
@@ -628,7 +645,13 @@ static bool try_decode_fused(const AttnArgs& a, const FusedArgs& f_in, int msl, 
     f.ctx_bound = t_ctx_max > 0 ? (t_ctx_max < msl ? t_ctx_max : msl) : msl;
     if (mode == 2 || g_variant.load() == 1) return false;
     if (!decode_fused_usable(a, f)) return false;
-    if (mode != 1 && mode != 3 && !tw_kv_decode_step_plan(a.G, a.num_heads, a.num_kv_heads, a.bits, msl, t_ctx_min, t_ctx_max)) return false;
+    // shares: the caller's tickets, and the attention scratch (G * num_heads * msl floats) for up to four shares' sums
+    const bool can_share = t_tickets != nullptr && a.ws != nullptr && shares_that_fit(msl) >= 2 &&
+                           (reinterpret_cast<uintptr_t>(a.ws) & 3u) == 0;
+    f.max_shares = 1;
+    if (can_share) { f.tickets = t_tickets; f.share_ws = a.ws; f.max_shares = shares_that_fit(msl); }
+    if (mode != 1 && mode != 3 &&
+        !tw_kv_decode_step_plan2(a.G, a.num_heads, a.num_kv_heads, a.bits, msl, t_ctx_min, t_ctx_max, can_share ? 1 : 0)) return false;
     attach_profiler(s);
     g_fused_launches.fetch_add(1);
     launch_decode_fused(a, f, s, /*allow_pairs=*/mode != 3);
@@ -876,6 +899,7 @@ void tw_layer_attention_step(const tw_layer_step_args* p, hipStream_t s) {
     t_gate_stride = p->gate ? p->gate_stride : 0;
     t_ctx_min = p->ctx_max > 0 ? p->ctx_min : 0;
     t_ctx_max = p->ctx_max > 0 ? p->ctx_max : 0;
+    t_tickets = p->tickets;
     if (p->kv_bits == 0) {
         if (producers) {
             tw_qk_norm_rope_append_attention_batch(p->out, p->q, p->k, p->v, p->q_weight, p->k_weight, p->eps, p->biased,
@@ -901,6 +925,7 @@ void tw_layer_attention_step(const tw_layer_step_args* p, hipStream_t s) {
     t_gate = nullptr;
     t_gate_stride = 0;
     t_ctx_min = t_ctx_max = 0;
+    t_tickets = nullptr;
 }
 
 // Steps 3-5b of a layer over a prompt (prefill_chunked, engine.cpp:2097-2150): rows are the prompt's tokens,

@@ -37,6 +37,7 @@
 // invalidation of the XCD's L2, cost 34 us per launch; with no fence at all, which is not correct, the launch took
 // 99 us against 97: the scan is not held up by the access pattern.)
 
+#include <atomic>
 #include <cmath>
 
 #include "kv_common.hpp"
@@ -57,6 +58,7 @@ constexpr unsigned kPairTileShare = 32;        // the same with eight waves in a
 constexpr int kFusedMaxQ = 32;                 // query heads of a unit: HKW * R <= 8 * 4
 constexpr int kRowFloats = kHeadDim + 4;       // LDS row of a vector: conflict-free 16-byte accesses
 constexpr int kStageStride = 2 * kHeadDim + 16;   // bytes per staged fp16 vector
+constexpr int kMaxShares = 8;                  // workgroups that may share one sequence's context
 static_assert(8 * (2 + 4) * kStageStride <= kFusedMaxQ * kRowFloats * 4, "staged vectors fit the output rows");
 
 }  // namespace
@@ -64,7 +66,15 @@ static_assert(8 * (2 + 4) * kStageStride <= kFusedMaxQ * kRowFloats * 4, "staged
 // EARLY (PAIR only): waves ask for their first tile in the middle of the prologue; for launches whose waves have few
 // tiles (the host decides from what it knows of the context lengths).  A template parameter because the mere presence
 // of that path, never taken, made the long-context launch 2 us slower.
-template <int R, int BITS, bool PROD, bool PAIR, bool EARLY>
+// SHARES: f.shares (2, 4 or 8) workgroups share the context of a unit -- for batches whose units alone leave compute units
+// idle.  Share c scans the c-th of f.shares even runs of the sequence's tiles; the last share appends the new row.  Each
+// leaves its unnormalised sums in memory, draws a ticket, and the workgroup with the last ticket merges all of them (in
+// share order, all read back from memory: the result does not depend on who was last) and finishes the unit.  The
+// hand-over uses device-scope accesses only where they are needed -- the partial sums and the ticket -- and no
+// cache-wide fence: stores with device scope are written through to where every compute unit's device-scope loads look
+// (a release / acquire pair at device scope writes back and invalidates a whole L2 and costs 20 us per launch where this
+// costs 4-9 us with every workgroup of a full-size launch taking part, measured with a stand-alone probe).
+template <int R, int BITS, bool PROD, bool PAIR, bool EARLY, bool SHARES = false>
 __global__ void __launch_bounds__((PAIR ? kPairWaves : kFusedWaves) * kWave)
 decode_fused_kernel(AttnArgs a, FusedArgs f) {
     constexpr int NW = PAIR ? kPairWaves : kFusedWaves;        // waves of the workgroup
@@ -95,18 +105,23 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
 
     // ---- unit of this workgroup.  Workgroups are dealt to the 8 XCDs in turn; the units of one sequence
     // go to one XCD so that the norm rows they all read (16 bytes per token for 8 heads) come out of one L2.
-    int g, hg;
+    int g, hg, share = 0;
+    const int nshares = SHARES ? f.shares : 1;
     {
-        const int b = (int)blockIdx.x;
+        int b = (int)blockIdx.x;
         if ((a.G & 7) == 0) {
-            const int xcd = b & 7, j = b >> 3;
+            const int xcd = b & 7;
+            int j = b >> 3;
+            if (SHARES) { share = j % nshares; j /= nshares; }      // the shares of a unit on one XCD as well
             g = (j / nhg) * 8 + xcd;
             hg = j % nhg;
         } else {
+            if (SHARES) { share = b % nshares; b /= nshares; }
             g = b / nhg;
             hg = b % nhg;
         }
     }
+    const bool appends = !SHARES || share == nshares - 1;          // the share that holds the sequence's last tile
     // ---- operands of the rotations first: nothing about them depends on the position.  The unit's vectors
     // (K heads, V heads, query heads) are fetched once by all threads, 16 bytes each, and staged in LDS;
     // the rotating waves fetch their 16 rows of R.
@@ -169,7 +184,10 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     // which started together -- reads one window of consecutive rows (1.2 % faster at 8192 tokens than giving
     // every part one contiguous run).  The parts of the upper eight waves stop after `rounds` rounds (31/64 of
     // the tiles); what is left goes round the lower waves' parts.
-    const int ntile = (n + 31) >> 5;
+    const int ntile_seq = (n + 31) >> 5;
+    // SHARES: this workgroup's run of the sequence's tiles (even runs, the last one ends with the sequence)
+    const int tile_lo = SHARES ? (int)((long long)share * ntile_seq / nshares) : 0;
+    const int ntile = SHARES ? (int)((long long)(share + 1) * ntile_seq / nshares) - tile_lo : ntile_seq;
     const int halfparts = SPLIT >> 1;                      // SPLIT is 2, 4, 8 or 16
     const int lower = min(ntile, (int)((ntile * (PAIR ? kPairTileShare : kFusedShare) + 63u) / 64u));
     const int rounds = (ntile - lower) / halfparts;
@@ -177,7 +195,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     const int left = ntile - tail0 - part;
     const int ntiles = rounds + ((part < halfparts && left > 0) ? (left + halfparts - 1) / halfparts : 0);
     auto tile_at = [&](int i) -> int {                     // first token of this wave's i-th tile
-        return 32 * (i < rounds ? i * SPLIT + part : tail0 + part + (i - rounds) * halfparts);
+        return 32 * (tile_lo + (i < rounds ? i * SPLIT + part : tail0 + part + (i - rounds) * halfparts));
     };
     const int first_tile = tile_at(0);
 
@@ -390,7 +408,7 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
             uint32_t p1 = (uint32_t)__shfl((int)packed, i16 + 16, 64);
             uint32_t p2 = (uint32_t)__shfl((int)packed, i16 + 32, 64);
             uint32_t p3 = (uint32_t)__shfl((int)packed, i16 + 48, 64);
-            if (kk == 0 && vi < nvec && !is_query) {
+            if (kk == 0 && vi < nvec && !is_query && appends) {
                 constexpr int BPH = kHeadDim * BITS / 8;
                 const long long crow = seq_row0 + pos;
                 uint8_t* dst = (kind == 0 ? f.k_codes : f.v_codes) + (crow * Hk + head) * BPH + dblk * (2 * BITS);
@@ -718,12 +736,11 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
     {   // merge: thread -> (vector tid / 32, coordinates 4 * (tid % 32) .. +3); vector = (local KV head, query head)
         const int vec = tid >> 5, k4 = (tid & 31) * 4;
         float4 o4 = {0.f, 0.f, 0.f, 0.f};
+        float mg = kNegBig, lsum = 0.0f;
+        float4 av = {0.f, 0.f, 0.f, 0.f};
         if (vec < nv) {
             const int hk_l = vec / R, r = vec - hk_l * R;
-            float mg = kNegBig;
             for (int p = 0; p < SPLIT; p++) mg = fmaxf(mg, part_s[p * HKW + hk_l][r][kHeadDim]);
-            float lsum = 0.0f;
-            float4 av = {0.f, 0.f, 0.f, 0.f};
             for (int p = 0; p < SPLIT; p++) {
                 const float* pr = &part_s[p * HKW + hk_l][r][0];
                 const float fs = __builtin_amdgcn_exp2f(pr[kHeadDim] - mg);
@@ -734,6 +751,52 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
                 av.z = __builtin_fmaf(c.z, fs, av.z);
                 av.w = __builtin_fmaf(c.w, fs, av.w);
             }
+        }
+        if constexpr (SHARES) {
+            // this share's sums to memory (device scope: written through), then the ticket
+            __shared__ unsigned last_s;
+            const long long unit = (long long)g * nhg + hg;
+            auto slot = [&](int sh) -> float* { return f.share_ws + ((unit * nshares + sh) * nv + vec) * kRowFloats; };
+            auto put = [](float* p, float x) { __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+            auto get = [](const float* p) -> float { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+            if (vec < nv) {
+                float* mine = slot(share);
+                put(mine + k4, av.x); put(mine + k4 + 1, av.y); put(mine + k4 + 2, av.z); put(mine + k4 + 3, av.w);
+                if (k4 == 0) { put(mine + kHeadDim, mg); put(mine + kHeadDim + 1, lsum); }
+            }
+            __builtin_amdgcn_s_waitcnt(0);          // every store of this wave has been acknowledged
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned old = __hip_atomic_fetch_add(f.tickets + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last_s = old == (unsigned)nshares - 1u ? 1u : 0u;
+            }
+            __syncthreads();
+            if (!last_s) return;                    // uniform over the workgroup: the last share finishes the unit
+            if (tid == 0) __hip_atomic_store(f.tickets + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+            if (vec < nv) {
+                float ms[kMaxShares], ls[kMaxShares];
+                float4 as[kMaxShares];
+                mg = kNegBig;
+                for (int sh = 0; sh < nshares; sh++) {
+                    const float* p = slot(sh);
+                    as[sh] = float4{get(p + k4), get(p + k4 + 1), get(p + k4 + 2), get(p + k4 + 3)};
+                    ms[sh] = get(p + kHeadDim);
+                    ls[sh] = get(p + kHeadDim + 1);
+                    mg = fmaxf(mg, ms[sh]);
+                }
+                lsum = 0.0f;
+                av = float4{0.f, 0.f, 0.f, 0.f};
+                for (int sh = 0; sh < nshares; sh++) {
+                    const float fs = __builtin_amdgcn_exp2f(ms[sh] - mg);
+                    lsum = __builtin_fmaf(ls[sh], fs, lsum);
+                    av.x = __builtin_fmaf(as[sh].x, fs, av.x);
+                    av.y = __builtin_fmaf(as[sh].y, fs, av.y);
+                    av.z = __builtin_fmaf(as[sh].z, fs, av.z);
+                    av.w = __builtin_fmaf(as[sh].w, fs, av.w);
+                }
+            }
+        }
+        if (vec < nv) {
             const float inv = 1.0f / (lsum + 1e-8f);             // kernels.cu:1746
             o4 = float4{av.x * inv, av.y * inv, av.z * inv, av.w * inv};
         }
@@ -820,6 +883,43 @@ int decode_fused_heads_per_workgroup(int G, int num_heads, int Hk, int bits, boo
     return best;
 }
 
+// With shares: a launch of G * (Hk / hkw) * shares workgroups, each with 1 / shares of the context, plus what the
+// hand-over costs at the end (measured on MI355X with a probe in which all 512 workgroups of a streaming launch take
+// part: 3.7, 5.4 and 8.7 us for 2, 4 and 8 shares).  Shares are only taken while all workgroups fit the compute units
+// in one round and a share still has a tile for every wave.
+namespace {
+constexpr double kShareHandoverUs[4] = {0.0, 3.7, 5.4, 8.7};       // by log2(shares)
+std::atomic<int> g_force_hkw{0}, g_force_shares{0};
+}  // namespace
+void decode_fused_force_shape(int hkw, int shares) { g_force_hkw.store(hkw); g_force_shares.store(shares); }
+
+FusedShape decode_fused_shape(int G, int num_heads, int Hk, int bits, bool allow_pairs, int max_shares, double ctx) {
+    const bool can_share = max_shares >= 2;
+    const int R = Hk > 0 ? num_heads / Hk : 1;
+    const double cus = compute_units();
+    FusedShape best{decode_fused_heads_per_workgroup(G, num_heads, Hk, bits, allow_pairs), 1, 0.0};
+    best.us = decode_fused_estimate_us(G, num_heads, Hk, bits, allow_pairs, best.hkw, ctx);
+    if (can_share) {
+        for (int c = 1; c <= 8; c <<= 1) {
+            if (Hk % c != 0) continue;
+            const bool pair = allow_pairs && pairs_fit(bits, R, c);
+            const int parts = (pair ? 2 * kPairWaves : kFusedWaves) / c;          // waves (parts of the context) per head
+            for (int sh = 2, lg = 1; sh <= kMaxShares && sh <= max_shares; sh <<= 1, lg++) {
+                if ((double)G * (Hk / c) * sh > cus) continue;
+                if (ctx < 32.0 * parts * sh) continue;
+                // every share is a launch of its own size: G * shares "sequences" of ctx / shares tokens
+                const double us = decode_fused_estimate_us(G * sh, num_heads, Hk, bits, allow_pairs, c, ctx / sh) +
+                                  kShareHandoverUs[lg];
+                if (us < best.us) best = FusedShape{c, sh, us};
+            }
+        }
+    }
+    const int fh = g_force_hkw.load(), fs = g_force_shares.load();
+    if (fh > 0 && Hk % fh == 0) best.hkw = fh;
+    if (fs > 0) best.shares = fs <= max_shares && fs <= kMaxShares ? fs : 1;
+    return best;
+}
+
 bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
     const int R = a.num_kv_heads > 0 ? a.num_heads / a.num_kv_heads : 0;
     if (a.bits != 4 && a.bits != 2) return false;
@@ -839,20 +939,27 @@ bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f) {
 
 void launch_decode_fused(const AttnArgs& a, const FusedArgs& f_in, hipStream_t s, bool allow_pairs) {
     FusedArgs f = f_in;
-    f.hkw = decode_fused_heads_per_workgroup(a.G, a.num_heads, a.num_kv_heads, a.bits, allow_pairs);
+    const FusedShape shape = decode_fused_shape(a.G, a.num_heads, a.num_kv_heads, a.bits, allow_pairs,
+                                                f.share_ws != nullptr && f.tickets != nullptr ? f.max_shares : 1,
+                                                f.ctx_bound > 0 ? (double)f.ctx_bound : 4096.0);
+    f.hkw = shape.hkw;
+    f.shares = shape.shares;
     f.q_scale = attention_mfma_q_scale(a.bits);
     const int R = a.num_heads / a.num_kv_heads;
     const bool pair = allow_pairs && decode_fused_pairs(a, f.hkw);
-    const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw))), b3((pair ? kPairWaves : kFusedWaves) * kWave);
+    const dim3 g3((unsigned)(a.G * (a.num_kv_heads / f.hkw) * f.shares)), b3((pair ? kPairWaves : kFusedWaves) * kWave);
     const bool prod = f.q_weight != nullptr || f.cos_table != nullptr;
     // first tile in the middle of the prologue: when no wave gets more than 8 tiles of 32 tokens by the caller's bound
     // of the context (two heads per wave: 16 / hkw parts per head)
-    const bool early = pair && f.ctx_bound > 0 && f.ctx_bound <= 8 * 32 * (2 * kPairWaves / f.hkw);
-    note_scan_kernel(pair ? "decode_fused_kernel, two KV heads per wave" : "decode_fused_kernel, one KV head per wave");
-#define TW_FUSED_E(RR, BB, PP, EE) \
-    do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true, PP, EE>, g3, b3, s, a, f); \
-         else launch_scan_kernel(decode_fused_kernel<RR, BB, false, PP, EE>, g3, b3, s, a, f); } while (0)
-#define TW_FUSED(RR, BB, PP) do { if (PP && early) TW_FUSED_E(RR, BB, PP, PP); else TW_FUSED_E(RR, BB, PP, false); } while (0)
+    const bool early = pair && f.shares == 1 && f.ctx_bound > 0 && f.ctx_bound <= 8 * 32 * (2 * kPairWaves / f.hkw);
+    note_scan_kernel(pair ? (f.shares > 1 ? "decode_fused_kernel, two KV heads per wave, context shared by workgroups"
+                                          : "decode_fused_kernel, two KV heads per wave")
+                          : (f.shares > 1 ? "decode_fused_kernel, one KV head per wave, context shared by workgroups"
+                                          : "decode_fused_kernel, one KV head per wave"));
+#define TW_FUSED_E(RR, BB, PP, EE, SS) \
+    do { if (prod) launch_scan_kernel(decode_fused_kernel<RR, BB, true, PP, EE, SS>, g3, b3, s, a, f); \
+         else launch_scan_kernel(decode_fused_kernel<RR, BB, false, PP, EE, SS>, g3, b3, s, a, f); } while (0)
+#define TW_FUSED(RR, BB, PP) do { if (f.shares > 1) TW_FUSED_E(RR, BB, PP, false, true); else if (PP && early) TW_FUSED_E(RR, BB, PP, PP, false); else TW_FUSED_E(RR, BB, PP, false, false); } while (0)
 #define TW_FUSED_R(BB, PP) do { if (R == 1) TW_FUSED(1, BB, PP); else if (R == 2) TW_FUSED(2, BB, PP); else TW_FUSED(4, BB, PP); } while (0)
     if (a.bits == 4) { if (pair) TW_FUSED_R(4, true); else TW_FUSED_R(4, false); }
     else { if (pair) TW_FUSED_R(2, true); else TW_FUSED_R(2, false); }

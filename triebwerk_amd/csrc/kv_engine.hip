@@ -46,6 +46,7 @@ struct tw_engine {
     float* attn_scores = nullptr;     // G * num_heads * msl floats, engine.cpp:1371
     int* d_positions = nullptr;
     tw_half* d_rotation = nullptr;
+    unsigned* d_tickets = nullptr;    // G * num_kv_heads words for the one-launch step's shared contexts: zero between steps
 
     hipStream_t stream = nullptr;     // engine_stream_, engine.cpp:309
 
@@ -58,6 +59,7 @@ struct tw_engine {
     float* single_scores = nullptr;
     tw_half* single_rotation = nullptr;
     int* single_d_pos = nullptr;
+    unsigned* single_tickets = nullptr;   // num_kv_heads words, zero between steps (tw_layer_step_args::tickets)
     int single_pos = 0;
     bool single_allocated = false;
     bool single_wanted = false;       // wake() re-allocates what sleep() freed (engine.cpp:985-1022)
@@ -139,7 +141,7 @@ struct tw_engine {
         arena = nullptr; arena_cap = 0; arena_owned = false;
         G = 0; batch_msl = 0;
         memset(cache, 0, sizeof(cache));
-        attn_scores = nullptr; d_positions = nullptr; d_rotation = nullptr;
+        attn_scores = nullptr; d_positions = nullptr; d_rotation = nullptr; d_tickets = nullptr;
     }
 };
 
@@ -162,6 +164,7 @@ size_t arena_need(const tw_engine* e, int G, int msl) {
     }
     add((size_t)G * sizeof(int));                                                    // positions
     add((size_t)e->shape.head_dim * e->shape.head_dim * 2);                          // rotation
+    add((size_t)G * e->shape.num_kv_heads * sizeof(unsigned));                       // tickets
     return align256(need);
 }
 
@@ -183,6 +186,7 @@ int carve(tw_engine* e, int G, int msl) {
     }
     e->d_positions = (int*)take((size_t)G * sizeof(int));
     e->d_rotation = (tw_half*)take((size_t)e->shape.head_dim * e->shape.head_dim * 2);
+    e->d_tickets = (unsigned*)take((size_t)G * e->shape.num_kv_heads * sizeof(unsigned));
     if (off > e->arena_cap) return -1;
     e->G = G;
     e->batch_msl = msl;
@@ -225,6 +229,7 @@ void free_single(tw_engine* e) {
     if (e->single_scores) { hipFree(e->single_scores); e->single_scores = nullptr; }
     if (e->single_rotation) { hipFree(e->single_rotation); e->single_rotation = nullptr; }
     if (e->single_d_pos) { hipFree(e->single_d_pos); e->single_d_pos = nullptr; }
+    if (e->single_tickets) { hipFree(e->single_tickets); e->single_tickets = nullptr; }
     e->single_allocated = false;
 }
 
@@ -234,6 +239,7 @@ int zero_single(tw_engine* e) {
         for (int w = 0; w < 4; w++)
             if (e->single[i][w] && hipMemset(e->single[i][w], 0, rows * cache_row_bytes(e, w)) != hipSuccess) return -1;
     if (hipMemset(e->single_d_pos, 0, sizeof(int)) != hipSuccess) return -1;
+    if (hipMemset(e->single_tickets, 0, (size_t)e->shape.num_kv_heads * sizeof(unsigned)) != hipSuccess) return -1;
     e->single_pos = 0;
     return 0;
 }
@@ -246,8 +252,9 @@ bool cache_full(const tw_engine* e) { return e->pos_known && e->pos_max >= e->ba
 // (one launch per layer or three); the captured graph holds the launches of one such choice.
 int step_plan(const tw_engine* e) {
     if (e->kv_bits == 0) return 0;
-    return tw_kv_decode_step_plan(e->G, e->shape.num_heads, e->shape.num_kv_heads, e->kv_bits, e->batch_msl,
-                                  e->pos_known ? e->pos_min + 1 : 0, e->pos_known ? e->pos_max + 1 : 0);
+    return tw_kv_decode_step_plan2(e->G, e->shape.num_heads, e->shape.num_kv_heads, e->kv_bits, e->batch_msl,
+                                   e->pos_known ? e->pos_min + 1 : 0, e->pos_known ? e->pos_max + 1 : 0,
+                                   e->d_tickets != nullptr);
 }
 
 // forward_layer_batch steps 4-5 (with producers: 3-5), engine.cpp:1972-2006.
@@ -282,6 +289,7 @@ void layer_step(tw_engine* e, int layer, const tw_half* q, const tw_half* k, con
     p.rotation = e->d_rotation; p.scratch = e->attn_scores;
     // what the host knows of the context lengths (positions + 1, the appended token included)
     if (e->pos_known) { p.ctx_min = e->pos_min + 1; p.ctx_max = e->pos_max + 1; }
+    p.tickets = e->d_tickets;
     tw_layer_attention_step(&p, s);
 }
 
@@ -385,6 +393,7 @@ int tw_engine_reset(tw_engine* e) {
         for (int w = 0; w < 4; w++)
             if (e->cache[i][w]) hipMemsetAsync(e->cache[i][w], 0, rows * cache_row_bytes(e, w), s);
     hipMemsetAsync(e->d_positions, 0, (size_t)e->G * sizeof(int), s);
+    hipMemsetAsync(e->d_tickets, 0, (size_t)e->G * e->shape.num_kv_heads * sizeof(unsigned), s);
     e->pos_known = true;
     e->pos_min = e->pos_max = 0;
     return hipStreamSynchronize(s) == hipSuccess ? 0 : -1;
@@ -462,6 +471,7 @@ int tw_engine_alloc_single(tw_engine* e) {
         }
     ok = ok && hipMalloc((void**)&e->single_scores, (size_t)e->shape.num_heads * rows * sizeof(float)) == hipSuccess;
     ok = ok && hipMalloc((void**)&e->single_d_pos, sizeof(int)) == hipSuccess;
+    ok = ok && hipMalloc((void**)&e->single_tickets, (size_t)e->shape.num_kv_heads * sizeof(unsigned)) == hipSuccess;
     if (ok && e->kv_bits > 0) {
         const size_t n = (size_t)e->shape.head_dim * e->shape.head_dim;
         ok = hipMalloc((void**)&e->single_rotation, n * 2) == hipSuccess;
@@ -517,6 +527,7 @@ int tw_engine_single_step(tw_engine* e, int layer, const tw_half* q, const tw_ha
     p.k_norms = (tw_half*)e->single[layer][2]; p.v_norms = (tw_half*)e->single[layer][3];
     p.rotation = e->single_rotation; p.scratch = e->single_scores;
     p.ctx_min = p.ctx_max = e->single_pos + 1;
+    p.tickets = e->single_tickets;          // one sequence leaves most compute units idle: its context may be shared
     tw_layer_attention_step(&p, s);
     return tw_kv_last_error();
 }

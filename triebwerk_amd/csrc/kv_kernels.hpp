@@ -196,6 +196,11 @@ struct FusedArgs {
     int ctx_bound;          // in: upper bound of positions + 1 that the host knows (0: none)
     int hkw;                // KV heads per workgroup (launch_decode_fused fills this in)
     float q_scale;          // likewise
+    // A unit's context shared by several workgroups, for batches whose units alone leave compute units idle:
+    int shares;             // 1, 2, 4 or 8 (launch_decode_fused fills this in; > 1 only with the three below)
+    int max_shares;         // as many shares as share_ws has room for (1: none)
+    float* share_ws;        // G * num_heads * max_shares * (kHeadDim + 4) floats for the shares' unnormalised sums
+    unsigned* tickets;      // one word per (sequence, KV head): zero before the first launch, left zero by every launch
     // optional producers of q and k applied on the way in, as RotArgs has them (V rows stay as they are)
     const half_t* q_weight; // per-head RMSNorm weights (128); both or neither
     const half_t* k_weight;
@@ -209,6 +214,12 @@ bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f);
 int decode_fused_heads_per_workgroup(int G, int num_heads, int num_kv_heads, int bits, bool allow_pairs);   // 8, 4, 2 or 1
 // estimated microseconds of one launch with hkw KV heads per workgroup, all sequences at ctx tokens
 double decode_fused_estimate_us(int G, int num_heads, int num_kv_heads, int bits, bool allow_pairs, int hkw, double ctx);
+// The launch's shape when a unit's context may be shared by up to max_shares workgroups (1: the caller has no tickets
+// or no room for the shares' sums): KV heads per workgroup, shares, and the estimate for sequences of ctx tokens.
+struct FusedShape { int hkw, shares; double us; };
+FusedShape decode_fused_shape(int G, int num_heads, int num_kv_heads, int bits, bool allow_pairs, int max_shares, double ctx);
+// test hook (tw_kv_debug_set_fused_shape): force hkw and / or shares (0 = automatic)
+void decode_fused_force_shape(int hkw, int shares);
 // allow_pairs: the 4-bit kernel whose waves scan two KV heads each, where the shape admits it (false: one head per wave)
 void launch_decode_fused(const AttnArgs& a, const FusedArgs& f, hipStream_t s, bool allow_pairs);
 // causal prefill with blocks of query tokens per wave (kv_prefill_mfma.hip); same workspace and merge

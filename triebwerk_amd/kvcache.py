@@ -280,6 +280,12 @@ def set_decode_fused(mode: int) -> None:
     _lib.load().tw_kv_debug_set_decode_fused(int(mode))
 
 
+def set_fused_shape(hkw: int = 0, shares: int = 0) -> None:
+    """tw_kv_debug_set_fused_shape: KV heads per workgroup and workgroups per (sequence, head group) of the one-launch
+    decode step; 0 = the library's own choice."""
+    _lib.load().tw_kv_debug_set_fused_shape(int(hkw), int(shares))
+
+
 def last_scan_kernel() -> str:
     """Name of the kernel that the last decode-attention call launched for the context scan (a test hook)."""
     return _lib.load().tw_kv_debug_last_scan_kernel().decode()
@@ -373,7 +379,7 @@ def tw_layer_attention_step(out, q, k, v, positions, max_seq_len, G, num_heads, 
                             cache_k, cache_v, scratch, kv_bits=0, k_norms=None, v_norms=None, rotation=None,
                             q_weight=None, k_weight=None, eps=1e-6, biased=False, cos_table=None, sin_table=None,
                             rope_dim=0, gate=None, gate_stride=0, gate_offset=0, ctx_min=0, ctx_max=0, stream=None,
-                            prompt=False):
+                            prompt=False, tickets=None):
     """Steps 3-6 of a layer (producers, append, attention, gate) through tw_layer_attention_step.
     `gate` may be the q tensor itself with gate_offset = num_heads*head_dim (gated q projection).
     prompt=True: the rows are the G = T tokens of a prompt of sequence 0 (tw_layer_prompt_step)."""
@@ -394,6 +400,8 @@ def tw_layer_attention_step(out, q, k, v, positions, max_seq_len, G, num_heads, 
     a.gate = (gp + 2 * gate_offset) if gp is not None else None
     a.gate_stride = gate_stride
     a.ctx_min, a.ctx_max = int(ctx_min), int(ctx_max)       # host knowledge of positions + 1; 0, 0 = none
+    # G * num_kv_heads zeroed int32 words: lets the one-launch step share a sequence's context between workgroups
+    a.tickets = _ptr(tickets, "i32", "tickets")
     (lib.tw_layer_prompt_step if prompt else lib.tw_layer_attention_step)(_lib.C.byref(a), _stream(stream))
     _done(lib)
 
