@@ -508,7 +508,11 @@ decode_fused_kernel(AttnArgs a, FusedArgs f) {
         // own row only exists after the barrier that ends the rotations).  Rollouts of a few hundred tokens gain
         // 4.5 % (128 sequences at 257..768 tokens: 21.6 against 22.6 us per launch); with 8 tiles per wave it makes no
         // difference, and with 16 and more the launch gets slower (64 x 4096 tokens: + 0.6 us, x 8192: + 2.2 us), as
-        // with every other way of putting more requests in flight at the start that was tried.
+        // with every other way of putting more requests in flight at the start that was tried.  (A second register set
+        // in this short-context form, so that the tile after next is in flight too -- the memory is far from busy there:
+        // 22.9 against 21.2 us per launch on the rollout, 24.7 against 23.5 at 64 x 1024 tokens, 8 % and 5 % slower; with
+        // four query heads per KV head it does not fit the registers.  A wave's tile time at these sizes is the tile's
+        // own chain of look-ups and matrix instructions, not the wait for its loads.)
         const bool first_early = EARLY && ntiles > 0 && tile_at(0) + 32 <= pos;      // uniform over the wave
         rotate_unit([&]() {
             if (first_early) { set_next(0); issue_k(t); issue_n(t); issue_v(t); }
