@@ -251,14 +251,13 @@ int tw_kv_decode_step_plan2(int G, int num_heads, int num_kv_heads, int bits, in
     const int bound = known ? ctx_max : max_seq_len;
     if (bound <= 256 * split) return 1;                           // at most 8 tiles of 32 tokens per wave
     if (!known || (long long)(ctx_max - ctx_min) * 8 > ctx_max) return 0;   // lengths unknown or ragged: the balanced walk
-    // Equal lengths: the cheaper of the two by estimates fitted to launches measured on MI355X (microseconds per
-    // layer): one launch as decode_fused_shape counts it (with a sequence's context shared by workgroups where the
-    // caller can hand over tickets and the batch alone leaves compute units idle); three launches: 27 us (25 at 2 bit)
-    // of launches, query rotation and merge, and the scan at its rate.
-    const double bpt = bits == 4 ? 132.0 : 68.0;                  // bytes per token and KV head: K and V codes and norms
+    // Equal lengths: the cheaper of the two by estimates fitted to measured launches (microseconds per layer; the
+    // figures live in one table, plan_constants): one launch as decode_fused_shape counts it (with a sequence's context
+    // shared by workgroups where the caller can hand over tickets and the batch alone leaves compute units idle), three
+    // launches as decode_three_estimate_us does.
     const int max_shares = can_share != 0 ? shares_that_fit(max_seq_len) : 1;
     const double one = decode_fused_shape(G, num_heads, num_kv_heads, bits, allow_pairs, max_shares, ctx_max).us;
-    const double three = (bits == 4 ? 27.0 : 25.0) + (double)G * num_kv_heads * bpt * ctx_max / (bits == 4 ? 7.2e6 : 5.4e6);
+    const double three = decode_three_estimate_us(G, num_kv_heads, bits, ctx_max);
     return one <= three ? 1 : 0;
 }
 int tw_kv_decode_step_plan(int G, int num_heads, int num_kv_heads, int bits, int max_seq_len, int ctx_min, int ctx_max) {

@@ -39,6 +39,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <cstring>
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
@@ -854,22 +855,55 @@ static bool pairs_fit(int bits, int R, int hkw) {
 }
 bool decode_fused_pairs(const AttnArgs& a, int hkw) { return pairs_fit(a.bits, a.num_heads / a.num_kv_heads, hkw); }
 
+// The measured figures behind the estimates below.  MI355X: launches at batches 8 to 256 and contexts 1k to 8k
+// reproduce within 5 %; hand-over costs from a probe in which all 512 workgroups of a streaming launch take part.
+namespace {
+constexpr PlanConstants kPlanTable[] = {
+    {"gfx950", 12.0, {3.08, 2.72}, 2.45, {5.95, 4.68}, {7200.0, 5500.0}, {27.0, 25.0}, {7.2e6, 5.4e6}, {0.0, 3.7, 5.4, 8.7}},
+};
+}  // namespace
+const PlanConstants& plan_constants() {
+    static const PlanConstants* chosen = nullptr;
+    if (!chosen) {
+        const PlanConstants* pick = &kPlanTable[0];
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+            for (const PlanConstants& c : kPlanTable)
+                if (strstr(prop.gcnArchName, c.device)) { pick = &c; break; }
+        } else {
+            (void)hipGetLastError();           // no device (a host-only process asking for the plan): the first entry
+        }
+        chosen = pick;
+    }
+    return *chosen;
+}
+
 // Microseconds one launch takes for G sequences of ctx tokens with hkw KV heads per workgroup, by a count fitted to
-// launches measured on MI355X at batches 16 to 256 and contexts 1k to 8k (it reproduces them within 5 %): the
-// workgroups run in rounds of one per CU; a round costs 12 us of prologue and epilogue and, per token of context, the
-// cube-root sum of what one CU sustains for the workgroup's heads (a workgroup whose waves scan one head each moves
-// its bytes at about half the rate of one whose waves scan two) and of the whole chip's rate for all the workgroups
-// of the round.
+// measured launches (plan_constants): the workgroups run in rounds of one per CU; a round costs its fixed part and,
+// per token of context, the cube-root sum of what one CU sustains for the workgroup's heads (a workgroup whose waves
+// scan one head each moves its bytes at about half the rate of one whose waves scan two) and of the whole chip's rate
+// for all the workgroups of the round.
 double decode_fused_estimate_us(int G, int num_heads, int Hk, int bits, bool allow_pairs, int hkw, double ctx) {
+    const PlanConstants& pc = plan_constants();
     const double cus = compute_units();
     const int R = Hk > 0 ? num_heads / Hk : 1;
+    const int w = bits == 4 ? 0 : 1;
     const double bpt = bits == 4 ? 132.0 : 68.0;                  // bytes per token and KV head: K and V codes and norms
     const double units = (double)G * (Hk / hkw);
     const double rounds = std::ceil(units / cus), active = units < cus ? units : cus;
     const bool pair = allow_pairs && pairs_fit(bits, R, hkw);
-    const double per_head_ns = pair ? (bits == 4 ? 3.08 : hkw >= 4 ? 2.45 : 2.72) : (bits == 4 ? 5.95 : 4.68);
-    const double k_cu = hkw * per_head_ns, k_bw = active * hkw * bpt / (bits == 4 ? 7200.0 : 5500.0);   // ns per token
-    return rounds * (12.0 + ctx * 1e-3 * std::cbrt(k_cu * k_cu * k_cu + k_bw * k_bw * k_bw));
+    const double per_head_ns = pair ? (bits == 2 && hkw >= 4 ? pc.pair_wide2_ns : pc.pair_ns[w]) : pc.single_ns[w];
+    const double k_cu = hkw * per_head_ns, k_bw = active * hkw * bpt / pc.one_bw[w];   // ns per token
+    return rounds * (pc.one_fixed_us + ctx * 1e-3 * std::cbrt(k_cu * k_cu * k_cu + k_bw * k_bw * k_bw));
+}
+
+// Three launches (rotation, scan, merge) for the same step: their fixed cost and the scan at its rate.
+double decode_three_estimate_us(int G, int Hk, int bits, double ctx) {
+    const PlanConstants& pc = plan_constants();
+    const int w = bits == 4 ? 0 : 1;
+    const double bpt = bits == 4 ? 132.0 : 68.0;
+    return pc.three_fixed_us[w] + (double)G * Hk * bpt * ctx / pc.three_bw[w];
 }
 
 // KV heads per workgroup (8, 4, 2 or 1): the choice with the smallest estimate at a context of 4096 tokens (the order
@@ -888,11 +922,9 @@ int decode_fused_heads_per_workgroup(int G, int num_heads, int Hk, int bits, boo
 }
 
 // With shares: a launch of G * (Hk / hkw) * shares workgroups, each with 1 / shares of the context, plus what the
-// hand-over costs at the end (measured on MI355X with a probe in which all 512 workgroups of a streaming launch take
-// part: 3.7, 5.4 and 8.7 us for 2, 4 and 8 shares).  Shares are only taken while all workgroups fit the compute units
-// in one round and a share still has a tile for every wave.
+// hand-over costs at the end (plan_constants).  Shares are only taken while all workgroups fit the compute units in
+// one round and a share still has a tile for every wave.
 namespace {
-constexpr double kShareHandoverUs[4] = {0.0, 3.7, 5.4, 8.7};       // by log2(shares)
 std::atomic<int> g_force_hkw{0}, g_force_shares{0};
 }  // namespace
 void decode_fused_force_shape(int hkw, int shares) { g_force_hkw.store(hkw); g_force_shares.store(shares); }
@@ -913,7 +945,7 @@ FusedShape decode_fused_shape(int G, int num_heads, int Hk, int bits, bool allow
                 if (ctx < 32.0 * parts * sh) continue;
                 // every share is a launch of its own size: G * shares "sequences" of ctx / shares tokens
                 const double us = decode_fused_estimate_us(G * sh, num_heads, Hk, bits, allow_pairs, c, ctx / sh) +
-                                  kShareHandoverUs[lg];
+                                  plan_constants().handover_us[lg];
                 if (us < best.us) best = FusedShape{c, sh, us};
             }
         }

@@ -210,10 +210,28 @@ struct FusedArgs {
     const half_t* sin_table;
     int rope_dim;            // 128, or a multiple of 16 up to 64
 };
+// Everything the choice between the forms of a decode step rests on, in one place: rates and fixed costs measured on
+// the device named, looked up once per process by the current device's name (plan_constants()).  A device that is
+// not in the table gets the first entry's figures scaled by its own number of compute units only where the estimates
+// use that number; tests/test_gpu_plan.py checks on the GPU at hand that the automatic choice is the faster form.
+struct PlanConstants {
+    const char* device;         // substring of hipDeviceProp_t::gcnArchName
+    double one_fixed_us;        // one launch: prologue, first tile, epilogue, launch and drain
+    double pair_ns[2];          // ns per token and KV head one compute unit sustains, waves with two heads: [4 bit, 2 bit]
+    double pair_wide2_ns;       // the same at 2 bit with four or more heads per workgroup
+    double single_ns[2];        // waves with one head each
+    double one_bw[2];           // bytes per us the whole chip streams in the one-launch pattern
+    double three_fixed_us[2];   // three launches: rotation, merge, launches and the scan's start and end
+    double three_bw[2];         // bytes per us of the scan
+    double handover_us[4];      // shares' sums through memory, by log2(shares)
+};
+const PlanConstants& plan_constants();
 bool decode_fused_usable(const AttnArgs& a, const FusedArgs& f);
 int decode_fused_heads_per_workgroup(int G, int num_heads, int num_kv_heads, int bits, bool allow_pairs);   // 8, 4, 2 or 1
 // estimated microseconds of one launch with hkw KV heads per workgroup, all sequences at ctx tokens
 double decode_fused_estimate_us(int G, int num_heads, int num_kv_heads, int bits, bool allow_pairs, int hkw, double ctx);
+// estimated microseconds of the same step as three launches (rotation, scan, merge)
+double decode_three_estimate_us(int G, int num_kv_heads, int bits, double ctx);
 // The launch's shape when a unit's context may be shared by up to max_shares workgroups (1: the caller has no tickets
 // or no room for the shares' sums): KV heads per workgroup, shares, and the estimate for sequences of ctx tokens.
 struct FusedShape { int hkw, shares; double us; };
