@@ -37,8 +37,10 @@ namespace twkv {
 namespace {
 
 constexpr int kPfWaves = 4;
-constexpr int kPfKRow = 2 * kHeadDim + 16;   // bytes per K row in LDS
-constexpr int kPfVRow = 2 * 32 + 16;         // bytes per V^T row (32 token slots) in LDS
+constexpr int kPfKRow = 2 * kHeadDim + 32;   // bytes per K row in LDS: with 288 the operand reads (16 rows x 4 column groups of 16 bytes) run at the LDS's full rate, with 272 at 53 % of it (measured)
+constexpr int kPfVRow = 2 * 32 + 32;         // bytes per V^T row (32 token slots) in LDS: 96 at the full rate, 80 at 54 %
+
+template <bool B> struct Flag { static constexpr bool value = B; };
 
 // column of a tile's token in the V^T rows: the contraction slot order of the second MFMA
 __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 2) + 4 * (token >> 4) + (token & 3); }
@@ -52,13 +54,26 @@ __global__ void __launch_bounds__(kPfWaves* kWave, 2)        // two workgroups p
 prefill_f16_mfma_kernel(AttnArgs a, int T) {
     constexpr int TPW = 16 * NQ * kPfWaves / R;            // query tokens per workgroup pass
     __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPfKRow];
-    __shared__ __attribute__((aligned(16))) char v_s[3][kHeadDim * kPfVRow];
+    __shared__ __attribute__((aligned(16))) char v_s[4][kHeadDim * kPfVRow];
 
     const int tid = threadIdx.x;
     const int wave = uniform(tid / kWave), lane = tid % kWave;
     const int ln = lane & 15, kg = lane >> 4;
     const int nblk = (T + TPW - 1) / TPW;
-    const int kvh = blockIdx.y;
+    // Workgroups are dealt to the 8 XCDs in turn (linear id % 8), each with an L2 of its own.  The workgroups of a
+    // KV head all walk the same K and V rows, so a head's workgroups go to one XCD (8, 16, ... heads) or to 8 / heads
+    // of them (1, 2, 4 heads), and its rows are fetched from memory into one L2 instead of eight.
+    int blk = blockIdx.x, kvh = blockIdx.y;
+    {
+        const int nbx = gridDim.x, nh = gridDim.y;
+        const int lin = blockIdx.x + nbx * blockIdx.y, xcd = lin & 7, slot = lin >> 3;
+        if ((nh & 7) == 0) {
+            kvh = xcd + 8 * (slot / nbx); blk = slot % nbx;
+        } else if ((nh == 1 || nh == 2 || nh == 4) && nbx % (8 / nh) == 0) {
+            const int per = 8 / nh;                      // XCDs per head
+            kvh = xcd % nh; blk = slot * per + xcd / nh;
+        }
+    }
     const int head = kvh * R + wave % R;
     const int kv_dim = a.num_kv_heads * kHeadDim;
     const half_t* kbase = reinterpret_cast<const half_t*>(a.k) + (long long)kvh * kHeadDim;
@@ -107,7 +122,7 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
 
     // A workgroup takes token block blockIdx.x and its mirror image from the other end, one after the
     // other: with causal rows the two together cost the same for every workgroup.
-    const int first = blockIdx.x, second = nblk - 1 - (int)blockIdx.x;   // without MIRROR: longest blocks first
+    const int first = blk, second = nblk - 1 - blk;   // without MIRROR: longest blocks first
     for (int pass = 0; pass < (MIRROR ? 2 : 1); pass++) {
         if (pass == 1 && second == first) break;           // the middle block of an odd count
         const int tb = pass == 0 ? second : first;         // the long one first
@@ -132,36 +147,56 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
             for (int j = 0; j < 8; j++) o[nq][j] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
 
-        // ---- O[query][dim 16j + ln] += P . V for one tile
-        auto pv = [&](int vbuf, const half8_t (&pa)[NQ]) {
-            const char* vrow = &v_s[vbuf][ln * kPfVRow + 16 * kg];
+        // ---- operand reads of a tile from LDS: K rows for the score MFMAs, V^T rows for the P.V MFMAs
+        auto read_k = [&](int kbuf, half8_t (&kf)[8]) {
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const half8_t vb = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
+            for (int sub = 0; sub < 2; sub++) {
+                const char* krow = &k_s[kbuf][(16 * sub + ln) * kPfKRow + 16 * kg];
 #pragma unroll
-                for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vb, o[nq][j], 0, 0, 0);
+                for (int j = 0; j < 4; j++) kf[4 * sub + j] = *reinterpret_cast<const half8_t*>(krow + 64 * j);
             }
         };
+        auto read_v = [&](int vbuf, half8_t (&vf)[8]) {
+            const char* vrow = &v_s[vbuf][ln * kPfVRow + 16 * kg];
+#pragma unroll
+            for (int j = 0; j < 8; j++) vf[j] = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
+        };
 
-        // The loop is skewed by one tile: iteration t computes the scores of tile t, then the P.V product of
-        // tile t - 1 (whose MFMAs do not depend on anything of tile t and run under the softmax arithmetic of
-        // tile t), then the softmax of tile t.  So V tiles live one iteration longer than K tiles: three
-        // V buffers, two K buffers.
+        // The loop is a pipeline over tiles, one barrier per tile.  Iteration `it`
+        //   hands tile it + 2 to LDS (its global loads were issued an iteration ago) and asks for tile it + 3,
+        //   reads the V^T operands of tile it - 1,
+        //   issues the score MFMAs of tile it on K operands that the previous iteration read into registers,
+        //   reads the K operands of tile it + 1 (in LDS since the previous barrier),
+        //   scales the scores and checks the running maxima,
+        //   then issues the P.V MFMAs of tile it - 1 with the exponentials of tile it between them.
+        // So no MFMA waits for an LDS read issued just before it, and the matrix cores work under the vector
+        // arithmetic of the softmax.  Tiles live in LDS from two iterations before their scores to one after:
+        // two K buffers, four V buffers.  The tiles up to a wave's diagonal (no masks, every wave busy) take a
+        // straight-line form of the step; the first tile and those on the diagonal the general one.
         __syncthreads();                                   // a previous pass may still be reading its last V tile
         uint4 kr[2], vr[2];
         load_tile(0, kr, vr);
         stash(0, 0, kr, vr);
+        if (ntiles > 1) { load_tile(32, kr, vr); stash(1, 1, kr, vr); }
+        if (ntiles > 2) load_tile(64, kr, vr);
         __syncthreads();
+        half8_t kf[8];
+        read_k(0, kf);
+        __syncthreads();                                   // the first step overwrites the K buffer just read
 
         half8_t pa_prev[NQ];
         bool have_prev = false;
-        for (int it = 0; it < ntiles; it++) {
-            const int buf = it & 1;
-            const int tile = 32 * it;
-            const bool more = it + 1 < ntiles;
-            if (more) load_tile(tile + 32, kr, vr);
+        const int n_steady = q0 < T ? min((q0 + 1) >> 5, ntiles - 2) : 0;   // tiles wholly below this wave's diagonal
 
-            const bool active = tile <= q0 + 16 * NQ - 1 && q0 < T;      // the tile reaches this wave's queries (uniform over the wave)
+        auto step = [&](auto steady_c, int it) {
+            constexpr bool STEADY = decltype(steady_c)::value;
+            const int tile = 32 * it;
+            if (STEADY || it + 2 < ntiles) stash(it & 1, (it + 2) & 3, kr, vr);
+            if (STEADY || it + 3 < ntiles) load_tile(tile + 96, kr, vr);    // STEADY: rows past the cache read as zeros
+            const bool active = STEADY || (tile <= q0 + 16 * NQ - 1 && q0 < T);  // the tile reaches this wave's queries
+            const bool prev = STEADY || have_prev;
+            half8_t vf[8];
+            if (prev) read_v((it + 3) & 3, vf);            // tile it - 1
             float4_t s[NQ][2];
             if (active) {
                 // ---- S^T[kv][query] for both 16-token halves and all query blocks
@@ -169,41 +204,38 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                 for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
                     for (int nq = 0; nq < NQ; nq++) s[nq][sub] = float4_t{0.f, 0.f, 0.f, 0.f};
-                    const char* krow = &k_s[buf][(16 * sub + ln) * kPfKRow + 16 * kg];
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        const half8_t ka = *reinterpret_cast<const half8_t*>(krow + 64 * j);
 #pragma unroll
                         for (int nq = 0; nq < NQ; nq++)
-                            s[nq][sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[nq][j], s[nq][sub], 0, 0, 0);
+                            s[nq][sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[4 * sub + j], qb[nq][j], s[nq][sub], 0, 0, 0);
                     }
                 }
             }
-            if (have_prev) pv((it + 2) % 3, pa_prev);      // tile it - 1 sits in V buffer (it - 1) % 3
-            have_prev = active;
+            if (STEADY || it + 1 < ntiles) read_k((it + 1) & 1, kf);
+            float x[NQ][8];
             if (active) {
-                // ---- online softmax per query: this lane holds kv tokens tile + 16 sub + 4kg + i
+                // ---- online softmax per query, first half: this lane holds kv tokens tile + 16 sub + 4kg + i
 #pragma unroll
                 for (int nq = 0; nq < NQ; nq++) {
                     const int tq = q0 + 16 * nq + ln;
-                    float x[8];
 #pragma unroll
                     for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++) x[4 * sub + i] = s[nq][sub][i] * scale2;
+                        for (int i = 0; i < 4; i++) x[nq][4 * sub + i] = s[nq][sub][i] * scale2;
                     }
-                    if (tile + 31 > q0 + 16 * nq) {        // the tile crosses this block's diagonal (uniform over the wave)
+                    if (!STEADY && tile + 31 > q0 + 16 * nq) {   // the tile crosses this block's diagonal (uniform over the wave)
 #pragma unroll
                         for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
                             for (int i = 0; i < 4; i++) {
-                                if (tile + 16 * sub + 4 * kg + i > tq) x[4 * sub + i] = kNegBig;
+                                if (tile + 16 * sub + 4 * kg + i > tq) x[nq][4 * sub + i] = kNegBig;
                             }
                         }
                     }
-                    float mx = x[0];
+                    float mx = x[nq][0];
 #pragma unroll
-                    for (int i = 1; i < 8; i++) mx = fmaxf(mx, x[i]);
+                    for (int i = 1; i < 8; i++) mx = fmaxf(mx, x[nq][i]);
                     if (__any(mx > m_run[nq] + kRaise)) {  // rare after the first tiles
                         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
@@ -211,6 +243,11 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                         const float alpha = __builtin_amdgcn_exp2f(m_run[nq] - m_new);
                         m_run[nq] = m_new;
                         l_run[nq] *= alpha;
+                        // the product of the previous tile is not in the accumulators yet: its P shrinks with them
+                        if (prev) {
+#pragma unroll
+                            for (int i = 0; i < 8; i++) pa_prev[nq][i] = (half_t)((float)pa_prev[nq][i] * alpha);
+                        }
 #pragma unroll
                         for (int i = 0; i < 4; i++) {      // accumulator register i belongs to query 4kg + i
                             const float ai = __shfl(alpha, 4 * kg + i, 64);
@@ -218,19 +255,47 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                             for (int j = 0; j < 8; j++) o[nq][j][i] *= ai;
                         }
                     }
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        const float p = __builtin_amdgcn_exp2f(x[i] - m_run[nq]);
-                        l_run[nq] += p;
-                        pa_prev[nq][i] = (half_t)p;
-                    }
                 }
             }
-
-            if (more) stash(buf ^ 1, (it + 1) % 3, kr, vr);
+            // ---- O[query][dim 16j + ln] += P . V of tile it - 1, and the exponentials of tile it
+            if (prev) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+#pragma unroll
+                    for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_prev[nq], vf[j], o[nq][j], 0, 0, 0);
+                }
+            }
+            if (active) {
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) {
+                    half8_t pn;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float p = __builtin_amdgcn_exp2f(x[nq][i] - m_run[nq]);
+                        l_run[nq] += p;
+                        pn[i] = (half_t)p;
+                    }
+                    pa_prev[nq] = pn;
+                }
+            }
+            have_prev = active;
             __syncthreads();
+        };
+        step(Flag<false>{}, 0);
+        int it = 1;
+#pragma clang loop unroll(disable)
+        for (; it < n_steady; it++) step(Flag<true>{}, it);
+#pragma clang loop unroll(disable)
+        for (; it < ntiles; it++) step(Flag<false>{}, it);
+        if (have_prev) {
+            half8_t vf[8];
+            read_v((ntiles - 1) & 3, vf);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_prev[nq], vf[j], o[nq][j], 0, 0, 0);
+            }
         }
-        if (have_prev) pv((ntiles - 1) % 3, pa_prev);
 
         // ---- normalise (kernels.cu:1146: 1 / (sum + 1e-8)) and store; accumulator register i is query 4kg + i
 #pragma unroll
