@@ -20,12 +20,13 @@
 // query head w % R and 16 NQ tokens; with NQ = 2 the two 16-row blocks share every operand read),
 // walks the kv tiles of 32 tokens up to its diagonal and shares each tile through LDS: K row-major
 // (padded rows), V transposed on the way in (each thread interleaves the same 8 dims of two
-// consecutive tokens and writes 8 dwords).  The next tile's global loads are issued before the
-// arithmetic and stored to LDS after it, one barrier per tile; the P.V product of a tile runs one
-// iteration late, under the softmax arithmetic of the next tile (three V buffers, two K buffers).  For long
-// prompts a workgroup does a token block and then its mirror image from the other end of the
-// sequence, so causal rows cost every workgroup the same; short prompts take one block each, longest
-// first.
+// consecutive tokens and writes 8 dwords).  The loop is a pipeline, one barrier per tile, a tile
+// taking five steps through it: global loads issued; written to LDS; K operands read into registers; score
+// MFMAs (with the previous tile's exponentials between them) and maxima; exponentials and P.V MFMAs (with the
+// next tile's maxima between them).  Two K buffers, four V buffers; the loop says which step does what.  For long prompts a workgroup does a token block and then its
+// mirror image from the other end of the sequence, so causal rows cost every workgroup the same; short
+// prompts take one block each, longest first.  The workgroups of a KV head run on one XCD, so the head's
+// rows come out of one L2.
 
 #include "kv_common.hpp"
 #include "kv_kernels.hpp"
@@ -162,17 +163,17 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
             for (int j = 0; j < 8; j++) vf[j] = *reinterpret_cast<const half8_t*>(vrow + 16 * j * kPfVRow);
         };
 
-        // The loop is a pipeline over tiles, one barrier per tile.  Iteration `it`
-        //   hands tile it + 2 to LDS (its global loads were issued an iteration ago) and asks for tile it + 3,
-        //   reads the V^T operands of tile it - 1,
-        //   issues the score MFMAs of tile it on K operands that the previous iteration read into registers,
-        //   reads the K operands of tile it + 1 (in LDS since the previous barrier),
-        //   scales the scores and checks the running maxima,
-        //   then issues the P.V MFMAs of tile it - 1 with the exponentials of tile it between them.
-        // So no MFMA waits for an LDS read issued just before it, and the matrix cores work under the vector
-        // arithmetic of the softmax.  Tiles live in LDS from two iterations before their scores to one after:
-        // two K buffers, four V buffers.  The tiles up to a wave's diagonal (no masks, every wave busy) take a
-        // straight-line form of the step; the first tile and those on the diagonal the general one.
+        // The loop is a pipeline over tiles, one barrier per tile, in two phases that each pair 16 MFMAs with
+        // vector arithmetic that does not depend on them.  Step t
+        //   phase 1: score MFMAs of tile t + 1 (K operands read into registers by step t - 1)
+        //            with the exponentials of tile t (scores from step t - 1) between them; V^T operands of tile t read;
+        //   phase 2: P.V MFMAs of tile t with the maxima of tile t + 1 between them (and, rarely, a rescale after them);
+        //            K operands of tile t + 2 read; tile t + 3 handed to LDS (its global loads were issued a step
+        //            ago) and tile t + 4 asked for.
+        // So no MFMA waits for an LDS read issued just before it, and a wave keeps the matrix cores and the
+        // vector ALU busy at once.  Tiles live in LDS from three steps before their P.V product: two K buffers,
+        // four V buffers.  Steps whose two tiles lie wholly below the wave's diagonal take a straight-line form;
+        // the filling step t = -1 and those on the diagonal the general one.
         __syncthreads();                                   // a previous pass may still be reading its last V tile
         uint4 kr[2], vr[2];
         load_tile(0, kr, vr);
@@ -184,22 +185,21 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
         read_k(0, kf);
         __syncthreads();                                   // the first step overwrites the K buffer just read
 
-        half8_t pa_prev[NQ];
-        bool have_prev = false;
-        const int n_steady = q0 < T ? min((q0 + 1) >> 5, ntiles - 2) : 0;   // tiles wholly below this wave's diagonal
+        float x[NQ][8];                                    // raw scores of the tile whose exponentials come next
+        bool have_x = false;
+        const int n_below = q0 < T ? (q0 + 1) >> 5 : 0;    // tiles wholly below this wave's diagonal
 
-        auto step = [&](auto steady_c, int it) {
+        auto step = [&](auto steady_c, int t) {
             constexpr bool STEADY = decltype(steady_c)::value;
-            const int tile = 32 * it;
-            if (STEADY || it + 2 < ntiles) stash(it & 1, (it + 2) & 3, kr, vr);
-            if (STEADY || it + 3 < ntiles) load_tile(tile + 96, kr, vr);    // STEADY: rows past the cache read as zeros
-            const bool active = STEADY || (tile <= q0 + 16 * NQ - 1 && q0 < T);  // the tile reaches this wave's queries
-            const bool prev = STEADY || have_prev;
+            const int tile1 = 32 * (t + 1);                // first token of tile t + 1
+            const bool do_s = STEADY || (t + 1 < ntiles && tile1 <= q0 + 16 * NQ - 1 && q0 < T);   // tile t + 1 reaches this wave's queries
+            const bool do_p = STEADY || have_x;
+            // ---- phase 1
             half8_t vf[8];
-            if (prev) read_v((it + 3) & 3, vf);            // tile it - 1
+            if (do_p) read_v(t & 3, vf);
             float4_t s[NQ][2];
-            if (active) {
-                // ---- S^T[kv][query] for both 16-token halves and all query blocks
+            if (do_s) {
+                // S^T[kv][query] for both 16-token halves and all query blocks
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
@@ -212,30 +212,62 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                     }
                 }
             }
-            if (STEADY || it + 1 < ntiles) read_k((it + 1) & 1, kf);
-            float x[NQ][8];
-            if (active) {
-                // ---- online softmax per query, first half: this lane holds kv tokens tile + 16 sub + 4kg + i
+            half8_t pa[NQ];
+            if (do_p) {
+#pragma unroll
+                for (int nq = 0; nq < NQ; nq++) {
+                    half8_t pn;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) pn[i] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(x[nq][i], scale2, -m_run[nq]));
+                    // the sum runs over the rounded values the matrix cores will see, two per instruction
+                    const half2_t one2 = {(half_t)1.0f, (half_t)1.0f};
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        l_run[nq] = __builtin_amdgcn_fdot2(half2_t{pn[2 * i], pn[2 * i + 1]}, one2, l_run[nq], false);
+                    pa[nq] = pn;
+                }
+            }
+            if (STEADY) {
+#pragma unroll
+                for (int g = 0; g < 16; g++) {             // 16 MFMAs, 16 fma + 16 exp + 8 cvt + 8 dot2 between them
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                }
+            }
+            // ---- phase 2: O[query][dim 16j + ln] += P . V of tile t
+            if (do_p) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+#pragma unroll
+                    for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[nq], vf[j], o[nq][j], 0, 0, 0);
+                }
+            }
+            if (STEADY || t + 2 < ntiles) read_k(t & 1, kf);                           // tile t + 2
+            if (STEADY || t + 3 < ntiles) stash((t + 1) & 1, (t + 3) & 3, kr, vr);      // tile t + 3
+            if (STEADY || t + 4 < ntiles) load_tile(32 * (t + 4), kr, vr);              // STEADY: rows past the cache read as zeros
+            if (do_s) {
+                // maxima of tile t + 1 per query: this lane holds kv tokens tile1 + 16 sub + 4kg + i
 #pragma unroll
                 for (int nq = 0; nq < NQ; nq++) {
                     const int tq = q0 + 16 * nq + ln;
 #pragma unroll
                     for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++) x[nq][4 * sub + i] = s[nq][sub][i] * scale2;
+                        for (int i = 0; i < 4; i++) x[nq][4 * sub + i] = s[nq][sub][i];     // raw: the scale goes into the exponent's fma
                     }
-                    if (!STEADY && tile + 31 > q0 + 16 * nq) {   // the tile crosses this block's diagonal (uniform over the wave)
+                    if (!STEADY && tile1 + 31 > q0 + 16 * nq) {   // the tile crosses this block's diagonal (uniform over the wave)
 #pragma unroll
                         for (int sub = 0; sub < 2; sub++) {
 #pragma unroll
                             for (int i = 0; i < 4; i++) {
-                                if (tile + 16 * sub + 4 * kg + i > tq) x[nq][4 * sub + i] = kNegBig;
+                                if (tile1 + 16 * sub + 4 * kg + i > tq) x[nq][4 * sub + i] = kNegBig;
                             }
                         }
                     }
                     float mx = x[nq][0];
 #pragma unroll
                     for (int i = 1; i < 8; i++) mx = fmaxf(mx, x[nq][i]);
+                    mx *= scale2;
                     if (__any(mx > m_run[nq] + kRaise)) {  // rare after the first tiles
                         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));    // the query's maximum over the tile
@@ -243,11 +275,6 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                         const float alpha = __builtin_amdgcn_exp2f(m_run[nq] - m_new);
                         m_run[nq] = m_new;
                         l_run[nq] *= alpha;
-                        // the product of the previous tile is not in the accumulators yet: its P shrinks with them
-                        if (prev) {
-#pragma unroll
-                            for (int i = 0; i < 8; i++) pa_prev[nq][i] = (half_t)((float)pa_prev[nq][i] * alpha);
-                        }
 #pragma unroll
                         for (int i = 0; i < 4; i++) {      // accumulator register i belongs to query 4kg + i
                             const float ai = __shfl(alpha, 4 * kg + i, 64);
@@ -257,45 +284,16 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                     }
                 }
             }
-            // ---- O[query][dim 16j + ln] += P . V of tile it - 1, and the exponentials of tile it
-            if (prev) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-#pragma unroll
-                    for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_prev[nq], vf[j], o[nq][j], 0, 0, 0);
-                }
-            }
-            if (active) {
-#pragma unroll
-                for (int nq = 0; nq < NQ; nq++) {
-                    half8_t pn;
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        const float p = __builtin_amdgcn_exp2f(x[nq][i] - m_run[nq]);
-                        l_run[nq] += p;
-                        pn[i] = (half_t)p;
-                    }
-                    pa_prev[nq] = pn;
-                }
-            }
-            have_prev = active;
+            have_x = do_s;
             __syncthreads();
         };
-        step(Flag<false>{}, 0);
-        int it = 1;
+        step(Flag<false>{}, -1);
+        int t = 0;
+        const int n_steady = min(n_below - 1, ntiles - 3);      // steps with tiles t and t + 1 below the diagonal and tile t + 3 in range
 #pragma clang loop unroll(disable)
-        for (; it < n_steady; it++) step(Flag<true>{}, it);
+        for (; t < n_steady; t++) step(Flag<true>{}, t);
 #pragma clang loop unroll(disable)
-        for (; it < ntiles; it++) step(Flag<false>{}, it);
-        if (have_prev) {
-            half8_t vf[8];
-            read_v((ntiles - 1) & 3, vf);
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-#pragma unroll
-                for (int nq = 0; nq < NQ; nq++) o[nq][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_prev[nq], vf[j], o[nq][j], 0, 0, 0);
-            }
-        }
+        for (; t < ntiles; t++) step(Flag<false>{}, t);
 
         // ---- normalise (kernels.cu:1146: 1 / (sum + 1e-8)) and store; accumulator register i is query 4kg + i
 #pragma unroll

@@ -24,11 +24,11 @@ namespace twkv {
 namespace {
 
 constexpr int kPtWaves = 4;
-constexpr int kPtKRow = 2 * kHeadDim + 16;   // bytes per expanded K row in LDS
-constexpr int kPtVRow = 2 * 32 + 16;         // bytes per V^T row (32 token slots) in LDS
+constexpr int kPtKRow = 2 * kHeadDim + 32;   // bytes per expanded K row in LDS (288: operand reads at the LDS's full rate, 272: 53 % of it)
+constexpr int kPtVRow = 2 * 32 + 32;         // bytes per V^T row (32 token slots) in LDS (96: full rate, 80: 54 %)
 constexpr int kPtVTile = kHeadDim * kPtVRow; // bytes of a V^T tile
-constexpr int kPtVBytes = 2 * kHeadDim * kHeadDim;   // >= 3 tiles, and the 128 x 128 fp16 rotation
-static_assert(kPtVBytes >= 3 * kPtVTile, "three V tiles fit");
+constexpr int kPtVBytes = 3 * kPtVTile;      // 3 tiles, and room for the 128 x 128 fp16 rotation
+static_assert(kPtVBytes >= 2 * kHeadDim * kHeadDim, "the rotation fits");
 
 // column of a tile's token in the V^T rows: the contraction slot order of the second MFMA
 __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 2) + 4 * (token >> 4) + (token & 3); }
@@ -55,7 +55,20 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
     const int wave = uniform(tid / kWave), lane = tid % kWave;
     const int ln = lane & 15, kg = lane >> 4;
     const int nblk = (T + TPW - 1) / TPW;
-    const int kvh = blockIdx.y;
+    // Workgroups are dealt to the 8 XCDs in turn (linear id % 8), each with an L2 of its own.  The workgroups of a
+    // KV head all walk the same rows, so a head's workgroups go to one XCD (8, 16, ... heads) or to 8 / heads of
+    // them (1, 2, 4 heads), and its rows are fetched from memory into one L2 instead of eight.
+    int blk = blockIdx.x, kvh = blockIdx.y;
+    {
+        const int nbx = gridDim.x, nh = gridDim.y;
+        const int lin = blockIdx.x + nbx * blockIdx.y, xcd = lin & 7, slot = lin >> 3;
+        if ((nh & 7) == 0) {
+            kvh = xcd + 8 * (slot / nbx); blk = slot % nbx;
+        } else if ((nh == 1 || nh == 2 || nh == 4) && nbx % (8 / nh) == 0) {
+            const int per = 8 / nh;                      // XCDs per head
+            kvh = xcd % nh; blk = slot * per + xcd / nh;
+        }
+    }
     const int head = kvh * R + wave % R;
     const int row_bytes = a.num_kv_heads * kHeadBytes;
     const char* kbase = reinterpret_cast<const char*>(a.k) + kvh * kHeadBytes;
@@ -149,7 +162,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
 
     // A workgroup takes token block blockIdx.x and its mirror image from the other end, one after the
     // other: with causal rows the two together cost the same for every workgroup.
-    const int first = blockIdx.x, second = nblk - 1 - (int)blockIdx.x;   // without MIRROR: longest blocks first
+    const int first = blk, second = nblk - 1 - blk;   // without MIRROR: longest blocks first
     for (int pass = 0; pass < (MIRROR ? 2 : 1); pass++) {
         if (pass == 1 && second == first) break;           // the middle block of an odd count
         const int tb = pass == 0 ? second : first;         // the long one first
@@ -224,8 +237,10 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
             }
         };
 
-        // The loop is skewed by one tile as in the fp16 kernel: scores of tile t, then the P.V product of tile
-        // t - 1 under the softmax arithmetic of tile t.  Three V (and norm) buffers, two K buffers.
+        // The loop is skewed by one tile: scores of tile t, then the P.V product of tile t - 1 (whose MFMAs do not
+        // depend on tile t) ahead of the softmax arithmetic of tile t.  Three V (and norm) buffers, two K buffers.
+        // (The fp16 kernel's deeper pipeline -- K operands a tile ahead in registers -- needs 64 registers more
+        // than the 226 this kernel already uses with its second set of operands.)
         __syncthreads();                                   // a previous pass may still be reading its last V tile
         Staged st;
         load_tile(0, st);
