@@ -742,6 +742,41 @@ def test_turbo_prefill_every_form(kv, oracle, rotation_fixture, bits, H, Hk, T, 
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("form", [1, 3])
+@pytest.mark.parametrize("Hk,R,T", [(1, 2, 290), (2, 1, 97), (2, 2, 418), (3, 1, 150), (4, 2, 163), (6, 2, 130), (16, 1, 200), (24, 1, 70)])
+@pytest.mark.parametrize("bits", [0, 4])
+def test_prefill_workgroup_placement_covers_every_block(kv, oracle, rotation_fixture, bits, Hk, R, T, form):
+    """The prompt kernels place the workgroups of a KV head on one XCD (8, 16, 24 heads), on 8 / heads of them
+    (1, 2, 4 heads, when the block count divides) or leave the grid as it is (3, 6 heads, odd block counts):
+    whatever the branch, every (token block, head) is computed exactly once -- the output equals the oracle's
+    for head counts and block counts that take each branch, with and without mirrored block pairs."""
+    import torch
+    H = Hk * R
+    r = gen.rng(900 + 31 * Hk + T + bits)
+    msl = T + 2
+    kv_dim, q_dim = Hk * D, H * D
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * max(T, 1024), dtype=torch.float32, device="cuda")
+    kv.set_prefill_form(form)
+    try:
+        if bits:
+            ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, 1, Hk, msl, [T], bits)
+            oracle.turbo_gqa_prefill_attention(want, q, ck[0], cv[0], kn[0], vn[0], rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+            kv.launch_turbo_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), dev(kn[0]), dev(vn[0]),
+                                                  dev(rotation_fixture), scratch, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+        else:
+            ck, cv = build_fp16_cache(r, 1, msl, kv_dim)
+            oracle.gqa_prefill_attention(want, q, ck[0], cv[0], T, msl, H, Hk, D, q_dim, kv_dim)
+            kv.launch_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), scratch, T, msl, H, Hk, D, q_dim, kv_dim)
+    finally:
+        kv.set_prefill_form(0)
+    got = host(out)
+    assert np.abs(got.astype(np.float32)).sum(axis=1).min() > 0, "a token block was left out"
+    assert rel_err(got, want) <= TOL
+
+
 @pytest.mark.parametrize("bits,H,Hk,T,pad", [(4, 16, 8, 333, 64), (2, 8, 4, 200, 8), (4, 8, 4, 150, 4), (2, 4, 4, 95, 1024)])
 def test_turbo_prefill_strided_rows_scratch_untouched(kv, oracle, rotation_fixture, bits, H, Hk, T, pad):
     """Compressed prefill with rows of q and out wider than the heads (q_dim = H * 128 + pad; a pad of 4 halves
