@@ -176,6 +176,7 @@ def prefill_bench(args):
     kv_bits = w["kv_bits"] if args.kv_bits is None else args.kv_bits
     H, Hk, D, T = w["H"], w["Hk"], 128, args.prefill
     kvcache.set_attention_variant(args.variant)
+    kvcache.set_prefill_form(args.prefill_form)
     g = torch.Generator(device="cuda"); g.manual_seed(11)
     q = torch.randn((T, H * D), generator=g, device="cuda", dtype=torch.float16)
     out = torch.zeros_like(q)
@@ -242,7 +243,7 @@ def prefill_bench(args):
         "steps": args.steps, "warmup": max(args.warmup, 1), "ms_per_step": ms, "higher_is_better": True,
         "dtype": "f16-operand MFMA, f32 accumulate" if not kv_bits else DTYPE[kv_bits], "data": "synthetic",
         "config": {"workload": f"causal prefill attention, one sequence, {T} tokens, {H} heads over {Hk} KV heads",
-                   "kv_bits": kv_bits if kv_bits else 16, "variant": args.variant,
+                   "kv_bits": kv_bits if kv_bits else 16, "variant": args.variant, "form": args.prefill_form,
                    "timed": ["the attention launch", "tw_layer_prompt_step: producers + T-token append + attention (+ 2 copies restoring q and k)",
                              "launch_qk_norm_batch, launch_rope_batch, 2 appends, the attention launch (+ 2 copies restoring q and k)"][args.prompt_step]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s", "frac": tflops / 2500.0,
@@ -423,6 +424,8 @@ def main():
     ap.add_argument("--per-config", action="store_true",
                     help="also measure the BASELINE configs 1-5 (and the reference's launchers at the target shape) with "
                          "few steps each and report them under per_config; the default run does this")
+    ap.add_argument("--prefill-form", type=int, default=0,
+                    help="with --prefill: force a form of the prompt kernel (tw_kv_debug_set_prefill_form; 0 = automatic)")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="instead of the decode step, time causal prefill attention over a T-token prompt of one "
                          "sequence (one layer's launch, the workload's head counts, --kv-bits cache) and exit")

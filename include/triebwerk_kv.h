@@ -169,7 +169,8 @@ int tw_kv_debug_get_attention_variant(void);
 void tw_kv_debug_set_num_splits(int nsplit);
 /* Form of the matrix-core prefill kernels: 0 = chosen from the prompt length, 1 = one 16-row query block per wave,
  * 2 = the same with mirrored block pairs, 3 = two query blocks per wave with mirrored pairs, 4 = compressed cache
- * only: the kernel that expands tiles per wave. */
+ * only: the kernel that expands tiles per wave, 5 and 6 = forms 2 and 3 with eight waves per
+ * workgroup instead of four. */
 void tw_kv_debug_set_prefill_form(int form);
 /* tw_turbo_append_attention_batch and the calls built on it can run a layer's decode step as ONE kernel (append,
  * query rotation, scan, merge, rotate-back; a workgroup owns a sequence's heads) instead of three.  0 (default):

@@ -428,12 +428,13 @@ def test_fp16_prefill_attention_long(kv, oracle, H, Hk, T, pad, variant):
     assert not got[:, H * D:].any()
 
 
-@pytest.mark.parametrize("form", [1, 2, 3])
-@pytest.mark.parametrize("H,Hk,T", [(16, 8, 300), (8, 8, 129), (16, 4, 97), (16, 8, 31)])
+@pytest.mark.parametrize("form", [1, 2, 3, 5, 6])
+@pytest.mark.parametrize("H,Hk,T", [(16, 8, 300), (8, 8, 129), (16, 4, 97), (16, 8, 31), (16, 4, 777)])
 def test_fp16_prefill_every_form_of_the_mfma_kernel(kv, oracle, H, Hk, T, form):
-    """The matrix-core prefill kernel picks one of three forms from the prompt length (one or two query
-    blocks per wave, with or without mirrored block pairs); each is forced here at lengths that put
-    the diagonal, the middle block of an odd count and a ragged last block in different places."""
+    """The matrix-core prefill kernel picks one of five forms from the prompt length (one or two query
+    blocks per wave, with or without mirrored block pairs, four or eight waves per workgroup); each is forced
+    here at lengths that put the diagonal, the middle block of an odd count and a ragged last block in
+    different places."""
     import torch
     r = gen.rng(270 + H + T)
     msl = T
@@ -716,11 +717,12 @@ def test_turbo_prefill_attention_long(kv, oracle, rotation_fixture, bits, H, Hk,
     kv.set_attention_variant(0)
 
 
-@pytest.mark.parametrize("form", [1, 2, 3, 4])
+@pytest.mark.parametrize("form", [1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("bits,H,Hk,T", [(4, 16, 8, 300), (2, 8, 8, 129), (4, 16, 4, 97), (2, 16, 8, 31), (4, 8, 4, 1),
-                                         (2, 4, 4, 7), (4, 4, 1, 16), (2, 8, 4, 33)])
+                                         (2, 4, 4, 7), (4, 4, 1, 16), (2, 8, 4, 33), (2, 16, 4, 777), (4, 8, 4, 515)])
 def test_turbo_prefill_every_form(kv, oracle, rotation_fixture, bits, H, Hk, T, form):
-    """Compressed prefill: the three forms of the kernel that expands a tile once per workgroup and (form 4)
+    """Compressed prefill: the five forms of the kernel that expands a tile once per workgroup (four or eight
+    waves per workgroup, one or two query blocks per wave, with or without mirrored block pairs) and (form 4)
     the kernel that expands per wave, each against the oracle."""
     import torch
     r = gen.rng(380 + bits + H + T)
@@ -742,7 +744,7 @@ def test_turbo_prefill_every_form(kv, oracle, rotation_fixture, bits, H, Hk, T, 
     assert err <= TOL, err
 
 
-@pytest.mark.parametrize("form", [1, 3])
+@pytest.mark.parametrize("form", [1, 3, 6])
 @pytest.mark.parametrize("Hk,R,T", [(1, 2, 290), (2, 1, 97), (2, 2, 418), (3, 1, 150), (4, 2, 163), (6, 2, 130), (16, 1, 200), (24, 1, 70)])
 @pytest.mark.parametrize("bits", [0, 4])
 def test_prefill_workgroup_placement_covers_every_block(kv, oracle, rotation_fixture, bits, Hk, R, T, form):

@@ -246,13 +246,13 @@ void launch_prefill_mfma_scan(const AttnArgs& a, hipStream_t s);
 // causal prefill over the fp16 cache on the matrix cores (kv_prefill_f16_mfma.hip); writes `out` directly
 bool prefill_f16_mfma_usable(const AttnArgs& a);
 // form: 0 = chosen from the prompt length; 1 one query block per wave, 2 the same with mirrored block pairs,
-// 3 two query blocks per wave with mirrored pairs
+// 3 two query blocks per wave with mirrored pairs (1-3: four waves per workgroup); 5 and 6 = 2 and 3 with eight waves
 void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form);
 // causal prefill over the compressed cache with tiles expanded once per workgroup (kv_prefill_tq_mfma.hip);
-// same workspace and merge as the scan; form as for launch_prefill_f16_mfma
+// one launch, no workspace; forms as for launch_prefill_f16_mfma
 bool prefill_tq_mfma_usable(const AttnArgs& a);
 void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form);
-// test hook (tw_kv_debug_set_prefill_form): 0 = automatic; 1-3 force a form of the flash prefill kernels; 4 = the
+// test hook (tw_kv_debug_set_prefill_form): 0 = automatic; 1-3, 5, 6 force a form of the flash prefill kernels; 4 = the
 // compressed prefill kernel that expands tiles per wave
 int prefill_form();
 // 4-bit decode scan whose waves take two KV heads each and read whole cache lines (kv_attention_pair.hip); same

@@ -37,7 +37,6 @@ namespace twkv {
 
 namespace {
 
-constexpr int kPfWaves = 4;
 constexpr int kPfKRow = 2 * kHeadDim + 32;   // bytes per K row in LDS: with 288 the operand reads (16 rows x 4 column groups of 16 bytes) run at the LDS's full rate, with 272 at 53 % of it (measured)
 constexpr int kPfVRow = 2 * 32 + 32;         // bytes per V^T row (32 token slots) in LDS: 96 at the full rate, 80 at 54 %
 
@@ -50,10 +49,12 @@ __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 
 
 // NQ: 16-row query blocks per wave (every K and V operand read feeds NQ MFMAs).  MIRROR: a workgroup does a
 // token block and then its mirror image from the other end of the sequence.
-template <int R, int NQ, bool MIRROR>
-__global__ void __launch_bounds__(kPfWaves* kWave, 2)        // two workgroups per CU (three would spill)
+// W: waves per workgroup, 4 (two workgroups per CU) or 8 (one: a tile is brought into LDS once for twice the queries).
+template <int R, int NQ, bool MIRROR, int W>
+__global__ void __launch_bounds__(W* kWave, W == 4 ? 2 : 1)  // two waves per SIMD either way (three would spill)
 prefill_f16_mfma_kernel(AttnArgs a, int T) {
-    constexpr int TPW = 16 * NQ * kPfWaves / R;            // query tokens per workgroup pass
+    static_assert(W == 4 || W == 8, "the staging maps are written for 256 and 512 threads");
+    constexpr int TPW = 16 * NQ * W / R;                   // query tokens per workgroup pass
     __shared__ __attribute__((aligned(16))) char k_s[2][32 * kPfKRow];
     __shared__ __attribute__((aligned(16))) char v_s[4][kHeadDim * kPfVRow];
 
@@ -83,9 +84,9 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
     constexpr float kRaise = 5.0f;
 
     // ---- staging of a tile: thread (r = tid / 16, c = tid % 16) carries 16 bytes (dims 8c..8c+7) of
-    // K rows r and r + 16; for V, thread (c = tid / 16, r = tid % 16) carries dims 8c..8c+7 of rows 2r and
-    // 2r + 1 (two consecutive tokens, interleaved on the way into the transposed tile).  Rows past the
-    // last token are clamped (they are masked anyway).
+    // K rows r and r + 16 (512 threads: of row r alone); for V, thread (c = tid / 16, r = tid % 16) carries dims
+    // 8c..8c+7 (512 threads: 4c..4c+3) of rows 2r and 2r + 1 (two consecutive tokens, interleaved on the way into the
+    // transposed tile).
     const int sr = tid >> 4, sc = tid & 15;
     // V: 16 consecutive threads take the 16 token pairs of one dim octet, so that their dwords fill one V^T row
     // (64 contiguous bytes, all banks different); with the K mapping they would hit rows 8 apart, 8 to a bank
@@ -95,27 +96,34 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
     const __amdgpu_buffer_rsrc_t krs = make_rsrc(reinterpret_cast<const char*>(kbase), T * kv_dim * 2 - kvh * kHeadDim * 2);
     const __amdgpu_buffer_rsrc_t vrs = make_rsrc(reinterpret_cast<const char*>(vbase), T * kv_dim * 2 - kvh * kHeadDim * 2);
     const int koff0 = (sr * kv_dim + 8 * sc) * 2, koff1 = koff0 + 16 * kv_dim * 2;
-    const int voff0 = (2 * vr_ * kv_dim + 8 * vc_) * 2, voff1 = voff0 + kv_dim * 2;
+    const int voff0 = (2 * vr_ * kv_dim + (W == 4 ? 8 : 4) * vc_) * 2, voff1 = voff0 + kv_dim * 2;
     auto load_tile = [&](int tile, uint4 (&kr)[2], uint4 (&vr)[2]) {
         const int toff = tile * kv_dim * 2;
         const uint32x4_t k0 = __builtin_amdgcn_raw_buffer_load_b128(krs, koff0, toff, 0);
-        const uint32x4_t k1 = __builtin_amdgcn_raw_buffer_load_b128(krs, koff1, toff, 0);
-        const uint32x4_t v0 = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff0, toff, 0);
-        const uint32x4_t v1 = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff1, toff, 0);
         kr[0] = uint4{k0[0], k0[1], k0[2], k0[3]};
-        kr[1] = uint4{k1[0], k1[1], k1[2], k1[3]};
-        vr[0] = uint4{v0[0], v0[1], v0[2], v0[3]};
-        vr[1] = uint4{v1[0], v1[1], v1[2], v1[3]};
+        if constexpr (W == 4) {
+            const uint32x4_t k1 = __builtin_amdgcn_raw_buffer_load_b128(krs, koff1, toff, 0);
+            const uint32x4_t v0 = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff0, toff, 0);
+            const uint32x4_t v1 = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff1, toff, 0);
+            kr[1] = uint4{k1[0], k1[1], k1[2], k1[3]};
+            vr[0] = uint4{v0[0], v0[1], v0[2], v0[3]};
+            vr[1] = uint4{v1[0], v1[1], v1[2], v1[3]};
+        } else {
+            const uint32x2_t v0 = __builtin_amdgcn_raw_buffer_load_b64(vrs, voff0, toff, 0);
+            const uint32x2_t v1 = __builtin_amdgcn_raw_buffer_load_b64(vrs, voff1, toff, 0);
+            vr[0] = uint4{v0[0], v0[1], 0u, 0u};
+            vr[1] = uint4{v1[0], v1[1], 0u, 0u};
+        }
     };
     const int vcol = 2 * vt_slot(2 * vr_);                  // byte column of the token pair in a V^T row
     auto stash = [&](int buf, int vbuf, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
         *reinterpret_cast<uint4*>(&k_s[buf][sr * kPfKRow + 16 * sc]) = kr[0];
-        *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPfKRow + 16 * sc]) = kr[1];
+        if constexpr (W == 4) *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPfKRow + 16 * sc]) = kr[1];
         const uint32_t va[4] = {vr[0].x, vr[0].y, vr[0].z, vr[0].w};
         const uint32_t vb[4] = {vr[1].x, vr[1].y, vr[1].z, vr[1].w};
-        char* dst = &v_s[vbuf][(8 * vc_) * kPfVRow + vcol];
+        char* dst = &v_s[vbuf][((W == 4 ? 8 : 4) * vc_) * kPfVRow + vcol];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
+        for (int i = 0; i < (W == 4 ? 4 : 2); i++) {       // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves); 512 threads: 4c + ...
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPfVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
             *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kPfVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x07060302u);
         }
@@ -335,27 +343,31 @@ bool prefill_f16_mfma_usable(const AttnArgs& a) {
 void launch_prefill_f16_mfma(const AttnArgs& a, hipStream_t s, int form) {
     const int R = a.num_heads / a.num_kv_heads;
     const int T = a.G;
-    // Long prompts: two query blocks per wave and mirrored block pairs (operand reuse, equal work per
-    // workgroup).  Short ones do not fill the GPU that way and take smaller, then unpaired workgroups
-    // (measured at 16 and 32 heads over 8 KV heads: each form wins from one workgroup per CU upwards).
+    // Long prompts: eight waves per workgroup, two query blocks per wave and mirrored block pairs (a tile is brought
+    // into LDS once for 256 query rows, every operand read feeds two MFMAs, equal work per workgroup).  Shorter ones
+    // do not fill the GPU that way and take one query block per wave, then four waves, then unpaired workgroups.
+    // Measured with 16 heads over 8 KV heads: the eight-wave forms win from three workgroups per four CUs upwards
+    // (6144 tokens: 0.196 against 0.203 ms; 4096: 0.090 against 0.098; 3072: 0.065 against 0.072; at one per two CUs
+    // they lose, 2048 tokens: 0.047 against 0.038), the four-wave ones from one per CU.
     const int cus = compute_units();
+    auto pairs = [&](int waves, int nq) { const int tpw = 16 * nq * waves / R; return ((T + tpw - 1) / tpw + 1) / 2 * a.num_kv_heads; };
     int mode = 1;
-    {
-        const int nblk2 = (T + 32 * kPfWaves / R - 1) / (32 * kPfWaves / R), nblk1 = (T + 16 * kPfWaves / R - 1) / (16 * kPfWaves / R);
-        if ((nblk2 + 1) / 2 * a.num_kv_heads >= cus) mode = 3;
-        else if ((nblk1 + 1) / 2 * a.num_kv_heads >= cus) mode = 2;
-    }
-    if (form >= 1 && form <= 3) mode = form;               // forced by a test
-    const int nq = mode >= 3 ? 2 : 1;
-    const bool mirror = mode == 2 || mode == 3;
-    const int tpw = 16 * nq * kPfWaves / R;
+    if (4 * pairs(8, 2) >= 3 * cus) mode = 6;
+    else if (4 * pairs(8, 1) >= 3 * cus) mode = 5;
+    else if (pairs(4, 1) >= cus) mode = 2;
+    if ((form >= 1 && form <= 3) || form == 5 || form == 6) mode = form;    // forced by a test (4 is the compressed cache's other kernel)
+    const int waves = mode >= 5 ? 8 : 4;
+    const int nq = (mode == 3 || mode == 6) ? 2 : 1;
+    const bool mirror = mode != 1;
+    const int tpw = 16 * nq * waves / R;
     const int nblk = (T + tpw - 1) / tpw;
-    const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(kPfWaves * kWave);
+    const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(waves * kWave);
     note_scan_kernel("prefill_f16_mfma_kernel");
-#define TW_PF_LAUNCH(RR, NN, MM) launch_scan_kernel(prefill_f16_mfma_kernel<RR, NN, MM>, grid, block, s, a, T)
+#define TW_PF_LAUNCH(RR, NN, MM, WW) launch_scan_kernel(prefill_f16_mfma_kernel<RR, NN, MM, WW>, grid, block, s, a, T)
 #define TW_PF_MODES(RR) \
-    do { if (mode == 1) TW_PF_LAUNCH(RR, 1, false); else if (mode == 2) TW_PF_LAUNCH(RR, 1, true); \
-         else TW_PF_LAUNCH(RR, 2, true); } while (0)
+    do { if (mode == 1) TW_PF_LAUNCH(RR, 1, false, 4); else if (mode == 2) TW_PF_LAUNCH(RR, 1, true, 4); \
+         else if (mode == 3) TW_PF_LAUNCH(RR, 2, true, 4); else if (mode == 5) TW_PF_LAUNCH(RR, 1, true, 8); \
+         else TW_PF_LAUNCH(RR, 2, true, 8); } while (0)
     if (R == 1) TW_PF_MODES(1); else if (R == 2) TW_PF_MODES(2); else TW_PF_MODES(4);
 #undef TW_PF_MODES
 #undef TW_PF_LAUNCH

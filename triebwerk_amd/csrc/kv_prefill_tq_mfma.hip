@@ -23,7 +23,6 @@ namespace twkv {
 
 namespace {
 
-constexpr int kPtWaves = 4;
 constexpr int kPtKRow = 2 * kHeadDim + 32;   // bytes per expanded K row in LDS (288: operand reads at the LDS's full rate, 272: 53 % of it)
 constexpr int kPtVRow = 2 * 32 + 32;         // bytes per V^T row (32 token slots) in LDS (96: full rate, 80: 54 %)
 constexpr int kPtVTile = kHeadDim * kPtVRow; // bytes of a V^T tile
@@ -37,10 +36,12 @@ __device__ __forceinline__ int vt_slot(int token) { return 8 * ((token & 15) >> 
 
 // NQ: 16-row query blocks per wave (every K and V operand read feeds NQ MFMAs).  MIRROR: a workgroup does a
 // token block and then its mirror image from the other end of the sequence.
-template <int R, int BITS, int NQ, bool MIRROR>
-__global__ void __launch_bounds__(kPtWaves* kWave, 2)        // two workgroups per CU: at most 256 registers per lane
+// W: waves per workgroup, 4 (two workgroups per CU) or 8 (one: a tile is expanded once for twice the queries).
+template <int R, int BITS, int NQ, bool MIRROR, int W>
+__global__ void __launch_bounds__(W* kWave, W == 4 ? 2 : 1)  // two waves per SIMD either way: at most 256 registers per lane
 prefill_tq_mfma_kernel(AttnArgs a, int T) {
-    constexpr int TPW = 16 * NQ * kPtWaves / R;            // query tokens per workgroup pass
+    static_assert(W == 4 || W == 8, "the staging maps are written for 256 and 512 threads");
+    constexpr int TPW = 16 * NQ * W / R;                   // query tokens per workgroup pass
     constexpr float kAlpha = BITS == 4 ? kAlpha4 : kAlpha2;
     constexpr float kQScale = kLog2e * kInvSqrtD / kAlpha;   // score scale of kernels.cu:1707 in base 2, table scale undone
     constexpr int kHeadBytes = BITS * 16;                  // bytes of one head in a cache row
@@ -76,7 +77,7 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
     constexpr float kRaise = 5.0f;
 
     // ---- table: byte -> its codes' centroids (low field first) as fp16(alpha c), kPtReplicas copies
-    for (int i = tid; i < 256 * kPtReplicas; i += kPtWaves * kWave) {
+    for (int i = tid; i < 256 * kPtReplicas; i += W * kWave) {
         const int e = i / kPtReplicas;
         if constexpr (BITS == 4) {
             half2_t p = {(half_t)(kAlpha * kCentroids4[e & 15]), (half_t)(kAlpha * kCentroids4[e >> 4])};
@@ -103,10 +104,22 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         }
     };
 
+    // the 4 halves (2 dwords) of 4 consecutive coordinates (2 bytes of codes at 4 bit, 1 at 2 bit)
+    auto expand4 = [&](uint32_t codes, uint32_t (&out)[4]) {
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int b = 0; b < 2; b++) out[b] = tab_s[((codes >> (8 * b)) & 255u) * kPtReplicas + rep];
+        } else {
+            const uint2 v = *reinterpret_cast<const uint2*>(&tab_s[2 * ((codes & 255u) * kPtReplicas + rep)]);
+            out[0] = v.x; out[1] = v.y;
+        }
+        out[2] = 0u; out[3] = 0u;
+    };
+
     // ---- staging of a tile: thread (r = tid / 16, c = tid % 16) carries the codes of coordinates 8c..8c+7 of
-    // K rows r and r + 16; for V, thread (c = tid / 16, r = tid % 16) carries those of rows 2r and 2r + 1 (two
-    // consecutive tokens, interleaved on the way into the transposed tile); threads 0..63 also carry a norm.
-    // Rows past the last token are clamped (masked anyway).
+    // K rows r and r + 16 (512 threads: of row r alone); for V, thread (c = tid / 16, r = tid % 16) carries those of
+    // coordinates 8c..8c+7 (512 threads: 4c..4c+3) of rows 2r and 2r + 1 (two consecutive tokens, interleaved on the
+    // way into the transposed tile); threads 0..63 also carry a norm.
     const int sr = tid >> 4, sc = tid & 15;
     // V: 16 consecutive threads take the 16 token pairs of one dim octet, so that their dwords fill one V^T row
     // (64 contiguous bytes, all banks different); with the K mapping they would hit rows 8 apart, 8 to a bank
@@ -121,19 +134,28 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
     const __amdgpu_buffer_rsrc_t knrs = make_rsrc(reinterpret_cast<const char*>(a.k_norms) + kvh * 2, T * nrow_bytes - kvh * 2);
     const __amdgpu_buffer_rsrc_t vnrs = make_rsrc(reinterpret_cast<const char*>(a.v_norms) + kvh * 2, T * nrow_bytes - kvh * 2);
     const int koff0 = sr * row_bytes + kPiece * sc, koff1 = koff0 + 16 * row_bytes;
-    const int voff0 = 2 * vr_ * row_bytes + kPiece * vc_, voff1 = voff0 + row_bytes;
+    const int voff0 = 2 * vr_ * row_bytes + (W == 4 ? kPiece : kPiece / 2) * vc_, voff1 = voff0 + row_bytes;
     const int noff = (tid & 31) * nrow_bytes;
     const __amdgpu_buffer_rsrc_t nrs = (wave & 1) ? vnrs : knrs;     // wave-uniform: a scalar choice
     auto load_codes = [&](__amdgpu_buffer_rsrc_t rs, int voff, int soff) -> uint32_t {
         if constexpr (BITS == 4) return __builtin_amdgcn_raw_buffer_load_b32(rs, voff, soff, 0);
         else return __builtin_amdgcn_raw_buffer_load_b16(rs, voff, soff, 0);
     };
+    auto load_half_codes = [&](__amdgpu_buffer_rsrc_t rs, int voff, int soff) -> uint32_t {     // 4 coordinates
+        if constexpr (BITS == 4) return __builtin_amdgcn_raw_buffer_load_b16(rs, voff, soff, 0);
+        else return __builtin_amdgcn_raw_buffer_load_b8(rs, voff, soff, 0);
+    };
     auto load_tile = [&](int tile, Staged& st) {
         const int toff = tile * row_bytes;
         st.k[0] = load_codes(krs, koff0, toff);
-        st.k[1] = load_codes(krs, koff1, toff);
-        st.v[0] = load_codes(vrs, voff0, toff);
-        st.v[1] = load_codes(vrs, voff1, toff);
+        if constexpr (W == 4) {
+            st.k[1] = load_codes(krs, koff1, toff);
+            st.v[0] = load_codes(vrs, voff0, toff);
+            st.v[1] = load_codes(vrs, voff1, toff);
+        } else {
+            st.v[0] = load_half_codes(vrs, voff0, toff);
+            st.v[1] = load_half_codes(vrs, voff1, toff);
+        }
         // Every thread asks for a norm of row tid % 32 -- even waves K's, odd waves V's; lanes 0..31 of waves 0 and 1
         // are the ones that keep it -- and holds the bits as they come: a load under a per-lane condition with a
         // descriptor that depends on the lane becomes a loop over the descriptors, and a value computed from a load
@@ -145,14 +167,21 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
         uint32_t e[4];
         expand8(st.k[0], e);
         *reinterpret_cast<uint4*>(&k_s[buf][sr * kPtKRow + 16 * sc]) = uint4{e[0], e[1], e[2], e[3]};
-        expand8(st.k[1], e);
-        *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPtKRow + 16 * sc]) = uint4{e[0], e[1], e[2], e[3]};
+        if constexpr (W == 4) {
+            expand8(st.k[1], e);
+            *reinterpret_cast<uint4*>(&k_s[buf][(sr + 16) * kPtKRow + 16 * sc]) = uint4{e[0], e[1], e[2], e[3]};
+        }
         uint32_t va[4], vb[4];
-        expand8(st.v[0], va);
-        expand8(st.v[1], vb);
-        char* dst = &v_s[vbuf * kPtVTile + (8 * vc_) * kPtVRow + vcol];
+        if constexpr (W == 4) {
+            expand8(st.v[0], va);
+            expand8(st.v[1], vb);
+        } else {
+            expand4(st.v[0], va);
+            expand4(st.v[1], vb);
+        }
+        char* dst = &v_s[vbuf * kPtVTile + ((W == 4 ? 8 : 4) * vc_) * kPtVRow + vcol];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {                      // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves)
+        for (int i = 0; i < (W == 4 ? 4 : 2); i++) {       // dims 8c + 2i (low halves) and 8c + 2i + 1 (high halves); 512 threads: 4c + ...
             *reinterpret_cast<uint32_t*>(dst + (2 * i) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x05040100u);
             *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kPtVRow) = __builtin_amdgcn_perm(vb[i], va[i], 0x07060302u);
         }
@@ -344,15 +373,16 @@ prefill_tq_mfma_kernel(AttnArgs a, int T) {
             // thread -> rows k = 16r + tid / 16, r = 0..7, columns 8c .. 8c + 7 with c = tid % 16; of k only r is
             // not fixed per thread, and r moves the destination by whole steps t = r / 2 and halves 4 (r % 2)
             const uint4* rsrc = reinterpret_cast<const uint4*>(a.rotation) + tid;
-            const int krow = tid >> 4, c = tid & 15;
-            char* dst0 = &v_s[(c >> 1) * 4096 + ((krow >> 2) & 3) * 256 + (c & 1) * 128 + 2 * (krow & 3)];
+            const int krow = tid >> 4, c = tid & 15;       // 512 threads: rows k = 32r + tid / 16, r = 0..3
+            char* dst0 = &v_s[(c >> 1) * 4096 + ((krow >> 2) & 3) * 256 + (c & 1) * 128 + 2 * (krow & 3) + (W == 8 ? 8 * (krow >> 4) : 0)];
 #pragma unroll
-            for (int r = 0; r < 8; r++) {
-                const uint4 rp = rsrc[r * (kPtWaves * kWave)];
+            for (int r = 0; r < 32 / W; r++) {
+                const uint4 rp = rsrc[r * (W * kWave)];
                 const uint32_t w[4] = {rp.x, rp.y, rp.z, rp.w};
+                const int step = W == 4 ? (r >> 1) * 1024 + (r & 1) * 8 : r * 1024;
 #pragma unroll
                 for (int x = 0; x < 8; x++)
-                    *reinterpret_cast<uint16_t*>(dst0 + (r >> 1) * 1024 + (r & 1) * 8 + x * 16) = (uint16_t)(w[x >> 1] >> (16 * (x & 1)));
+                    *reinterpret_cast<uint16_t*>(dst0 + step + x * 16) = (uint16_t)(w[x >> 1] >> (16 * (x & 1)));
             }
         }
         __syncthreads();
@@ -418,25 +448,27 @@ bool prefill_tq_mfma_usable(const AttnArgs& a) {
 void launch_prefill_tq_mfma(const AttnArgs& a, hipStream_t s, int form) {
     const int R = a.num_heads / a.num_kv_heads;
     const int T = a.G;
-    // forms as for the fp16 prefill kernel: long prompts take two query blocks per wave and mirrored block pairs
+    // forms as for the fp16 prefill kernel: long prompts take eight waves per workgroup, two query blocks per wave and
+    // mirrored block pairs; shorter ones one query block per wave, then four waves, then unpaired workgroups
     const int cus = compute_units();
+    auto pairs = [&](int waves, int nq) { const int tpw = 16 * nq * waves / R; return ((T + tpw - 1) / tpw + 1) / 2 * a.num_kv_heads; };
     int mode = 1;
-    {
-        const int nblk2 = (T + 32 * kPtWaves / R - 1) / (32 * kPtWaves / R), nblk1 = (T + 16 * kPtWaves / R - 1) / (16 * kPtWaves / R);
-        if ((nblk2 + 1) / 2 * a.num_kv_heads >= cus) mode = 3;
-        else if ((nblk1 + 1) / 2 * a.num_kv_heads >= cus) mode = 2;
-    }
-    if (form >= 1 && form <= 3) mode = form;               // forced by a test
-    const int nq = mode >= 3 ? 2 : 1;
-    const bool mirror = mode == 2 || mode == 3;
-    const int tpw = 16 * nq * kPtWaves / R;
+    if (4 * pairs(8, 2) >= 3 * cus) mode = 6;
+    else if (4 * pairs(8, 1) >= 3 * cus) mode = 5;
+    else if (pairs(4, 1) >= cus) mode = 2;
+    if ((form >= 1 && form <= 3) || form == 5 || form == 6) mode = form;    // forced by a test
+    const int waves = mode >= 5 ? 8 : 4;
+    const int nq = (mode == 3 || mode == 6) ? 2 : 1;
+    const bool mirror = mode != 1;
+    const int tpw = 16 * nq * waves / R;
     const int nblk = (T + tpw - 1) / tpw;
-    const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(kPtWaves * kWave);
+    const dim3 grid(mirror ? (nblk + 1) / 2 : nblk, a.num_kv_heads), block(waves * kWave);
     note_scan_kernel("prefill_tq_mfma_kernel");
-#define TW_PT_LAUNCH(RR, BB, NN, MM) launch_scan_kernel(prefill_tq_mfma_kernel<RR, BB, NN, MM>, grid, block, s, a, T)
+#define TW_PT_LAUNCH(RR, BB, NN, MM, WW) launch_scan_kernel(prefill_tq_mfma_kernel<RR, BB, NN, MM, WW>, grid, block, s, a, T)
 #define TW_PT_MODES(RR, BB) \
-    do { if (mode == 1) TW_PT_LAUNCH(RR, BB, 1, false); else if (mode == 2) TW_PT_LAUNCH(RR, BB, 1, true); \
-         else TW_PT_LAUNCH(RR, BB, 2, true); } while (0)
+    do { if (mode == 1) TW_PT_LAUNCH(RR, BB, 1, false, 4); else if (mode == 2) TW_PT_LAUNCH(RR, BB, 1, true, 4); \
+         else if (mode == 3) TW_PT_LAUNCH(RR, BB, 2, true, 4); else if (mode == 5) TW_PT_LAUNCH(RR, BB, 1, true, 8); \
+         else TW_PT_LAUNCH(RR, BB, 2, true, 8); } while (0)
 #define TW_PT_BITS(RR) do { if (a.bits == 4) TW_PT_MODES(RR, 4); else TW_PT_MODES(RR, 2); } while (0)
     if (R == 1) TW_PT_BITS(1); else if (R == 2) TW_PT_BITS(2); else TW_PT_BITS(4);
 #undef TW_PT_BITS
