@@ -167,7 +167,7 @@ def cpu_baseline(w, kv_bits, seconds_budget=15.0):
                        f"{os.cpu_count()} logical CPUs visible")
 
 
-def prefill_bench(args):
+def prefill_bench(args, quiet=False):
     """Causal prefill attention of one sequence, one layer: ms per launch and the matrix-core rate.
     FLOPs counted: 4 * head_dim per (query head, query token, attended token), causal half only."""
     import torch
@@ -238,7 +238,7 @@ def prefill_bench(args):
     ms = e0.elapsed_time(e1) / args.steps
     flop = 4.0 * D * H * T * (T + 1) / 2
     tflops = flop / (ms * 1e-3) * 1e-12
-    print(json.dumps({
+    result = {
         "metric": "prefill-attn prompt tokens/s (one layer)", "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": max(args.warmup, 1), "ms_per_step": ms, "higher_is_better": True,
         "dtype": "f16-operand MFMA, f32 accumulate" if not kv_bits else DTYPE[kv_bits], "data": "synthetic",
@@ -248,7 +248,12 @@ def prefill_bench(args):
                              "launch_qk_norm_batch, launch_rope_batch, 2 appends, the attention launch (+ 2 copies restoring q and k)"][args.prompt_step]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s", "frac": tflops / 2500.0,
                      "flops_per_launch": flop, "traffic": None},
-    }))
+    }
+    kvcache.set_prefill_form(0)
+    if quiet:
+        return result
+    print(json.dumps(result))
+    return result
 
 
 def paged_bench(args):
@@ -526,6 +531,16 @@ def per_config(args):
                     "launches_per_layer": r["config"]["launches_per_layer"],
                     "kernel_name": r["roofline"]["kernel_name"], "launch_ms": r["roofline"]["launch_ms"],
                     "launch_algorithmic_MB": r["roofline"]["launch_algorithmic_MB"], "launch_frac_of_hbm_peak": r["roofline"]["frac"]}
+    # the prompt side of the cache (not a BASELINE config; bound by the matrix cores, not by HBM): causal attention over
+    # an 8192-token prompt, one layer, the target workload's head counts, a sustained burst of launches
+    for key, bits in (("prefill_8192_fp16", 0), ("prefill_8192_tq4", 4)):
+        a = copy.copy(args)
+        a.workload, a.kv_bits, a.prefill, a.prompt_step, a.prefill_form = "target", bits, 8192, 0, 0
+        a.steps, a.warmup = 300, 100
+        r = prefill_bench(a, quiet=True)
+        out[key] = {"workload": r["config"]["workload"], "kv_bits": bits if bits else 16, "steps": r["steps"],
+                    "ms_per_launch": r["ms_per_step"], "prompt_tokens_per_s": r["value"], "bound": "mfma",
+                    "tflops": r["roofline"]["achieved"], "frac_of_dense_fp16_mfma_peak": r["roofline"]["frac"]}
     return out
 
 
