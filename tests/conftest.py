@@ -46,7 +46,7 @@ def rotation_fixture():
 
 def pytest_terminal_summary(terminalreporter, exitstatus, config):
     """How much of the attention tolerance the GPU parity tests used: one line (shown with -q too) and the table of
-    every test's largest relative error as JSON under gpurun_out/."""
+    every test's largest relative error as a JSON file in the run's output folder."""
     import json
     import parity_log
     if not parity_log.WORST:
