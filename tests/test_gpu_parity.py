@@ -744,6 +744,39 @@ def test_turbo_prefill_every_form(kv, oracle, rotation_fixture, bits, H, Hk, T, 
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("form", [3, 5, 6])
+@pytest.mark.parametrize("R,T", [(1, 255), (1, 256), (1, 257), (2, 127), (2, 128), (2, 129), (2, 383), (4, 63), (4, 64), (4, 65), (4, 193)])
+@pytest.mark.parametrize("bits", [0, 2])
+def test_prefill_lengths_around_the_token_blocks(kv, oracle, rotation_fixture, bits, R, T, form):
+    """Prompt lengths one below, at and one above a multiple of the workgroup's token block (64 to 256 tokens,
+    by GQA group and form): the last block is ragged or exactly full, the mirrored pair of a block may be the
+    block itself, and the steady part of the tile loop may be empty."""
+    import torch
+    Hk = 2
+    H = Hk * R
+    r = gen.rng(1300 + 17 * R + T + bits)
+    msl = T + 1
+    kv_dim, q_dim = Hk * D, H * D
+    q = gen.normal_f16(r, (T, q_dim))
+    want = np.zeros((T, q_dim), np.float16)
+    out = torch.zeros((T, q_dim), dtype=torch.float16, device="cuda")
+    scratch = torch.zeros(T * H * max(T, 1024), dtype=torch.float32, device="cuda")
+    kv.set_prefill_form(form)
+    try:
+        if bits:
+            ck, cv, kn, vn = build_turbo_cache(oracle, rotation_fixture, r, 1, Hk, msl, [T], bits)
+            oracle.turbo_gqa_prefill_attention(want, q, ck[0], cv[0], kn[0], vn[0], rotation_fixture, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+            kv.launch_turbo_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), dev(kn[0]), dev(vn[0]),
+                                                  dev(rotation_fixture), scratch, T, msl, H, Hk, D, q_dim, kv_dim, bits)
+        else:
+            ck, cv = build_fp16_cache(r, 1, msl, kv_dim)
+            oracle.gqa_prefill_attention(want, q, ck[0], cv[0], T, msl, H, Hk, D, q_dim, kv_dim)
+            kv.launch_gqa_prefill_attention(out, dev(q), dev(ck[0]), dev(cv[0]), scratch, T, msl, H, Hk, D, q_dim, kv_dim)
+    finally:
+        kv.set_prefill_form(0)
+    assert rel_err(host(out), want) <= TOL
+
+
 @pytest.mark.parametrize("form", [1, 3, 6])
 @pytest.mark.parametrize("Hk,R,T", [(1, 2, 290), (2, 1, 97), (2, 2, 418), (3, 1, 150), (4, 2, 163), (6, 2, 130), (16, 1, 200), (24, 1, 70)])
 @pytest.mark.parametrize("bits", [0, 4])
