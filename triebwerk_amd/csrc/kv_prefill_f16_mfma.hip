@@ -184,10 +184,14 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
         // the filling step t = -1 and those on the diagonal the general one.
         __syncthreads();                                   // a previous pass may still be reading its last V tile
         uint4 kr[2], vr[2];
-        load_tile(0, kr, vr);
-        stash(0, 0, kr, vr);
-        if (ntiles > 1) { load_tile(32, kr, vr); stash(1, 1, kr, vr); }
-        if (ntiles > 2) load_tile(64, kr, vr);
+        {
+            uint4 kr1[2], vr1[2];                          // tiles 0, 1 and 2 are asked for together: one trip to memory, not three
+            load_tile(0, kr, vr);
+            if (ntiles > 1) load_tile(32, kr1, vr1);
+            stash(0, 0, kr, vr);
+            if (ntiles > 2) load_tile(64, kr, vr);
+            if (ntiles > 1) stash(1, 1, kr1, vr1);
+        }
         __syncthreads();
         half8_t kf[8];
         read_k(0, kf);
