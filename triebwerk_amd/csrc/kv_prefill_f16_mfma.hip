@@ -206,7 +206,9 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
             const int tile1 = 32 * (t + 1);                // first token of tile t + 1
             const bool do_s = STEADY || (t + 1 < ntiles && tile1 <= q0 + 16 * NQ - 1 && q0 < T);   // tile t + 1 reaches this wave's queries
             const bool do_p = STEADY || have_x;
-            // ---- phase 1
+            // ---- phase 1 (the wave's priority falls through the step: of the two waves of a SIMD the one in its score
+            // MFMAs goes first, 4 % at 8192 and 16384 tokens, whichever of the orders 1-0-0, 2-1-0, 3-1-0, 3-0-0)
+            __builtin_amdgcn_s_setprio(2);
             half8_t vf[8];
             if (do_p) read_v(t & 3, vf);
             float4_t s[NQ][2];
@@ -246,6 +248,7 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                     __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
                 }
             }
+            __builtin_amdgcn_s_setprio(1);
             // ---- phase 2: O[query][dim 16j + ln] += P . V of tile t
             if (do_p) {
 #pragma unroll
@@ -297,6 +300,7 @@ prefill_f16_mfma_kernel(AttnArgs a, int T) {
                 }
             }
             have_x = do_s;
+            __builtin_amdgcn_s_setprio(0);
             __syncthreads();
         };
         step(Flag<false>{}, -1);
